@@ -1,0 +1,25 @@
+"""MI355X-native attention path with brotensor-style operator entry points.
+
+The compute lives in lib/libmi_attention.so (hand-written HIP for gfx950 behind the C ABI in
+include/mi_attention.h). This package is the Python mirror of the host interface, used by the
+tests and the benchmark; PyTorch only provides device memory and streams.
+"""
+from .ops import (  # noqa: F401
+    SdpaMask,
+    build_axial_rope_tables,
+    device_info,
+    flash_attention_forward,
+    flash_attention_windowed_forward,
+    gqa_attention_masked,
+    joint_attention,
+    linear_attention_relu_forward,
+    rope_apply,
+    rope_apply_perhead,
+    sdpa_forward,
+)
+
+__all__ = [
+    "SdpaMask", "build_axial_rope_tables", "device_info", "flash_attention_forward",
+    "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
+    "linear_attention_relu_forward", "rope_apply", "rope_apply_perhead", "sdpa_forward",
+]

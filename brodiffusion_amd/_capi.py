@@ -1,0 +1,123 @@
+"""ctypes binding of libmi_attention.so (the C ABI declared in include/mi_attention.h).
+
+Loading fails loudly when the library has not been built: there is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libmi_attention.so")
+
+MI_DTYPE_F16 = 1
+MI_DTYPE_BF16 = 2
+MI_MASK_NONE = 0
+MI_MASK_CAUSAL = 1
+MI_MASK_BLOCK_CAUSAL = 2
+MI_MAX_SEGMENTS = 32
+
+EXPORTS = [
+    "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
+    "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
+    "mi_sdpa_forward", "mi_sdpa_supported", "mi_rope_apply",
+    "mi_linear_attn_workspace_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
+]
+
+
+class MiDeviceInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
+                ("clock_khz", C.c_int32), ("lds_bytes_per_cu", C.c_int32), ("l2_bytes", C.c_int32),
+                ("hbm_bytes", C.c_int64), ("peak_mfma_16bit_flops", C.c_double)]
+
+
+class MiSdpaArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+        ("k_prefix", C.c_void_p), ("v_prefix", C.c_void_p),
+        ("batch", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32), ("num_kv_heads", C.c_int32),
+        ("q_len", C.c_int32), ("kv_len", C.c_int32), ("prefix_len", C.c_int32),
+        ("q_row_stride", C.c_int64), ("q_batch_stride", C.c_int64),
+        ("k_row_stride", C.c_int64), ("k_batch_stride", C.c_int64),
+        ("v_row_stride", C.c_int64), ("v_batch_stride", C.c_int64),
+        ("o_row_stride", C.c_int64), ("o_batch_stride", C.c_int64),
+        ("kp_row_stride", C.c_int64), ("kp_batch_stride", C.c_int64),
+        ("vp_row_stride", C.c_int64), ("vp_batch_stride", C.c_int64),
+        ("scale", C.c_float), ("mask_mode", C.c_int32), ("q_offset", C.c_int32), ("window", C.c_int32),
+        ("kv_valid_len", C.c_void_p), ("key_mask", C.c_void_p), ("key_mask_batch_stride", C.c_int64),
+        ("n_segments", C.c_int32),
+        ("seg_q_end", C.c_int32 * MI_MAX_SEGMENTS), ("seg_k_end", C.c_int32 * MI_MAX_SEGMENTS),
+        ("seg_causal", C.c_int32 * MI_MAX_SEGMENTS),
+        ("rope_cos_q", C.c_void_p), ("rope_sin_q", C.c_void_p), ("rope_cos_k", C.c_void_p), ("rope_sin_k", C.c_void_p),
+        ("stream", C.c_void_p),
+    ]
+
+
+class MiRopeArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("x", C.c_void_p), ("out", C.c_void_p), ("cos", C.c_void_p), ("sin", C.c_void_p),
+        ("rows", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32),
+        ("x_row_stride", C.c_int64), ("out_row_stride", C.c_int64),
+        ("split_half", C.c_int32), ("per_head", C.c_int32), ("stream", C.c_void_p),
+    ]
+
+
+class MiLinearAttnArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("o", C.c_void_p),
+        ("batch", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32), ("n_tokens", C.c_int32),
+        ("q_row_stride", C.c_int64), ("q_batch_stride", C.c_int64),
+        ("k_row_stride", C.c_int64), ("k_batch_stride", C.c_int64),
+        ("v_row_stride", C.c_int64), ("v_batch_stride", C.c_int64),
+        ("o_row_stride", C.c_int64), ("o_batch_stride", C.c_int64),
+        ("eps", C.c_float), ("accumulate_state", C.c_int32),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("stream", C.c_void_p),
+    ]
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """The loaded C-ABI library; raises if it has not been built (python -m brodiffusion_amd.build)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP extension first (python -m brodiffusion_amd.build). "
+                "There is no CPU fallback.")
+        L = C.CDLL(LIB_PATH)
+        L.mi_last_error.restype = C.c_char_p
+        L.mi_version.restype = C.c_char_p
+        L.mi_device_info.argtypes = [C.POINTER(MiDeviceInfo)]
+        L.mi_set_stream.argtypes = [C.c_void_p]
+        L.mi_get_stream.restype = C.c_void_p
+        L.mi_stream_synchronize.argtypes = [C.c_void_p]
+        L.mi_malloc.argtypes = [C.c_size_t]
+        L.mi_malloc.restype = C.c_void_p
+        L.mi_free.argtypes = [C.c_void_p]
+        L.mi_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.mi_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.mi_memcpy_d2d_async.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.mi_memset_async.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
+        L.mi_sdpa_forward.argtypes = [C.POINTER(MiSdpaArgs)]
+        L.mi_sdpa_supported.argtypes = [C.c_int32, C.c_int32]
+        L.mi_rope_apply.argtypes = [C.POINTER(MiRopeArgs)]
+        L.mi_linear_attn_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+        L.mi_linear_attn_workspace_bytes.restype = C.c_size_t
+        L.mi_linear_attn_relu_forward.argtypes = [C.POINTER(MiLinearAttnArgs)]
+        L.mi_linear_attn_supported.argtypes = [C.c_int32, C.c_int32]
+        _lib = L
+    return _lib
+
+
+def last_error() -> str:
+    return lib().mi_last_error().decode()
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what}: {last_error()}")

@@ -1,0 +1,173 @@
+// C ABI of libmi_attention.so: argument validation, error reporting, stream and memory
+// helpers. All HIP calls of the library live behind these entry points.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "internal.h"
+
+namespace mi {
+namespace {
+thread_local char g_err[512] = "";
+thread_local hipStream_t g_stream = nullptr;
+}  // namespace
+
+int fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+void clear_error() { g_err[0] = '\0'; }
+hipStream_t resolve_stream(void* s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
+
+namespace {
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+}  // namespace
+}  // namespace mi
+
+using mi::fail;
+
+extern "C" {
+
+const char* mi_last_error(void) { return mi::g_err; }
+const char* mi_version(void) { return "mi_attention 0.1 (gfx950)"; }
+
+int mi_device_info(mi_device_info_t* out) {
+    mi::clear_error();
+    if (!out) return fail("mi_device_info: null output");
+    int dev = 0;
+    MI_HIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t p;
+    MI_HIP_CHECK(hipGetDeviceProperties(&p, dev));
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", p.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", p.gcnArchName);
+    out->compute_units = p.multiProcessorCount;
+    out->clock_khz = p.clockRate;
+    out->lds_bytes_per_cu = static_cast<int32_t>(p.maxSharedMemoryPerMultiProcessor);
+    out->l2_bytes = p.l2CacheSize;
+    out->hbm_bytes = static_cast<int64_t>(p.totalGlobalMem);
+    out->peak_mfma_16bit_flops = static_cast<double>(p.multiProcessorCount) * p.clockRate * 1e3 * 4096.0;
+    return 0;
+}
+
+int mi_set_stream(void* stream) { mi::clear_error(); mi::g_stream = static_cast<hipStream_t>(stream); return 0; }
+void* mi_get_stream(void) { return mi::g_stream; }
+int mi_stream_synchronize(void* stream) {
+    mi::clear_error();
+    MI_HIP_CHECK(hipStreamSynchronize(mi::resolve_stream(stream)));
+    return 0;
+}
+
+void* mi_malloc(size_t bytes) {
+    mi::clear_error();
+    void* p = nullptr;
+    const hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) { fail("mi_malloc(%zu): %s", bytes, hipGetErrorString(e)); return nullptr; }
+    return p;
+}
+int mi_free(void* ptr) { mi::clear_error(); if (ptr) MI_HIP_CHECK(hipFree(ptr)); return 0; }
+int mi_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    mi::clear_error(); MI_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); return 0;
+}
+int mi_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    mi::clear_error(); MI_HIP_CHECK(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); return 0;
+}
+int mi_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) {
+    mi::clear_error();
+    MI_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, mi::resolve_stream(stream)));
+    return 0;
+}
+int mi_memset_async(void* dst, int value, size_t bytes, void* stream) {
+    mi::clear_error(); MI_HIP_CHECK(hipMemsetAsync(dst, value, bytes, mi::resolve_stream(stream))); return 0;
+}
+
+int mi_sdpa_supported(int32_t dtype, int32_t head_dim) { return mi::sdpa_supported(dtype, head_dim) ? 1 : 0; }
+
+int mi_sdpa_forward(const mi_sdpa_args* a) {
+    mi::clear_error();
+    if (!a) return fail("mi_sdpa_forward: null args");
+    if (a->struct_size != sizeof(mi_sdpa_args))
+        return fail("mi_sdpa_forward: struct_size %u != %zu (header mismatch)", a->struct_size, sizeof(mi_sdpa_args));
+    if (!mi::sdpa_supported(a->dtype, a->head_dim))
+        return fail("mi_sdpa_forward: no kernel for dtype %d head_dim %d", a->dtype, a->head_dim);
+    if (a->batch <= 0 || a->num_heads <= 0) return fail("mi_sdpa_forward: batch and num_heads must be positive");
+    if (a->q_len < 0 || a->kv_len < 0 || a->prefix_len < 0) return fail("mi_sdpa_forward: negative length");
+    if (a->q_len == 0) return 0;
+    if (!a->q || !a->o) return fail("mi_sdpa_forward: q and o must not be null");
+    if (a->kv_len > 0 && (!a->k || !a->v)) return fail("mi_sdpa_forward: k and v must not be null");
+    if (a->prefix_len > 0 && (!a->k_prefix || !a->v_prefix))
+        return fail("mi_sdpa_forward: prefix_len %d but k_prefix / v_prefix is null", a->prefix_len);
+    const int Hkv = a->num_kv_heads > 0 ? a->num_kv_heads : a->num_heads;
+    if (a->num_heads % Hkv != 0) return fail("mi_sdpa_forward: num_kv_heads %d does not divide num_heads %d", Hkv, a->num_heads);
+    const long D = static_cast<long>(a->num_heads) * a->head_dim;
+    const long Dkv = static_cast<long>(Hkv) * a->head_dim;
+    const long Lk = static_cast<long>(a->prefix_len) + a->kv_len;
+    if (Lk > 0x7fffff00L) return fail("mi_sdpa_forward: too many keys");
+
+    mi::SdpaDev p;
+    std::memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
+    p.kp = a->prefix_len > 0 ? a->k_prefix : nullptr;
+    p.vp = a->prefix_len > 0 ? a->v_prefix : nullptr;
+    p.B = a->batch; p.H = a->num_heads; p.Lq = a->q_len; p.Lk = static_cast<int>(Lk); p.Lp = a->prefix_len;
+    p.kv_group = a->num_heads / Hkv;
+    auto rs = [](int64_t s, long dense) { return s ? static_cast<long>(s) : dense; };
+    p.q_rs = rs(a->q_row_stride, D); p.k_rs = rs(a->k_row_stride, Dkv); p.v_rs = rs(a->v_row_stride, Dkv);
+    p.o_rs = rs(a->o_row_stride, D); p.kp_rs = rs(a->kp_row_stride, Dkv); p.vp_rs = rs(a->vp_row_stride, Dkv);
+    p.q_bs = a->q_batch_stride ? a->q_batch_stride : p.q_rs * a->q_len;
+    p.o_bs = a->o_batch_stride ? a->o_batch_stride : p.o_rs * a->q_len;
+    p.k_bs = a->k_batch_stride ? a->k_batch_stride : p.k_rs * a->kv_len;
+    p.v_bs = a->v_batch_stride ? a->v_batch_stride : p.v_rs * a->kv_len;
+    p.kp_bs = a->kp_batch_stride ? a->kp_batch_stride : p.kp_rs * a->prefix_len;
+    p.vp_bs = a->vp_batch_stride ? a->vp_batch_stride : p.vp_rs * a->prefix_len;
+    // 16-byte vector loads: bases 16-byte aligned, strides multiples of 8 elements, row at least one head wide
+    const void* ptrs[] = {a->q, a->k, a->v, a->o, p.kp, p.vp};
+    for (const void* ptr : ptrs)
+        if (ptr && !mi::aligned16(ptr)) return fail("mi_sdpa_forward: tensor pointers must be 16-byte aligned");
+    const long strides[] = {p.q_rs, p.k_rs, p.v_rs, p.o_rs, p.kp_rs, p.vp_rs, p.q_bs, p.k_bs, p.v_bs, p.o_bs, p.kp_bs, p.vp_bs};
+    for (long s : strides)
+        if (s % 8 != 0) return fail("mi_sdpa_forward: strides must be multiples of 8 elements (got %ld)", s);
+    if (p.q_rs < D || p.o_rs < D) return fail("mi_sdpa_forward: q/o row stride smaller than heads*head_dim %ld", D);
+    if (p.k_rs < Dkv || p.v_rs < Dkv || p.kp_rs < Dkv || p.vp_rs < Dkv)
+        return fail("mi_sdpa_forward: k/v row stride smaller than kv_heads*head_dim %ld", Dkv);
+
+    const float scale = a->scale > 0.f ? a->scale : 1.0f / std::sqrt(static_cast<float>(a->head_dim));
+    p.scale_log2 = scale * 1.4426950408889634f;
+    p.mask_mode = a->mask_mode; p.q_offset = a->q_offset; p.window = 0;
+    if (a->mask_mode == MI_MASK_CAUSAL) {
+        if (a->window < 0) return fail("mi_sdpa_forward: window must be >= 0");
+        p.window = a->window;
+    } else if (a->mask_mode == MI_MASK_BLOCK_CAUSAL) {
+        if (a->n_segments < 1 || a->n_segments > MI_MAX_SEGMENTS)
+            return fail("mi_sdpa_forward: n_segments %d outside 1..%d", a->n_segments, MI_MAX_SEGMENTS);
+        p.n_seg = a->n_segments;
+        for (int s = 0; s < a->n_segments; ++s) {
+            if (s > 0 && a->seg_q_end[s] < a->seg_q_end[s - 1])
+                return fail("mi_sdpa_forward: seg_q_end must be non-decreasing");
+            if (a->seg_k_end[s] < 0) return fail("mi_sdpa_forward: seg_k_end must be >= 0");
+            p.seg_q_end[s] = a->seg_q_end[s]; p.seg_k_end[s] = a->seg_k_end[s]; p.seg_causal[s] = a->seg_causal[s] ? 1 : 0;
+        }
+        if (a->seg_q_end[a->n_segments - 1] < a->q_len)
+            return fail("mi_sdpa_forward: segments cover %d query rows, q_len is %d", a->seg_q_end[a->n_segments - 1], a->q_len);
+    } else if (a->mask_mode != MI_MASK_NONE) {
+        return fail("mi_sdpa_forward: unknown mask_mode %d", a->mask_mode);
+    }
+    p.kv_valid_len = a->kv_valid_len;
+    p.key_mask = a->key_mask; p.key_mask_bs = a->key_mask_batch_stride;
+    if ((a->rope_cos_q == nullptr) != (a->rope_sin_q == nullptr) || (a->rope_cos_k == nullptr) != (a->rope_sin_k == nullptr))
+        return fail("mi_sdpa_forward: rope cos and sin tables must be given together");
+    const void* tabs[] = {a->rope_cos_q, a->rope_sin_q, a->rope_cos_k, a->rope_sin_k};
+    for (const void* t : tabs)
+        if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
+    p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
+    p.n_q_tiles = (a->q_len + 127) / 128;
+    const long nb = static_cast<long>(a->batch) * a->num_heads * p.n_q_tiles;
+    if (nb > 0x3fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
+    p.n_blocks = static_cast<int>(nb);
+    return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
+}
+
+}  // extern "C"

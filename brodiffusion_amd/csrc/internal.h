@@ -1,0 +1,51 @@
+// Internal declarations shared by the translation units of libmi_attention.so.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+
+#include "mi_attention.h"
+
+namespace mi {
+
+// Records the message mi_last_error() returns for this thread; always returns -1.
+int fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+hipStream_t resolve_stream(void* s);
+
+#define MI_HIP_CHECK(expr)                                                          \
+    do {                                                                            \
+        hipError_t _e = (expr);                                                     \
+        if (_e != hipSuccess) return ::mi::fail("%s: %s", #expr, hipGetErrorString(_e)); \
+    } while (0)
+
+// Device-side view of one softmax-attention launch. Strides in elements.
+struct SdpaDev {
+    const void* q; const void* k; const void* v; void* o;
+    const void* kp; const void* vp;
+    int B, H, Lq, Lk, Lp;  // Lk = Lp + fresh rows
+    int kv_group;          // query heads per K/V head
+    long q_rs, q_bs, k_rs, k_bs, v_rs, v_bs, o_rs, o_bs, kp_rs, kp_bs, vp_rs, vp_bs;
+    float scale_log2;      // scale * log2(e)
+    int mask_mode, q_offset, window;
+    const int* kv_valid_len;
+    const float* key_mask; long key_mask_bs;
+    int n_seg;
+    int seg_q_end[MI_MAX_SEGMENTS];
+    int seg_k_end[MI_MAX_SEGMENTS];
+    int seg_causal[MI_MAX_SEGMENTS];
+    const float* cos_q; const float* sin_q;
+    const float* cos_k; const float* sin_k;
+    int n_q_tiles; int n_blocks;  // logical work items = B*H*n_q_tiles
+};
+
+// One rotation, written with explicit fused multiply-adds so that every kernel that rotates
+// (stand-alone pass, Q load, K tile load) rounds identically: (a + ib)(c + is).
+__device__ __forceinline__ float rope_re(float a, float b, float c, float s) { return __builtin_fmaf(a, c, -(b * s)); }
+__device__ __forceinline__ float rope_im(float a, float b, float c, float s) { return __builtin_fmaf(a, s, b * c); }
+
+int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
+bool sdpa_supported(int dtype, int head_dim);
+
+}  // namespace mi

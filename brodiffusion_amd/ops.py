@@ -1,0 +1,335 @@
+"""Python mirror of the host-side operator interface for the attention path.
+
+Names, argument order and error behaviour follow the brotensor operators the reference calls
+(citations are paths in the reference repository):
+
+    flash_attention_forward(Q, K, V, d_mask, num_heads, causal, out)        src/dit/common.cpp:194
+    flash_attention_windowed_forward(Q, K, V, d_mask, num_heads, window, out) src/dit/qwenimage21_forward.cpp:662
+    rope_apply(X, cos, sin, head_dim, num_heads, out)                        src/dit/common.cpp:192
+    rope_apply_perhead(X, cos, sin, head_dim, num_heads, out)                src/triposplat/flow_model.cpp:374
+    joint_attention(Q, K, V, cos, sin, head_dim, num_heads, out, Qr, Kr)     include/brodiffusion/dit/common.h:80-88
+    gqa_attention_masked(...)                                                include/brodiffusion/dit/common.h:144-153
+    build_axial_rope_tables(txt_len, hp, wp, head_dim, axes, theta)          src/dit/common.cpp:116-184
+
+Tensors are torch CUDA tensors (rows = tokens, cols = heads*head_dim), used for device memory
+and the current stream only; every computation is a call through the C ABI. Shape and dtype
+precondition failures raise RuntimeError("<op>: <message>") as the reference's ops throw
+std::runtime_error; a CPU tensor is refused, never copied.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _capi as capi
+
+
+@dataclass
+class SdpaMask:
+    """Visibility rule of one attention call (see mi_sdpa_args in include/mi_attention.h)."""
+    mode: int = capi.MI_MASK_NONE
+    q_offset: int = 0
+    window: int = 0
+    seg_q_end: Sequence[int] = field(default_factory=list)
+    seg_k_end: Sequence[int] = field(default_factory=list)
+    seg_causal: Sequence[int] = field(default_factory=list)
+
+    @staticmethod
+    def causal(q_offset: int, window: int = 0) -> "SdpaMask":
+        return SdpaMask(capi.MI_MASK_CAUSAL, q_offset, window)
+
+    @staticmethod
+    def block_causal(q_offset: int, seg_q_end, seg_k_end, seg_causal) -> "SdpaMask":
+        return SdpaMask(capi.MI_MASK_BLOCK_CAUSAL, q_offset, 0, list(seg_q_end), list(seg_k_end), list(seg_causal))
+
+
+def _fail(op: str, msg: str):
+    raise RuntimeError(f"{op}: {msg}")
+
+
+def _dtype_code(op: str, t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return capi.MI_DTYPE_BF16
+    if t.dtype == torch.float16:
+        return capi.MI_DTYPE_F16
+    _fail(op, f"dtype {t.dtype} not supported (float16 / bfloat16)")
+
+
+def _dev(op: str, *ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            _fail(op, "tensor is not on the GPU (CPU tensors are refused, not copied)")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _as3(op: str, t: torch.Tensor, name: str):
+    """(rows, cols) or (batch, rows, cols) -> (batch, rows, cols, row_stride, batch_stride)."""
+    if t.dim() == 2:
+        if t.stride(1) != 1:
+            _fail(op, f"{name} must be contiguous along columns")
+        return 1, t.shape[0], t.shape[1], t.stride(0), t.stride(0) * t.shape[0]
+    if t.dim() == 3:
+        if t.stride(2) != 1:
+            _fail(op, f"{name} must be contiguous along columns")
+        return t.shape[0], t.shape[1], t.shape[2], t.stride(1), t.stride(0)
+    _fail(op, f"{name} must be (rows, cols) or (batch, rows, cols)")
+
+
+def device_info() -> dict:
+    info = capi.MiDeviceInfo()
+    capi.check(capi.lib().mi_device_info(C.byref(info)), "mi_device_info")
+    return {"name": info.name.decode(), "arch": info.arch.decode(), "compute_units": info.compute_units,
+            "clock_khz": info.clock_khz, "lds_bytes_per_cu": info.lds_bytes_per_cu, "l2_bytes": info.l2_bytes,
+            "hbm_bytes": info.hbm_bytes, "peak_mfma_16bit_flops": info.peak_mfma_16bit_flops}
+
+
+def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int, *, out: Optional[torch.Tensor] = None,
+                 num_kv_heads: int = 0, k_prefix: Optional[torch.Tensor] = None, v_prefix: Optional[torch.Tensor] = None,
+                 scale: Optional[float] = None, mask: Optional[SdpaMask] = None,
+                 kv_valid_len: Optional[torch.Tensor] = None, key_mask: Optional[torch.Tensor] = None,
+                 rope_q: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, op: str = "sdpa_forward") -> torch.Tensor:
+    """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None)."""
+    _dev(op, q, k, v, out, k_prefix, v_prefix, kv_valid_len, key_mask)
+    dt = _dtype_code(op, q)
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        _fail(op, "Q, K, V must share one dtype")
+    B, Lq, Dq, q_rs, q_bs = _as3(op, q, "Q")
+    Bk, Lk, Dk, k_rs, k_bs = _as3(op, k, "K")
+    Bv, Lv, Dv, v_rs, v_bs = _as3(op, v, "V")
+    if num_heads <= 0 or Dq % num_heads != 0:
+        _fail(op, "D must equal head_dim * num_heads")
+    hd = Dq // num_heads
+    hkv = num_kv_heads if num_kv_heads > 0 else num_heads
+    if num_heads % hkv != 0:
+        _fail(op, "num_kv_heads must divide num_heads")
+    if (Bk, Dk) != (B, hkv * hd) or (Bv, Lv, Dv) != (B, Lk, hkv * hd):
+        _fail(op, "K and V must be (Lk, kv_heads*head_dim) with Q's batch")
+    if out is None:
+        out = torch.empty_like(q)
+    if out.shape != q.shape or out.dtype != q.dtype:
+        _fail(op, "out must have Q's shape and dtype")
+    _, _, _, o_rs, o_bs = _as3(op, out, "out")
+    a = capi.MiSdpaArgs()
+    a.struct_size = C.sizeof(capi.MiSdpaArgs)
+    a.dtype = dt
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.batch, a.num_heads, a.head_dim, a.num_kv_heads = B, num_heads, hd, hkv
+    a.q_len, a.kv_len = Lq, Lk
+    a.q_row_stride, a.q_batch_stride = q_rs, q_bs
+    a.k_row_stride, a.k_batch_stride = k_rs, k_bs
+    a.v_row_stride, a.v_batch_stride = v_rs, v_bs
+    a.o_row_stride, a.o_batch_stride = o_rs, o_bs
+    Lp = 0
+    if (k_prefix is None) != (v_prefix is None):
+        _fail(op, "k_prefix and v_prefix must be given together")
+    if k_prefix is not None:
+        if k_prefix.dtype != q.dtype or v_prefix.dtype != q.dtype:
+            _fail(op, "prefix K/V must have Q's dtype")
+        Bp, Lp, Dp, kp_rs, kp_bs = _as3(op, k_prefix, "k_prefix")
+        Bp2, Lp2, Dp2, vp_rs, vp_bs = _as3(op, v_prefix, "v_prefix")
+        if (Bp, Dp) != (B, hkv * hd) or (Bp2, Lp2, Dp2) != (B, Lp, hkv * hd):
+            _fail(op, "prefix K/V must be (prefix_len, kv_heads*head_dim) with Q's batch")
+        a.k_prefix, a.v_prefix, a.prefix_len = k_prefix.data_ptr(), v_prefix.data_ptr(), Lp
+        a.kp_row_stride, a.kp_batch_stride, a.vp_row_stride, a.vp_batch_stride = kp_rs, kp_bs, vp_rs, vp_bs
+    a.scale = float(scale) if scale is not None else 0.0
+    if mask is not None:
+        a.mask_mode, a.q_offset, a.window = mask.mode, mask.q_offset, mask.window
+        if mask.mode == capi.MI_MASK_BLOCK_CAUSAL:
+            n = len(mask.seg_q_end)
+            if n < 1 or n > capi.MI_MAX_SEGMENTS or len(mask.seg_k_end) != n or len(mask.seg_causal) != n:
+                _fail(op, f"block-causal mask needs 1..{capi.MI_MAX_SEGMENTS} segments")
+            a.n_segments = n
+            for i in range(n):
+                a.seg_q_end[i], a.seg_k_end[i], a.seg_causal[i] = int(mask.seg_q_end[i]), int(mask.seg_k_end[i]), int(mask.seg_causal[i])
+    if kv_valid_len is not None:
+        if kv_valid_len.dtype != torch.int32 or kv_valid_len.numel() != B or not kv_valid_len.is_contiguous():
+            _fail(op, "kv_valid_len must be a contiguous int32 tensor of length batch")
+        a.kv_valid_len = kv_valid_len.data_ptr()
+    if key_mask is not None:
+        if key_mask.dtype != torch.float32 or not key_mask.is_contiguous():
+            _fail(op, "d_mask must be a contiguous float32 tensor")
+        if key_mask.numel() == Lp + Lk:
+            a.key_mask_batch_stride = 0
+        elif key_mask.numel() == B * (Lp + Lk):
+            a.key_mask_batch_stride = Lp + Lk
+        else:
+            _fail(op, "d_mask must hold Lk (or batch*Lk) values")
+        a.key_mask = key_mask.data_ptr()
+    for nm, tab, rows in (("rope_q", rope_q, Lq), ("rope_k", rope_k, Lk)):
+        if tab is None:
+            continue
+        cs, sn = tab
+        _dev(op, cs, sn)
+        for t in (cs, sn):
+            if t.dtype != torch.float32 or tuple(t.shape) != (rows, hd // 2) or not t.is_contiguous():
+                _fail(op, f"{nm} tables must be contiguous float32 ({rows}, head_dim/2)")
+        if nm == "rope_q":
+            a.rope_cos_q, a.rope_sin_q = cs.data_ptr(), sn.data_ptr()
+        else:
+            a.rope_cos_k, a.rope_sin_k = cs.data_ptr(), sn.data_ptr()
+    a.stream = _stream()
+    capi.check(capi.lib().mi_sdpa_forward(C.byref(a)), op)
+    return out
+
+
+def flash_attention_forward(Q, K, V, d_mask, num_heads: int, causal: bool, out: Optional[torch.Tensor] = None):
+    """out = softmax(Q K^T / sqrt(d) [+ key mask]) V per head. causal aligns the last query with the
+    last key (q_offset = Lk - Lq), as the windowed form does."""
+    op = "flash_attention_forward"
+    Lq, Lk = Q.shape[-2], K.shape[-2]
+    mask = SdpaMask.causal(Lk - Lq) if causal else None
+    return sdpa_forward(Q, K, V, num_heads, out=out, key_mask=d_mask, mask=mask, op=op)
+
+
+def flash_attention_windowed_forward(Q, K, V, d_mask, num_heads: int, window: int, out: Optional[torch.Tensor] = None):
+    """Causal attention with q_offset = Lk - Lq: query row r sees keys [0, q_offset + r]; window > 0
+    keeps the last `window` of them, window = 0 is unbounded (src/dit/qwenimage21_forward.cpp:8-13)."""
+    op = "flash_attention_windowed_forward"
+    if window < 0:
+        _fail(op, "window must be >= 0")
+    Lq, Lk = Q.shape[-2], K.shape[-2]
+    return sdpa_forward(Q, K, V, num_heads, out=out, key_mask=d_mask, mask=SdpaMask.causal(Lk - Lq, window), op=op)
+
+
+def _rope(op: str, X, cos, sin, head_dim, num_heads, out, per_head: bool, split_half: bool):
+    _dev(op, X, cos, sin, out)
+    dt = _dtype_code(op, X)
+    if X.dim() != 2 or X.stride(1) != 1:
+        _fail(op, "X must be (L, heads*head_dim), contiguous along columns")
+    L, D = X.shape
+    if head_dim <= 0 or num_heads <= 0 or D != head_dim * num_heads:
+        _fail(op, "D must equal head_dim * num_heads")
+    trows = L * num_heads if per_head else L
+    for t in (cos, sin):
+        if t.dtype != torch.float32 or tuple(t.shape) != (trows, head_dim // 2) or not t.is_contiguous():
+            _fail(op, f"cos/sin must be contiguous float32 ({trows}, head_dim/2)")
+    if out is None:
+        out = torch.empty_like(X)
+    if out.shape != X.shape or out.dtype != X.dtype or out.stride(1) != 1:
+        _fail(op, "out must have X's shape and dtype")
+    a = capi.MiRopeArgs()
+    a.struct_size = C.sizeof(capi.MiRopeArgs)
+    a.dtype = dt
+    a.x, a.out, a.cos, a.sin = X.data_ptr(), out.data_ptr(), cos.data_ptr(), sin.data_ptr()
+    a.rows, a.num_heads, a.head_dim = L, num_heads, head_dim
+    a.x_row_stride, a.out_row_stride = X.stride(0), out.stride(0)
+    a.split_half, a.per_head = int(split_half), int(per_head)
+    a.stream = _stream()
+    capi.check(capi.lib().mi_rope_apply(C.byref(a)), op)
+    return out
+
+
+def rope_apply(X, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None, split_half: bool = False):
+    return _rope("rope_apply", X, cos, sin, head_dim, num_heads, out, False, split_half)
+
+
+def rope_apply_perhead(X, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
+                       split_half: bool = False):
+    return _rope("rope_apply_perhead", X, cos, sin, head_dim, num_heads, out, True, split_half)
+
+
+def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
+                    Qr: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
+    """Full-bidirectional joint attention with RoPE on Q and K (include/brodiffusion/dit/common.h:74-88).
+    The rotation happens while Q and K are loaded; the Qr / Kr scratch tensors of the reference
+    signature are accepted and left untouched."""
+    op = "joint_attention"
+    if Q.dim() != 2 or Q.shape[1] != head_dim * num_heads:
+        _fail(op, "D must equal head_dim * num_heads")
+    if K.shape != Q.shape or V.shape != Q.shape:
+        _fail(op, "Q/K/V must share shape (L, D)")
+    return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), op=op)
+
+
+def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num_kv_heads: int, d_mask,
+                         out: Optional[torch.Tensor] = None):
+    """Bidirectional grouped-query attention with optional RoPE and key-padding mask
+    (include/brodiffusion/dit/common.h:131-153). K/V heads are indexed in place, not widened."""
+    op = "gqa_attention_masked"
+    if num_kv_heads <= 0 or num_q_heads % num_kv_heads != 0:
+        _fail(op, "num_kv_heads must divide num_q_heads")
+    if (cos is None) != (sin is None):
+        _fail(op, "cos and sin must be given together")
+    rope = (cos, sin) if cos is not None else None
+    return sdpa_forward(Q, K, V, num_q_heads, num_kv_heads=num_kv_heads, out=out, key_mask=d_mask,
+                        rope_q=rope, rope_k=rope, op=op)
+
+
+def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
+                                  workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False):
+    """Sana's ReLU linear attention core (src/dit/sana.cpp:470-586) on token-major (N, heads*head_dim)
+    or (batch, N, heads*head_dim) operands. `workspace` (float32, batch*heads*(d*d+d)) receives the
+    (S, z) state; pass it to capture the state or, with accumulate_state, to inject one."""
+    op = "linear_attention_relu_forward"
+    _dev(op, Q, K, V, out, workspace)
+    dt = _dtype_code(op, Q)
+    if K.dtype != Q.dtype or V.dtype != Q.dtype:
+        _fail(op, "Q, K, V must share one dtype")
+    if K.shape != Q.shape or V.shape != Q.shape:
+        _fail(op, "Q/K/V must share one shape")
+    B, N, D, q_rs, q_bs = _as3(op, Q, "Q")
+    _, _, _, k_rs, k_bs = _as3(op, K, "K")
+    _, _, _, v_rs, v_bs = _as3(op, V, "V")
+    if num_heads <= 0 or D % num_heads != 0:
+        _fail(op, "D must equal head_dim * num_heads")
+    hd = D // num_heads
+    if out is None:
+        out = torch.empty_like(Q)
+    if out.shape != Q.shape or out.dtype != Q.dtype:
+        _fail(op, "out must have Q's shape and dtype")
+    _, _, _, o_rs, o_bs = _as3(op, out, "out")
+    need = capi.lib().mi_linear_attn_workspace_bytes(B, num_heads, hd)
+    if workspace is None:
+        if accumulate_state:
+            _fail(op, "accumulate_state needs a caller workspace holding a state")
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=Q.device)
+    if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() * 4 < need:
+        _fail(op, f"workspace must be contiguous float32 with at least {need // 4} elements")
+    a = capi.MiLinearAttnArgs()
+    a.struct_size = C.sizeof(capi.MiLinearAttnArgs)
+    a.dtype = dt
+    a.q, a.k, a.v, a.o = Q.data_ptr(), K.data_ptr(), V.data_ptr(), out.data_ptr()
+    a.batch, a.num_heads, a.head_dim, a.n_tokens = B, num_heads, hd, N
+    a.q_row_stride, a.q_batch_stride, a.k_row_stride, a.k_batch_stride = q_rs, q_bs, k_rs, k_bs
+    a.v_row_stride, a.v_batch_stride, a.o_row_stride, a.o_batch_stride = v_rs, v_bs, o_rs, o_bs
+    a.eps = eps
+    a.accumulate_state = int(accumulate_state)
+    a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * 4
+    a.stream = _stream()
+    capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
+    return out
+
+
+def build_axial_rope_tables(txt_len: int, hp: int, wp: int, head_dim: int, axes_dims_rope: Sequence[int],
+                            theta: float = 10000.0, device="cuda"):
+    """cos / sin tables (txt_len + hp*wp, head_dim/2) FP32 for the joint [text ; image] sequence
+    (src/dit/common.cpp:116-184): text rows are the identity rotation, image token (i, j) has axial
+    position (0, i, j), pair p of axis a turns by pos * theta^(-2p / axes[a])."""
+    op = "build_axial_rope_tables"
+    if head_dim % 2 != 0:
+        _fail(op, "head_dim must be even")
+    if sum(axes_dims_rope) != head_dim:
+        _fail(op, "axes_dims_rope must sum to head_dim")
+    half = head_dim // 2
+    ang = np.zeros((txt_len + hp * wp, half), dtype=np.float64)
+    ii, jj = np.meshgrid(np.arange(hp), np.arange(wp), indexing="ij")
+    pos = [np.zeros(hp * wp), ii.reshape(-1).astype(np.float64), jj.reshape(-1).astype(np.float64)]
+    off = 0
+    for a, dim in enumerate(axes_dims_rope):
+        cnt = dim // 2
+        if a < 3 and cnt > 0:
+            omega = 1.0 / np.power(float(theta), 2.0 * np.arange(cnt) / float(dim))
+            ang[txt_len:, off:off + cnt] = pos[a][:, None] * omega[None, :]
+        off += cnt
+    cos = torch.from_numpy(np.cos(ang).astype(np.float32)).to(device)
+    sin = torch.from_numpy(np.sin(ang).astype(np.float32)).to(device)
+    return cos, sin

@@ -1,0 +1,200 @@
+/* mi_attention.h — flat C ABI of the MI355X (gfx950) attention library.
+ *
+ * This is the only boundary through which host code reaches HIP. It replaces, for
+ * the attention path, the brotensor operators the reference calls
+ * (paths below are relative to the reference repository root):
+ *
+ *   bt::flash_attention_forward            src/dit/common.cpp:194, :356, :376;
+ *                                          src/dit/qwenimage21_forward.cpp:648, :667, :674;
+ *                                          src/dit/pixart.cpp:340; src/dit/sana.cpp:623
+ *   bt::flash_attention_windowed_forward   src/dit/qwenimage21_forward.cpp:662
+ *   bt::rope_apply / rope_apply_perhead    src/dit/common.cpp:192-193;
+ *                                          src/dit/qwenimage21_forward.cpp:584-585;
+ *                                          src/triposplat/flow_model.cpp:374
+ *   ReLU linear-attention core             src/dit/sana.cpp:470-586
+ *
+ * Conventions (the reference's own C-API conventions, include/brodiffusion/krea2_capi.h:12-18):
+ *   - functions return 0 on success, -1 on failure; mi_last_error() holds the message
+ *     for the calling thread; no exception crosses the boundary;
+ *   - not thread-safe per stream: drive one stream from one thread;
+ *   - every launch goes on the stream given in the args (NULL = the library's current
+ *     stream, see mi_set_stream), performs no host synchronisation and allocates
+ *     nothing, so a caller may capture it in a HIP graph.
+ *
+ * Tensors are 2-D row-major per batch item: rows = tokens, cols = heads * head_dim,
+ * head h in columns [h*head_dim, (h+1)*head_dim). Strides are in ELEMENTS; a stride
+ * of 0 means dense (row stride = heads*head_dim, batch stride = rows*row stride).
+ */
+#ifndef MI_ATTENTION_H
+#define MI_ATTENTION_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#define MI_API __attribute__((visibility("default")))
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { MI_DTYPE_F16 = 1, MI_DTYPE_BF16 = 2 };
+enum { MI_MASK_NONE = 0, MI_MASK_CAUSAL = 1, MI_MASK_BLOCK_CAUSAL = 2 };
+enum { MI_MAX_SEGMENTS = 32 };
+
+/* Message for the most recent failure on this thread ("" if none). */
+MI_API const char* mi_last_error(void);
+MI_API const char* mi_version(void);
+
+typedef struct mi_device_info_t {
+    char name[128];
+    char arch[64];
+    int32_t compute_units;
+    int32_t clock_khz;
+    int32_t lds_bytes_per_cu;
+    int32_t l2_bytes;
+    int64_t hbm_bytes;
+    double peak_mfma_16bit_flops; /* compute_units * clock * 4096 FLOP/clk/CU (dense fp16/bf16) */
+} mi_device_info_t;
+MI_API int mi_device_info(mi_device_info_t* out);
+
+/* The library's current stream (void* is a hipStream_t). Entry points whose args carry a
+ * NULL stream launch here. Mirrors brotensor's cuda_current_stream() contract
+ * (src/fused_transformer.cu:38-54). */
+MI_API int mi_set_stream(void* stream);
+MI_API void* mi_get_stream(void);
+MI_API int mi_stream_synchronize(void* stream);
+
+/* Device memory for host code that owns no HIP of its own (the C++ Tensor type). */
+MI_API void* mi_malloc(size_t bytes);
+MI_API int mi_free(void* ptr);
+MI_API int mi_memcpy_h2d(void* dst, const void* src, size_t bytes);
+MI_API int mi_memcpy_d2h(void* dst, const void* src, size_t bytes);
+MI_API int mi_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream);
+MI_API int mi_memset_async(void* dst, int value, size_t bytes, void* stream);
+
+/* ── softmax attention ─────────────────────────────────────────────────────
+ * O = softmax(Q K^T * scale + mask) V per (batch, head), flash style: scores never
+ * reach HBM, softmax statistics and the output accumulate in FP32.
+ *
+ * Replaces bt::flash_attention_forward(Q,K,V,d_mask,num_heads,causal,out) and
+ * bt::flash_attention_windowed_forward(Q,K,V,d_mask,num_heads,window,out), plus what
+ * the reference does around them:
+ *   - k_prefix/v_prefix: leading key rows read from a second buffer, so the cached
+ *     prefix K/V of the Qwen-Image step (src/dit/qwenimage21_forward.cpp:599-649) is
+ *     consumed in place instead of being copied into [cache ; fresh];
+ *   - rope_*: RoPE applied to Q and to the rows of `k` as they are loaded, replacing the
+ *     two bt::rope_apply passes of dit::joint_attention (src/dit/common.cpp:188-196).
+ *     Adjacent-pair convention (x[2p], x[2p+1]); prefix rows are taken as already rotated
+ *     (the reference caches post-RoPE K, qwenimage21_forward.cpp:587-597);
+ *   - block-causal segments: the per-segment calls of the prefill form
+ *     (qwenimage21_forward.cpp:650-676) in one launch; key tiles no query row of a work
+ *     group can see are skipped.
+ *
+ * Keys are indexed over the concatenation [k_prefix ; k]: Lk = prefix_len + kv_len.
+ * Visibility of key j for query row r:
+ *   j < kv_valid_len[b]            (if given)
+ *   key_mask[b][j] != 0            (if given; FP32, 1 valid / 0 invalid,
+ *                                   include/brodiffusion/dit/common.h:138-139)
+ *   MI_MASK_CAUSAL:        j <= q_offset + r, and j > q_offset + r - window if window > 0
+ *   MI_MASK_BLOCK_CAUSAL:  with s the segment holding r (rows [seg_q_end[s-1], seg_q_end[s])):
+ *                          j < seg_k_end[s], and j <= q_offset + r if seg_causal[s]
+ * A query row with no visible key produces zeros (src/dit/common.cpp:293).
+ */
+typedef struct mi_sdpa_args {
+    uint32_t struct_size; /* = sizeof(mi_sdpa_args) */
+    int32_t dtype;        /* MI_DTYPE_F16 / MI_DTYPE_BF16: type of q, k, v, o */
+    const void* q;        /* (batch, q_len, heads*head_dim) */
+    const void* k;        /* (batch, kv_len, heads*head_dim) */
+    const void* v;
+    void* o;              /* (batch, q_len, heads*head_dim) */
+    const void* k_prefix; /* (batch, prefix_len, heads*head_dim) or NULL */
+    const void* v_prefix;
+    int32_t batch, num_heads, head_dim;
+    int32_t num_kv_heads; /* 0 or num_heads: plain MHA; a divisor of num_heads: grouped-query, query head h
+                             reads K/V head h / (num_heads/num_kv_heads), K/V rows are num_kv_heads*head_dim wide
+                             (replaces the K/V widening copies of dit::gqa_attention_masked, src/dit/common.cpp:333-378) */
+    int32_t q_len, kv_len, prefix_len;
+    int64_t q_row_stride, q_batch_stride;
+    int64_t k_row_stride, k_batch_stride;
+    int64_t v_row_stride, v_batch_stride;
+    int64_t o_row_stride, o_batch_stride;
+    int64_t kp_row_stride, kp_batch_stride;
+    int64_t vp_row_stride, vp_batch_stride;
+    float scale;                 /* <= 0: 1/sqrt(head_dim) */
+    int32_t mask_mode;           /* MI_MASK_* */
+    int32_t q_offset;            /* joint-sequence position of query row 0 */
+    int32_t window;              /* MI_MASK_CAUSAL only; 0 = unbounded */
+    const int32_t* kv_valid_len; /* device, [batch], or NULL */
+    const float* key_mask;       /* device, [batch or 1][Lk], or NULL */
+    int64_t key_mask_batch_stride; /* elements; 0 = one mask shared by all batch items */
+    int32_t n_segments;          /* MI_MASK_BLOCK_CAUSAL: 1..MI_MAX_SEGMENTS */
+    int32_t seg_q_end[MI_MAX_SEGMENTS];
+    int32_t seg_k_end[MI_MAX_SEGMENTS];
+    int32_t seg_causal[MI_MAX_SEGMENTS];
+    const float* rope_cos_q;     /* device FP32 (q_len, head_dim/2) or NULL */
+    const float* rope_sin_q;
+    const float* rope_cos_k;     /* device FP32 (kv_len, head_dim/2) or NULL; rows of `k` only */
+    const float* rope_sin_k;
+    void* stream;                /* hipStream_t; NULL = library current stream */
+} mi_sdpa_args;
+
+MI_API int mi_sdpa_forward(const mi_sdpa_args* args);
+/* 1 if (dtype, head_dim) has a compiled kernel, else 0. */
+MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);
+
+/* ── stand-alone RoPE ──────────────────────────────────────────────────────
+ * Replaces bt::rope_apply(X,cos,sin,head_dim,num_heads,out) and
+ * bt::rope_apply_perhead. Needed where the rotated tensor itself is kept (the prefix
+ * cache stores post-RoPE K). Tables are FP32 (rows, head_dim/2), or
+ * (rows*num_heads, head_dim/2) when per_head != 0. split_half = 0: pairs
+ * (x[2p], x[2p+1]); 1: pairs (x[p], x[p+head_dim/2]). In-place (out == x) is allowed. */
+typedef struct mi_rope_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* x;
+    void* out;
+    const float* cos;
+    const float* sin;
+    int32_t rows, num_heads, head_dim;
+    int64_t x_row_stride, out_row_stride;
+    int32_t split_half;
+    int32_t per_head;
+    void* stream;
+} mi_rope_args;
+MI_API int mi_rope_apply(const mi_rope_args* args);
+
+/* ── ReLU linear attention ─────────────────────────────────────────────────
+ * Per (batch, head): Kr = relu(K), Qr = relu(Q); S = V^T Kr (d x d), z = sum_n Kr (d);
+ * O[n] = (S Qr[n]) / (z . Qr[n] + eps). Replaces the core of
+ * SanaDenoiser::self_attention_ (src/dit/sana.cpp:470-586). Operands are token-major
+ * (batch, n_tokens, heads*head_dim). The FP32 state (S, z) lives in `workspace`
+ * ((batch*heads) blocks of head_dim*head_dim + head_dim floats, S row-major with rows =
+ * value channel, then z): after the call it holds the (S, z) the reference captures at
+ * its identity seam (sana.cpp:489-506). accumulate_state != 0 adds this call's (S, z) to
+ * what the workspace already holds instead of starting from zero (the inject form). */
+typedef struct mi_linear_attn_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    int32_t batch, num_heads, head_dim, n_tokens;
+    int64_t q_row_stride, q_batch_stride;
+    int64_t k_row_stride, k_batch_stride;
+    int64_t v_row_stride, v_batch_stride;
+    int64_t o_row_stride, o_batch_stride;
+    float eps;
+    int32_t accumulate_state;
+    void* workspace;
+    size_t workspace_bytes;
+    void* stream;
+} mi_linear_attn_args;
+MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
+MI_API int mi_linear_attn_relu_forward(const mi_linear_attn_args* args);
+MI_API int mi_linear_attn_supported(int32_t dtype, int32_t head_dim);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI_ATTENTION_H */

@@ -1,0 +1,252 @@
+"""GPU parity of the softmax-attention path against the CPU checker, through the C ABI."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import TOL, assert_close, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_batched(oracle, q, k, v, H, **kw):
+    return np.stack([oracle.sdpa(q[b], k[b], v[b], H, **kw) for b in range(q.shape[0])])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("d", [40, 64, 72, 80, 96, 112, 128, 160])
+def test_noncausal_all_head_dims(oracle, d, dtype):
+    B, H, Lq, Lk = 2, 2, 200, 333          # ragged: neither a multiple of the 128 / 64 tiles
+    q = randn(10 + d, (B, Lq, H * d), dtype); k = randn(20 + d, (B, Lk, H * d), dtype); v = randn(30 + d, (B, Lk, H * d), dtype)
+    out = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, H, False)
+    assert_close(_oracle_batched(oracle, q, k, v, H), to_np(out), dtype, f"d={d}")
+
+
+@pytest.mark.parametrize("Lq,Lk", [(1, 1), (1, 64), (64, 1), (128, 64), (129, 65), (127, 63), (300, 17), (5, 700)])
+def test_edge_lengths(oracle, Lq, Lk):
+    dtype, H, d = "bf16", 3, 128
+    q = randn(1, (Lq, H * d), dtype); k = randn(2, (Lk, H * d), dtype); v = randn(3, (Lk, H * d), dtype)
+    out = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, H, False)
+    assert_close(oracle.sdpa(q, k, v, H), to_np(out), dtype, f"{Lq}x{Lk}")
+
+
+def test_empty_query_is_noop():
+    dtype, H, d = "bf16", 2, 64
+    q = torch.empty((0, H * d), dtype=torch.bfloat16, device="cuda")
+    k = to_dev(randn(2, (8, H * d), dtype), dtype)
+    out = bd.flash_attention_forward(q, k, k, None, H, False)
+    assert out.shape == (0, H * d)
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72)])
+@pytest.mark.parametrize("window", [0, 50])
+def test_causal_windowed(oracle, dtype, d, window):
+    H, Lq, Lk = 2, 150, 290                  # q_offset = 140: the diagonal cuts tiles mid-way
+    q = randn(41, (Lq, H * d), dtype); k = randn(42, (Lk, H * d), dtype); v = randn(43, (Lk, H * d), dtype)
+    out = bd.flash_attention_windowed_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, H, window)
+    lo, hi = oracle.rows_causal(Lq, Lk, window=window)
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), to_np(out), dtype, f"window={window}")
+    if window == 0:
+        out2 = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, H, True)
+        assert torch.equal(out, out2)
+
+
+def test_causal_rows_without_keys_are_zero(oracle):
+    # q_offset = Lk - Lq < 0: the first rows see no key at all -> zeros (src/dit/common.cpp:293)
+    dtype, H, d, Lq, Lk = "bf16", 2, 64, 100, 40
+    q = randn(51, (Lq, H * d), dtype); k = randn(52, (Lk, H * d), dtype); v = randn(53, (Lk, H * d), dtype)
+    out = to_np(bd.flash_attention_windowed_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, H, 0))
+    lo, hi = oracle.rows_causal(Lq, Lk)
+    assert (hi[:59] == 0).all() and hi[60] == 1
+    assert not out[:60].any()
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), out, dtype)
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 72), ("fp16", 40), ("bf16", 128)])
+def test_key_mask_equals_trimmed(oracle, dtype, d):
+    """Key padding three ways (kv_valid_len, 0/1 d_mask, trimmed K/V) must agree: the reference handles
+    padding by trimming to the valid rows (src/pipeline.cpp:391-414)."""
+    B, H, Lq, Lk = 2, 2, 130, 300
+    valid = [77, 300]
+    q = randn(61, (B, Lq, H * d), dtype); k = randn(62, (B, Lk, H * d), dtype); v = randn(63, (B, Lk, H * d), dtype)
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    vl = torch.tensor(valid, dtype=torch.int32, device="cuda")
+    o_len = bd.sdpa_forward(dq, dk, dv, H, kv_valid_len=vl)
+    m = np.zeros((B, Lk), dtype=np.float32)
+    for b in range(B):
+        m[b, :valid[b]] = 1
+    o_mask = bd.flash_attention_forward(dq, dk, dv, torch.from_numpy(m).cuda(), H, False)
+    for b in range(B):
+        ref = oracle.sdpa(q[b], k[b, :valid[b]], v[b, :valid[b]], H)
+        assert_close(ref, to_np(o_len[b]), dtype, "kv_valid_len")
+        assert_close(ref, to_np(o_mask[b]), dtype, "d_mask")
+        o_trim = bd.flash_attention_forward(dq[b], dk[b, :valid[b]], dv[b, :valid[b]], None, H, False)
+        assert torch.equal(o_trim, o_len[b]) and torch.equal(o_trim, o_mask[b])
+
+
+def test_scattered_key_mask_and_empty_mask(oracle):
+    dtype, H, d, Lq, Lk = "bf16", 2, 128, 70, 200
+    q = randn(71, (Lq, H * d), dtype); k = randn(72, (Lk, H * d), dtype); v = randn(73, (Lk, H * d), dtype)
+    rng = np.random.default_rng(7)
+    m = (rng.uniform(size=Lk) > 0.5).astype(np.float32)
+    m[64:128] = 0                                   # one whole key tile masked out
+    out = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), torch.from_numpy(m).cuda(), H, False)
+    assert_close(oracle.sdpa(q, k, v, H, key_mask=m), to_np(out), dtype)
+    out0 = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), torch.zeros(Lk, device="cuda"), H, False)
+    assert not to_np(out0).any()
+
+
+def _block_causal_case(prefix, blocks):
+    """cfg4-shaped: cached prefix of `prefix` text keys; query blocks of sizes `blocks`; block b sees
+    the prefix plus blocks 0..b."""
+    seg_q_end = list(np.cumsum(blocks))
+    seg_k_end = [prefix + e for e in seg_q_end]
+    return seg_q_end, seg_k_end, [0] * len(blocks)
+
+
+@pytest.mark.parametrize("prefix,blocks", [(96, [80, 80, 80, 80]), (64, [128, 128]), (70, [33, 190, 60])])
+def test_block_causal_prefix_kv(oracle, prefix, blocks):
+    dtype, H, d = "bf16", 2, 128
+    Lq = sum(blocks)
+    q = randn(81, (Lq, H * d), dtype); kf = randn(82, (Lq, H * d), dtype); vf = randn(83, (Lq, H * d), dtype)
+    kp = randn(84, (prefix, H * d), dtype); vp = randn(85, (prefix, H * d), dtype)
+    sq, sk, sc = _block_causal_case(prefix, blocks)
+    mask = bd.SdpaMask.block_causal(prefix, sq, sk, sc)
+    out = bd.sdpa_forward(to_dev(q, dtype), to_dev(kf, dtype), to_dev(vf, dtype), H, k_prefix=to_dev(kp, dtype),
+                          v_prefix=to_dev(vp, dtype), mask=mask)
+    k = np.concatenate([kp, kf]); v = np.concatenate([vp, vf])
+    lo, hi = oracle.rows_block_causal(Lq, prefix + Lq, prefix, sq, sk, sc)
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), to_np(out), dtype)
+    # the reference reaches the same result as one unmasked call per image segment over keys [0, e)
+    # (src/dit/qwenimage21_forward.cpp:664-669); tile skipping must not change visible-tile numerics
+    dk, dv = to_dev(k, dtype), to_dev(v, dtype)
+    s = 0
+    for e, ke in zip(sq, sk):
+        seg = bd.flash_attention_forward(to_dev(q[s:e], dtype), dk[:ke], dv[:ke], None, H, False)
+        assert torch.equal(seg, out[s:e])
+        s = e
+
+
+def test_block_causal_with_text_segments(oracle):
+    """Prefill form with causal text runs and bidirectional image blocks in one launch
+    (src/dit/qwenimage21_forward.cpp:650-676)."""
+    dtype, H, d = "bf16", 2, 128
+    kinds = [("t", 70), ("i", 100), ("t", 30), ("i", 150)]
+    L = sum(n for _, n in kinds)
+    sq = list(np.cumsum([n for _, n in kinds])); sk = sq; sc = [1 if kd == "t" else 0 for kd, _ in kinds]
+    q = randn(91, (L, H * d), dtype); k = randn(92, (L, H * d), dtype); v = randn(93, (L, H * d), dtype)
+    out = bd.sdpa_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, mask=bd.SdpaMask.block_causal(0, sq, sk, sc))
+    block_id, img = [], 0
+    for kd, n in kinds:
+        block_id += [-1] * n if kd == "t" else [img] * n
+        img += kd == "i"
+    dense = oracle.dense_block_causal(L, L, 0, block_id)
+    assert_close(oracle.sdpa(q, k, v, H, dense_mask=dense), to_np(out), dtype)
+    # per-segment calls through the reference's own entry points
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    s = 0
+    for (kd, n), e in zip(kinds, sq):
+        if kd == "t":
+            seg = bd.flash_attention_windowed_forward(dq[s:e], dk[:e], dv[:e], None, H, 0)
+        else:
+            seg = bd.flash_attention_forward(dq[s:e], dk[:e], dv[:e], None, H, False)
+        assert torch.equal(seg, out[s:e])
+        s = e
+
+
+@pytest.mark.parametrize("dtype,d,axes", [("bf16", 128, (16, 56, 56)), ("fp16", 64, (16, 24, 24)), ("bf16", 40, (8, 16, 16))])
+def test_joint_attention_fused_rope(oracle, dtype, d, axes):
+    H, txt, hp, wp = 2, 37, 9, 11
+    L = txt + hp * wp
+    q = randn(101, (L, H * d), dtype); k = randn(102, (L, H * d), dtype); v = randn(103, (L, H * d), dtype)
+    cos, sin = bd.build_axial_rope_tables(txt, hp, wp, d, axes)
+    ocos, osin = oracle.build_axial_rope_tables(txt, hp, wp, d, axes)
+    assert np.max(np.abs(to_np(cos) - ocos)) < 1e-6 and np.max(np.abs(to_np(sin) - osin)) < 1e-6
+    out = bd.joint_attention(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), cos, sin, d, H)
+    # the reference rotates into tensors of Q's dtype before attention (src/dit/common.cpp:192-193)
+    qr = oracle.rope_apply(q, ocos, osin, H, d, round_to_dtype=dtype)
+    kr = oracle.rope_apply(k, ocos, osin, H, d, round_to_dtype=dtype)
+    assert_close(oracle.sdpa(qr, kr, v, H), to_np(out), dtype)
+    # fused == stand-alone rope_apply followed by plain attention
+    dqr = bd.rope_apply(to_dev(q, dtype), cos, sin, d, H)
+    dkr = bd.rope_apply(to_dev(k, dtype), cos, sin, d, H)
+    out2 = bd.flash_attention_forward(dqr, dkr, to_dev(v, dtype), None, H, False)
+    assert torch.equal(out, out2)
+
+
+def test_rope_on_fresh_keys_only_with_prefix(oracle):
+    """Cached step: prefix K is stored post-RoPE, fresh K and Q are rotated with the table rows of
+    their positions (src/dit/qwenimage21_forward.cpp:301-307, :587-649)."""
+    dtype, H, d, prefix, hp, wp = "bf16", 2, 128, 50, 8, 8
+    img = hp * wp
+    cos, sin = oracle.build_qwen_rope_tables([("text", prefix)], hp, wp, d)
+    k_all = randn(111, (prefix + img, H * d), dtype); v_all = randn(112, (prefix + img, H * d), dtype)
+    q = randn(113, (img, H * d), dtype)
+    kr_all = oracle.rope_apply(k_all, cos, sin, H, d, round_to_dtype=dtype)
+    qr = oracle.rope_apply(q, cos[prefix:], sin[prefix:], H, d, round_to_dtype=dtype)
+    ref = oracle.sdpa(qr, kr_all, v_all, H)
+    tc = torch.from_numpy(cos[prefix:].copy()).cuda(); ts = torch.from_numpy(sin[prefix:].copy()).cuda()
+    out = bd.sdpa_forward(to_dev(q, dtype), to_dev(k_all[prefix:], dtype), to_dev(v_all[prefix:], dtype), H,
+                          k_prefix=to_dev(kr_all[:prefix], dtype), v_prefix=to_dev(v_all[:prefix], dtype),
+                          rope_q=(tc, ts), rope_k=(tc, ts))
+    assert_close(ref, to_np(out), dtype)
+
+
+def test_gqa_masked(oracle):
+    dtype, d, Hq, Hkv, L = "bf16", 128, 4, 2, 150
+    q = randn(121, (L, Hq * d), dtype); k = randn(122, (L, Hkv * d), dtype); v = randn(123, (L, Hkv * d), dtype)
+    m = np.ones(L, dtype=np.float32); m[120:] = 0
+    out = bd.gqa_attention_masked(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), None, None, d, Hq, Hkv,
+                                  torch.from_numpy(m).cuda())
+    # widen K/V as the reference does (src/dit/common.cpp:359-375): kv head g serves q heads [g*r, (g+1)*r)
+    kw = k.reshape(L, Hkv, 1, d).repeat(2, axis=2).reshape(L, Hq * d)
+    vw = v.reshape(L, Hkv, 1, d).repeat(2, axis=2).reshape(L, Hq * d)
+    assert_close(oracle.sdpa(q, kw, vw, Hq, key_mask=m), to_np(out), dtype)
+
+
+def test_scale_strides_and_views(oracle):
+    dtype, H, d, Lq, Lk = "fp16", 2, 64, 90, 140
+    q = randn(131, (Lq, H * d), dtype); k = randn(132, (Lk, H * d), dtype); v = randn(133, (Lk, H * d), dtype)
+    # K and V as column slices of one packed (Lk, 2*H*d) tensor: row stride != H*d
+    kv = torch.cat([to_dev(k, dtype), to_dev(v, dtype)], dim=1)
+    out = torch.zeros((Lq, 2 * H * d), dtype=torch.float16, device="cuda")
+    bd.sdpa_forward(to_dev(q, dtype), kv[:, :H * d], kv[:, H * d:], H, scale=0.2, out=out[:, H * d:])
+    assert_close(oracle.sdpa(q, k, v, H, scale=0.2), to_np(out[:, H * d:]), dtype)
+    assert not out[:, :H * d].any()
+
+
+def test_deterministic(oracle):
+    dtype, H, d, L = "bf16", 4, 128, 500
+    dq, dk, dv = (to_dev(randn(s, (L, H * d), dtype), dtype) for s in (141, 142, 143))
+    a = bd.flash_attention_forward(dq, dk, dv, None, H, False)
+    b = bd.flash_attention_forward(dq, dk, dv, None, H, False)
+    assert torch.equal(a, b)          # bit-exact across runs, as the reference's smoke tests demand
+
+
+def test_closed_forms_on_device():
+    dtype, H, d, Lq, Lk = "bf16", 2, 128, 100, 260
+    q = to_dev(randn(151, (Lq, H * d), dtype), dtype)
+    v = randn(152, (Lk, H * d), dtype)
+    k_same = to_dev(np.tile(randn(153, (1, H * d), dtype), (Lk, 1)), dtype)
+    out = to_np(bd.flash_attention_forward(q, k_same, to_dev(v, dtype), None, H, False))
+    assert np.max(np.abs(out - v.mean(axis=0)[None, :])) < 2e-2     # equal keys -> mean of V
+    v_const = np.tile(randn(154, (1, H * d), dtype), (Lk, 1))
+    k = to_dev(randn(155, (Lk, H * d), dtype), dtype)
+    out = to_np(bd.flash_attention_forward(q, k, to_dev(v_const, dtype), None, H, False))
+    assert np.max(np.abs(out - v_const[:1])) < 2e-2                 # constant V -> that constant
+
+
+def test_errors():
+    q = torch.zeros((8, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="flash_attention_forward: D must equal"):
+        bd.flash_attention_forward(q, q, q, None, 3, False)
+    with pytest.raises(RuntimeError, match="no kernel"):
+        bd.flash_attention_forward(q, q, q, None, 8, False)          # head_dim 32
+    with pytest.raises(RuntimeError, match="not on the GPU"):
+        bd.flash_attention_forward(q.cpu(), q, q, None, 2, False)
+    with pytest.raises(RuntimeError, match="dtype"):
+        bd.flash_attention_forward(q.float(), q.float(), q.float(), None, 2, False)
+    with pytest.raises(RuntimeError, match="K and V must be"):
+        bd.flash_attention_forward(q, q[:, :128], q, None, 2, False)
