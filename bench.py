@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Attention hot-path benchmark on one MI355X.
+
+A step is one call of the hot path on the headline workload: Flux.1 double-stream joint attention,
+B=1, H=24, head_dim=128, 512 text + 4096 image tokens, bf16, RoPE (axes 16/56/56, theta 1e4) applied
+to Q and K inside the attention launch. Inputs are synthetic N(0,1), resident in HBM before the
+timed region. Prints ONE JSON line.
+
+  metric      attention TFLOP/s, algorithmic FLOPs = 4 * B * H * Lq * Lk * d (QK^T and PV, nothing else)
+  roofline    the flash kernel against MI355X dense bf16 MFMA peak (2.5 PFLOP/s), kernel time from HIP
+              events on the launch stream over the timed region
+  cpu_baseline the CPU checker (a port of the reference's FP32/FP64 host attention loop) timed on this
+              host's cores on a bounded sample of the same workload
+  configs     ms per call and TFLOP/s (GB/s for linear attention) of every BASELINE config, measured
+              outside the timed region
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
+PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, published
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured.
+TRAFFIC_BYTES_PER_LAUNCH = None
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true")
+    return ap.parse_args()
+
+
+def event_ms(torch, fn, iters, warm=3):
+    """Per-call milliseconds (min, mean) from HIP events on the current stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = [a.elapsed_time(b) for a, b in evs]
+    return min(ts), sum(ts) / len(ts)
+
+
+def all_configs(torch, bd):
+    """Every BASELINE config: ms per call (min and mean over 20 calls), TFLOP/s or GB/s, fraction of peak."""
+    g = torch.Generator(device="cuda").manual_seed(1234)
+
+    def rnd(*shape, dt=torch.bfloat16):
+        return torch.randn(*shape, device="cuda", dtype=torch.float32, generator=g).to(dt)
+
+    out = {}
+
+    def sdpa_entry(name, flops, fn, dtype):
+        mn, av = event_ms(torch, fn, 20)
+        out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "tflops": round(flops / (mn * 1e-3) / 1e12, 1),
+                     "frac_mfma_peak": round(flops / (mn * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, 4), "dtype": dtype,
+                     "gflop": round(flops / 1e9, 2)}
+
+    q, k, v = (rnd(2, 4096, 320, dt=torch.float16) for _ in range(3))
+    sdpa_entry("cfg1_sd15_selfattn_d40_fp16", 4 * 2 * 8 * 4096 * 4096 * 40, lambda: bd.flash_attention_forward(q, k, v, None, 8, False), "fp16")
+    q, k, v = (rnd(2, 4096, 1152) for _ in range(3))
+    sdpa_entry("cfg2a_pixart_selfattn_d72_bf16", 4 * 2 * 16 * 4096 * 4096 * 72, lambda: bd.flash_attention_forward(q, k, v, None, 16, False), "bf16")
+    kc, vc = rnd(2, 300, 1152), rnd(2, 300, 1152)
+    gen = torch.Generator().manual_seed(2099)
+    valid = [int(20 + torch.randint(0, 281, (1,), generator=gen).item()) for _ in range(2)]
+    vl = torch.tensor(valid, dtype=torch.int32, device="cuda")
+    sdpa_entry("cfg2b_pixart_crossattn_d72_bf16", 4 * 16 * 4096 * sum(valid) * 72, lambda: bd.sdpa_forward(q, kc, vc, 16, kv_valid_len=vl), "bf16")
+    out["cfg2b_pixart_crossattn_d72_bf16"]["valid_len"] = valid
+    q, k, v = (rnd(4608, 3072) for _ in range(3))
+    cos, sin = bd.build_axial_rope_tables(512, 64, 64, 128, (16, 56, 56))
+    sdpa_entry("cfg3_flux_joint_d128_bf16_rope", 4 * 24 * 4608 * 4608 * 128, lambda: bd.joint_attention(q, k, v, cos, sin, 128, 24), "bf16")
+    qb, kb, vb = (rnd(4096, 3072) for _ in range(3))
+    kp, vp = rnd(512, 3072), rnd(512, 3072)
+    sq = [1024, 2048, 3072, 4096]
+    sk = [512 + e for e in sq]
+    mask = bd.SdpaMask.block_causal(512, sq, sk, [0] * 4)
+    sdpa_entry("cfg4_qwen_blockcausal_prefixkv_d128_bf16", 4 * 24 * sum(1024 * e for e in sk) * 128,
+               lambda: bd.sdpa_forward(qb, kb, vb, 24, k_prefix=kp, v_prefix=vp, mask=mask), "bf16")
+    out["cfg4_qwen_blockcausal_prefixkv_d128_bf16"]["dense_equivalent_gflop"] = round(4 * 24 * 4096 * 4608 * 128 / 1e9, 2)
+    for name, n in (("cfg5a_sana_linear_n1024_d112_bf16", 1024), ("cfg5b_sana_linear_n4096_d112_bf16", 4096)):
+        ql, kl, vl_ = (rnd(2, n, 2240) for _ in range(3))
+        ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
+        o = torch.empty_like(ql)
+        mn, av = event_ms(torch, lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws), 20)
+        nbytes = 4 * 2 * n * 2240 * 2
+        out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
+                     "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16 in, f32 accumulate",
+                     "mbytes": round(nbytes / 1e6, 2)}
+    return out
+
+
+def cpu_baseline():
+    """The CPU checker on a bounded sample of the headline workload: RoPE on all of Q and K, then the
+    exact attention loop for a subset of query rows (all heads, all 4608 keys), sized for ~10-20 s."""
+    import numpy as np
+    import oracle as orc
+    H, d, L = 24, 128, 4608
+    q, k, v = (orc.round_to(orc.torch_randn_f32(3000 + i, L * H * d).reshape(L, H * d), "bf16") for i in (1, 2, 3))
+    cos, sin = orc.build_axial_rope_tables(512, 64, 64, d, (16, 56, 56))
+    threads = orc.max_threads()
+    probe = np.arange(0, L, L // 32, dtype=np.int32)[:32]
+    t0 = time.perf_counter()
+    orc.sdpa(q, k, v, H, rows=probe)
+    per_row = (time.perf_counter() - t0) / len(probe)
+    n_rows = int(max(64, min(L, 12.0 / max(per_row, 1e-6))))
+    rows = np.unique(np.linspace(0, L - 1, n_rows).astype(np.int32))
+    t0 = time.perf_counter()
+    qr = orc.rope_apply(q, cos, sin, H, d, round_to_dtype="bf16")
+    kr = orc.rope_apply(k, cos, sin, H, d, round_to_dtype="bf16")
+    orc.sdpa(qr, kr, v, H, rows=rows)
+    dt = time.perf_counter() - t0
+    flops = 4.0 * H * len(rows) * L * d
+    return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{len(rows)} of {L} query rows x 24 heads x all 4608 keys, RoPE on all of Q and K included, "
+                      f"{dt:.1f} s on {threads} OpenMP threads; full call extrapolates to {dt * L / len(rows):.0f} s"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {args.gpus}): this attention path has no multi-GPU leg; "
+              "heads shard across GPUs without exchange.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import brodiffusion_amd as bd
+    from brodiffusion_amd import _capi
+    _capi.lib()                              # fails loudly if the HIP extension is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    B, H, d, txt, hp, wp = 1, 24, 128, 512, 64, 64
+    L = txt + hp * wp
+    g = torch.Generator(device="cuda").manual_seed(3000)
+    q, k, v = (torch.randn(L, H * d, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(3))
+    cos, sin = bd.build_axial_rope_tables(txt, hp, wp, d, (16, 56, 56))
+    out = torch.empty_like(q)
+    flops = 4.0 * B * H * L * L * d
+
+    def step():
+        bd.joint_attention(q, k, v, cos, sin, d, H, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = e0.elapsed_time(e1) / args.steps      # back-to-back launches of the one kernel on this stream
+
+    ms_per_step = wall * 1e3 / args.steps
+    achieved = flops / (kernel_ms * 1e-3) / 1e12
+    res = {
+        "metric": "attention TFLOP/s + % of MI355X bf16 MFMA peak (Flux 4608-token SDPA)",
+        "value": round(flops / (ms_per_step * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "Flux.1 joint attention B=1 H=24 d=128 L=512+4096, RoPE axes 16/56/56 fused into Q/K load, non-causal",
+                   "gflop_per_step": round(flops / 1e9, 2)},
+        "pct_of_mfma_peak": round(100.0 * achieved / PEAK_MFMA_BF16_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_MFMA_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "sdpa_fwd_kernel<bf16, 128, rope>", "kernel_ms": round(kernel_ms, 4)},
+        "device": bd.device_info(),
+    }
+    if not args.no_configs:
+        res["configs"] = all_configs(torch, bd)
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

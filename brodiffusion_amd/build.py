@@ -54,5 +54,36 @@ def build(save_temps: bool = False, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(LIB_DIR, "libbrodiffusion_amd_host.so")
+HOST_TEST = os.path.join(LIB_DIR, "test_host_ops")
+CXX = os.environ.get("CXX", "g++")
+
+
+def build_host(with_test: bool = True, verbose: bool = False) -> str:
+    """C++20 host operator layer (no HIP in it; g++) on top of the C ABI, plus its test executable,
+    which also links the CPU checker (test-only)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    common = [CXX, "-std=c++20", "-O2", "-fPIC", "-Wall", "-Wextra", "-I" + os.path.join(ROOT, "include"), "-I" + HOST_DIR]
+    rpath = ["-Wl,-rpath,$ORIGIN", "-L" + LIB_DIR]
+    cmd = [*common, "-shared", os.path.join(HOST_DIR, "attention_ops.cpp"), "-o", HOST_LIB, *rpath, "-lmi_attention"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(r.stdout + r.stderr)
+        raise RuntimeError("host library build failed")
+    if with_test:
+        oracle_dir = os.path.join(ROOT, "oracle")
+        cmd = [*common, os.path.join(ROOT, "tests", "cpp", "test_host_ops.cpp"), "-o", HOST_TEST, *rpath,
+               "-Wl,-rpath,$ORIGIN/../../oracle", "-L" + oracle_dir, "-lbrodiffusion_amd_host", "-lmi_attention", "-loracle"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("host test build failed")
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
+
+
 if __name__ == "__main__":
     build(save_temps="--save-temps" in sys.argv, verbose=True)
+    build_host(verbose=True)

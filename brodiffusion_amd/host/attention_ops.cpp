@@ -1,0 +1,231 @@
+#include "attention_ops.h"
+
+#include <cmath>
+#include <cstring>
+
+namespace bdamd {
+namespace {
+
+int dtype_code(const char* op, Dtype d) {
+    if (d == Dtype::BF16) return MI_DTYPE_BF16;
+    if (d == Dtype::FP16) return MI_DTYPE_F16;
+    fail(std::string(op) + ": dtype must be FP16 or BF16 on the GPU path");
+}
+void need_gpu(const char* op, const Tensor& t) {
+    if (t.device != Device::GPU) fail(std::string(op) + ": tensor is on the CPU; this path is GPU-only and does not copy");
+    if (t.size() != 0 && t.data == nullptr) fail(std::string(op) + ": tensor has no storage");
+}
+void check(const char* op, int rc) {
+    if (rc != 0) fail(std::string(op) + ": " + mi_last_error());
+}
+void init_args(mi_sdpa_args& a, const char* op, const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads,
+               int num_kv_heads, Tensor& out) {
+    need_gpu(op, Q); need_gpu(op, K); need_gpu(op, V);
+    if (num_heads <= 0 || Q.cols % num_heads != 0) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    const int hd = Q.cols / num_heads;
+    const int dt = dtype_code(op, Q.dtype);
+    if (K.dtype != Q.dtype || V.dtype != Q.dtype) fail(std::string(op) + ": Q, K, V must share one dtype");
+    if (K.cols != num_kv_heads * hd || V.cols != K.cols || V.rows != K.rows)
+        fail(std::string(op) + ": K and V must be (Lk, kv_heads*head_dim)");
+    if (out.data == nullptr || out.rows != Q.rows || out.cols != Q.cols || out.dtype != Q.dtype)
+        out.resize(Q.rows, Q.cols, Q.dtype, Q.device);
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dt;
+    a.q = Q.data; a.k = K.data; a.v = V.data; a.o = out.data;
+    a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.num_kv_heads = num_kv_heads;
+    a.q_len = Q.rows; a.kv_len = K.rows;
+}
+void set_rope(mi_sdpa_args& a, const char* op, const Tensor* cos, const Tensor* sin, int rows, bool for_q) {
+    if (!cos && !sin) return;
+    if (!cos || !sin) fail(std::string(op) + ": cos and sin must be given together");
+    need_gpu(op, *cos); need_gpu(op, *sin);
+    if (cos->dtype != Dtype::FP32 || sin->dtype != Dtype::FP32) fail(std::string(op) + ": RoPE tables must be FP32");
+    if (cos->rows != rows || sin->rows != rows || cos->cols != a.head_dim / 2 || sin->cols != a.head_dim / 2)
+        fail(std::string(op) + ": RoPE tables must be (L, head_dim/2)");
+    if (for_q) { a.rope_cos_q = static_cast<const float*>(cos->data); a.rope_sin_q = static_cast<const float*>(sin->data); }
+    else { a.rope_cos_k = static_cast<const float*>(cos->data); a.rope_sin_k = static_cast<const float*>(sin->data); }
+}
+
+}  // namespace
+
+namespace bt {
+
+void flash_attention_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask, int num_heads,
+                             bool causal, Tensor& out) {
+    const char* op = "flash_attention_forward";
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_heads, num_heads, out);
+    a.key_mask = d_mask;
+    if (causal) { a.mask_mode = MI_MASK_CAUSAL; a.q_offset = K.rows - Q.rows; }
+    check(op, mi_sdpa_forward(&a));
+}
+
+void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask,
+                                      int num_heads, int window, Tensor& out) {
+    const char* op = "flash_attention_windowed_forward";
+    if (window < 0) fail(std::string(op) + ": window must be >= 0");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_heads, num_heads, out);
+    a.key_mask = d_mask;
+    a.mask_mode = MI_MASK_CAUSAL; a.q_offset = K.rows - Q.rows; a.window = window;
+    check(op, mi_sdpa_forward(&a));
+}
+
+static void rope_impl(const char* op, const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads,
+                      Tensor& out, bool per_head) {
+    need_gpu(op, X); need_gpu(op, cos); need_gpu(op, sin);
+    if (head_dim <= 0 || num_heads <= 0 || X.cols != head_dim * num_heads) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    const int trows = per_head ? X.rows * num_heads : X.rows;
+    if (cos.dtype != Dtype::FP32 || sin.dtype != Dtype::FP32 || cos.rows != trows || sin.rows != trows ||
+        cos.cols != head_dim / 2 || sin.cols != head_dim / 2)
+        fail(std::string(op) + ": cos/sin must be FP32 (rows, head_dim/2)");
+    if (out.data == nullptr || out.rows != X.rows || out.cols != X.cols || out.dtype != X.dtype)
+        out.resize(X.rows, X.cols, X.dtype, X.device);
+    mi_rope_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    a.x = X.data; a.out = out.data;
+    a.cos = static_cast<const float*>(cos.data); a.sin = static_cast<const float*>(sin.data);
+    a.rows = X.rows; a.num_heads = num_heads; a.head_dim = head_dim; a.per_head = per_head ? 1 : 0;
+    check(op, mi_rope_apply(&a));
+}
+void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out) {
+    rope_impl("rope_apply", X, cos, sin, head_dim, num_heads, out, false);
+}
+void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out) {
+    rope_impl("rope_apply_perhead", X, cos, sin, head_dim, num_heads, out, true);
+}
+
+void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
+                                   Tensor& state, Tensor& out, bool accumulate_state) {
+    const char* op = "linear_attention_relu_forward";
+    need_gpu(op, Q); need_gpu(op, K); need_gpu(op, V);
+    if (num_heads <= 0 || Q.cols % num_heads != 0) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if (K.rows != Q.rows || V.rows != Q.rows || K.cols != Q.cols || V.cols != Q.cols || K.dtype != Q.dtype || V.dtype != Q.dtype)
+        fail(std::string(op) + ": Q/K/V must share shape (N, D) and dtype");
+    const int hd = Q.cols / num_heads;
+    const int per_head = hd * hd + hd;
+    if (accumulate_state) {
+        if (state.data == nullptr || state.rows != num_heads || state.cols != per_head || state.dtype != Dtype::FP32)
+            fail(std::string(op) + ": accumulate_state needs a (heads, d*d+d) FP32 state");
+    } else if (state.data == nullptr || state.rows != num_heads || state.cols != per_head || state.dtype != Dtype::FP32) {
+        state.resize(num_heads, per_head, Dtype::FP32, Q.device);
+    }
+    if (out.data == nullptr || out.rows != Q.rows || out.cols != Q.cols || out.dtype != Q.dtype)
+        out.resize(Q.rows, Q.cols, Q.dtype, Q.device);
+    mi_linear_attn_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, Q.dtype);
+    a.q = Q.data; a.k = K.data; a.v = V.data; a.o = out.data;
+    a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.n_tokens = Q.rows;
+    a.eps = eps; a.accumulate_state = accumulate_state ? 1 : 0;
+    a.workspace = state.data; a.workspace_bytes = state.bytes();
+    check(op, mi_linear_attn_relu_forward(&a));
+}
+
+}  // namespace bt
+
+namespace dit {
+
+RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const std::vector<int>& axes, float theta) {
+    if (head_dim % 2 != 0) fail("build_axial_rope_tables: head_dim must be even");
+    int sum = 0;
+    for (int d : axes) sum += d;
+    if (sum != head_dim) fail("build_axial_rope_tables: axes_dims_rope must sum to head_dim");
+    const int half = head_dim / 2;
+    const std::size_t L = static_cast<std::size_t>(txt_len) + static_cast<std::size_t>(hp) * wp;
+    std::vector<float> cs(L * half, 1.0f), sn(L * half, 0.0f);
+    // per pair: owning axis and angular frequency theta^(-2p/D_a); positions (0, i, j)
+    std::vector<int> pair_axis(half);
+    std::vector<double> omega(half);
+    int off = 0;
+    for (std::size_t a = 0; a < axes.size(); ++a) {
+        for (int p = 0; p < axes[a] / 2; ++p) {
+            pair_axis[off + p] = static_cast<int>(a);
+            omega[off + p] = std::pow(static_cast<double>(theta), -2.0 * p / static_cast<double>(axes[a]));
+        }
+        off += axes[a] / 2;
+    }
+    for (int i = 0; i < hp; ++i)
+        for (int j = 0; j < wp; ++j) {
+            const std::size_t row = static_cast<std::size_t>(txt_len) + static_cast<std::size_t>(i) * wp + j;
+            for (int p = 0; p < half; ++p) {
+                const int ax = pair_axis[p];
+                if (ax > 2) continue;
+                const double ang = (ax == 0 ? 0.0 : ax == 1 ? static_cast<double>(i) : static_cast<double>(j)) * omega[p];
+                cs[row * half + p] = static_cast<float>(std::cos(ang));
+                sn[row * half + p] = static_cast<float>(std::sin(ang));
+            }
+        }
+    RopeTables t;
+    t.cos = Tensor::from_host(cs.data(), static_cast<int>(L), half, Dtype::FP32);
+    t.sin = Tensor::from_host(sn.data(), static_cast<int>(L), half, Dtype::FP32);
+    return t;
+}
+
+void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin, int head_dim,
+                     int num_heads, Tensor& out, Tensor& /*Qr*/, Tensor& /*Kr*/) {
+    const char* op = "joint_attention";
+    if (head_dim <= 0 || num_heads <= 0 || Q.cols != head_dim * num_heads) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if (K.rows != Q.rows || V.rows != Q.rows || K.cols != Q.cols || V.cols != Q.cols) fail(std::string(op) + ": Q/K/V must share shape (L, D)");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_heads, num_heads, out);
+    set_rope(a, op, &cos, &sin, Q.rows, true);
+    set_rope(a, op, &cos, &sin, K.rows, false);
+    check(op, mi_sdpa_forward(&a));
+}
+
+void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin, int head_dim,
+                          int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out, Tensor& /*Qr*/, Tensor& /*Kr*/,
+                          Tensor& /*Krep*/, Tensor& /*Vrep*/) {
+    const char* op = "gqa_attention_masked";
+    if (num_kv_heads <= 0 || num_q_heads <= 0 || num_q_heads % num_kv_heads != 0)
+        fail(std::string(op) + ": num_kv_heads must divide num_q_heads");
+    if (Q.cols != head_dim * num_q_heads) fail(std::string(op) + ": D must equal head_dim * num_q_heads");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_q_heads, num_kv_heads, out);
+    a.key_mask = d_mask;
+    set_rope(a, op, cos, sin, Q.rows, true);
+    set_rope(a, op, cos, sin, K.rows, false);
+    check(op, mi_sdpa_forward(&a));
+}
+
+void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix, const Tensor* v_prefix,
+                            const std::vector<Segment>& segments, int q_offset, int num_heads, const Tensor* cos_q,
+                            const Tensor* sin_q, Tensor& out) {
+    const char* op = "block_causal_attention";
+    if (segments.empty() || segments.size() > static_cast<std::size_t>(MI_MAX_SEGMENTS))
+        fail(std::string(op) + ": between 1 and 32 segments");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_heads, num_heads, out);
+    if ((k_prefix == nullptr) != (v_prefix == nullptr)) fail(std::string(op) + ": prefix K and V must be given together");
+    if (k_prefix && k_prefix->rows > 0) {
+        need_gpu(op, *k_prefix); need_gpu(op, *v_prefix);
+        if (k_prefix->cols != K.cols || v_prefix->cols != K.cols || v_prefix->rows != k_prefix->rows ||
+            k_prefix->dtype != Q.dtype || v_prefix->dtype != Q.dtype)
+            fail(std::string(op) + ": prefix K/V must be (prefix_len, D) in Q's dtype");
+        a.k_prefix = k_prefix->data; a.v_prefix = v_prefix->data; a.prefix_len = k_prefix->rows;
+    }
+    a.mask_mode = MI_MASK_BLOCK_CAUSAL;
+    a.q_offset = q_offset;
+    a.n_segments = static_cast<int>(segments.size());
+    int row = 0;
+    for (std::size_t s = 0; s < segments.size(); ++s) {
+        row += segments[s].n_tokens;
+        a.seg_q_end[s] = row;
+        a.seg_k_end[s] = q_offset + row;           // a segment sees every key up to its own end
+        a.seg_causal[s] = segments[s].kind == Segment::Kind::Text ? 1 : 0;
+    }
+    if (row != Q.rows) fail(std::string(op) + ": segments must cover exactly Q's rows");
+    // fresh keys get the same table rows as the queries when Q and K cover the same positions
+    set_rope(a, op, cos_q, sin_q, Q.rows, true);
+    if (cos_q && K.rows == Q.rows) set_rope(a, op, cos_q, sin_q, K.rows, false);
+    else if (cos_q) fail(std::string(op) + ": fused RoPE needs K and Q to cover the same positions");
+    check(op, mi_sdpa_forward(&a));
+}
+
+}  // namespace dit
+}  // namespace bdamd

@@ -1,0 +1,66 @@
+// Host-side operator interface of the attention path, C++20, no HIP: every computation is a call
+// into the C ABI of libmi_attention.so. Names and argument order follow the brotensor operators and
+// the brodiffusion wrappers the reference calls (paths in the reference repository):
+//   bt::flash_attention_forward            src/dit/common.cpp:194
+//   bt::flash_attention_windowed_forward   src/dit/qwenimage21_forward.cpp:662
+//   bt::rope_apply / rope_apply_perhead    src/dit/common.cpp:192, src/triposplat/flow_model.cpp:374
+//   dit::joint_attention                   include/brodiffusion/dit/common.h:80-88
+//   dit::gqa_attention_masked              include/brodiffusion/dit/common.h:144-153
+//   dit::build_axial_rope_tables           include/brodiffusion/dit/common.h:70-72
+// Precondition failures throw std::runtime_error("<op>: <message>"); a CPU tensor is refused.
+#pragma once
+#include <vector>
+
+#include "tensor.h"
+
+namespace bdamd {
+namespace bt {
+
+void flash_attention_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask,
+                             int num_heads, bool causal, Tensor& out);
+void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask,
+                                      int num_heads, int window, Tensor& out);
+void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
+void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
+
+// Sana's ReLU linear-attention core on token-major (N, heads*head_dim) operands
+// (src/dit/sana.cpp:470-586). `state` receives the FP32 (S, z) blocks, heads x (d*d + d).
+void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
+                                   Tensor& state, Tensor& out, bool accumulate_state = false);
+
+}  // namespace bt
+
+namespace dit {
+
+struct RopeTables {
+    Tensor cos;  // (L, head_dim/2) FP32
+    Tensor sin;
+};
+RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const std::vector<int>& axes_dims_rope,
+                                   float theta = 10000.0f);
+
+// RoPE on Q and K, then full-bidirectional attention. The rotation is applied while Q and K are
+// loaded; Qr / Kr (the reference's scratch) are accepted and left untouched.
+void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin,
+                     int head_dim, int num_heads, Tensor& out, Tensor& Qr, Tensor& Kr);
+
+void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin,
+                          int head_dim, int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out,
+                          Tensor& Qr, Tensor& Kr, Tensor& Krep, Tensor& Vrep);
+
+// One segment of the Qwen-Image joint sequence (src/dit/qwenimage21_forward.cpp:650-676).
+struct Segment {
+    enum class Kind { Text, Image } kind;
+    int n_tokens;
+};
+// Block-causal attention over [prefix ; target] in ONE launch. Q holds `q_rows` rows starting at
+// joint position q_offset; keys are [k_prefix ; K] (k_prefix may be null / empty: prefill form).
+// `segments` describe the query rows in order: a Text run is causal, an Image block sees every key
+// up to its own end. Equals the reference's one-call-per-segment decomposition; with a single Image
+// segment covering all keys it is the cached form (qwenimage21_forward.cpp:599-649).
+void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix,
+                            const Tensor* v_prefix, const std::vector<Segment>& segments, int q_offset,
+                            int num_heads, const Tensor* cos_q, const Tensor* sin_q, Tensor& out);
+
+}  // namespace dit
+}  // namespace bdamd

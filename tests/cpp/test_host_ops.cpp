@@ -1,0 +1,193 @@
+// Parity test of the C++20 host operator layer, in the reference's test style: one executable,
+// a CHECK macro that counts failures (reference: tests/test_flux_blocks.cpp:38-44).
+//   test_host_ops --cpu   precondition / error-path checks that need no GPU
+//   test_host_ops         the GPU parity run against the CPU checker (liboracle.so, test-only)
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "attention_ops.h"
+
+extern "C" {
+int orc_torch_randn_f32(uint64_t seed, size_t n, float* out);
+void orc_round_bf16(float* x, size_t n);
+void orc_f32_to_bf16_bits(const float* x, size_t n, uint16_t* out);
+void orc_bf16_bits_to_f32(const uint16_t* x, size_t n, float* out);
+int orc_build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const int* axes, int n_axes, float theta,
+                                float* cos_out, float* sin_out);
+void orc_rope_apply(const float* x, const float* cs, const float* sn, int L, int H, int d, int split_half, int round_mode, float* out);
+void orc_sdpa(const float* q, const float* k, const float* v, int Lq, int Lk, int H, int d, double scale, const float* key_mask,
+              const int* row_lo, const int* row_hi, const uint8_t* dense_mask, const float* bias, int bias_q0, int bias_cols,
+              const int* rows, int n_rows, float* out, float* attn_avg, int n_threads);
+void orc_rows_causal(int Lq, int Lk, int q_offset, int window, int* row_lo, int* row_hi);
+void orc_rows_block_causal(int Lq, int Lk, int q_offset, const int* seg_q_end, const int* seg_k_end, const int* seg_causal,
+                           int n_seg, int* row_lo, int* row_hi);
+void orc_linear_attn_relu(const float* q, const float* k, const float* v, int N, int H, int d, float eps, float* out,
+                          float* S_out, float* z_out, int n_threads);
+}
+
+using namespace bdamd;
+
+static int g_failures = 0;
+#define CHECK(cond)                                                              \
+    do {                                                                         \
+        if (!(cond)) { std::printf("CHECK failed %s:%d: %s\n", __FILE__, __LINE__, #cond); ++g_failures; } \
+    } while (0)
+
+template <typename F>
+static bool throws_with(F&& f, const char* needle) {
+    try { f(); } catch (const std::runtime_error& e) { return std::strstr(e.what(), needle) != nullptr; }
+    return false;
+}
+
+static std::vector<float> randn_bf16(uint64_t seed, size_t n) {
+    std::vector<float> x(n < 16 ? 16 : n);
+    orc_torch_randn_f32(seed, x.size(), x.data());
+    x.resize(n);
+    orc_round_bf16(x.data(), n);
+    return x;
+}
+static Tensor upload_bf16(const std::vector<float>& x, int rows, int cols) {
+    std::vector<uint16_t> bits(x.size());
+    orc_f32_to_bf16_bits(x.data(), x.size(), bits.data());
+    return Tensor::from_host(bits.data(), rows, cols, Dtype::BF16);
+}
+static std::vector<float> download_bf16(const Tensor& t) {
+    const std::vector<uint8_t> raw = t.to_host_bytes();
+    std::vector<float> out(t.size());
+    orc_bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(raw.data()), out.size(), out.data());
+    return out;
+}
+struct Err { double rel_l2, max_abs; };
+static Err compare(const std::vector<float>& ref, const std::vector<float>& got) {
+    double num = 0, den = 0, mx = 0;
+    for (size_t i = 0; i < ref.size(); ++i) {
+        const double d = static_cast<double>(ref[i]) - got[i];
+        num += d * d; den += static_cast<double>(ref[i]) * ref[i];
+        if (std::fabs(d) > mx) mx = std::fabs(d);
+    }
+    return {std::sqrt(num / (den + 1e-300)), mx};
+}
+// bf16 bar of the port: rel-L2 <= 5e-3, max-abs <= 2e-2
+static bool within_bf16(const Err& e) { return e.rel_l2 <= 5e-3 && e.max_abs <= 2e-2; }
+
+static void cpu_checks() {
+    float dummy[64 * 64] = {0};
+    Tensor q = Tensor::view(Device::CPU, dummy, 8, 256, Dtype::BF16);
+    Tensor out;
+    CHECK(throws_with([&] { bt::flash_attention_forward(q, q, q, nullptr, 2, false, out); }, "flash_attention_forward: tensor is on the CPU"));
+    Tensor g = Tensor::view(Device::GPU, dummy, 8, 256, Dtype::BF16);   // never dereferenced: validation fails first
+    CHECK(throws_with([&] { bt::flash_attention_forward(g, g, g, nullptr, 3, false, out); }, "D must equal head_dim * num_heads"));
+    Tensor k = Tensor::view(Device::GPU, dummy, 8, 128, Dtype::BF16);
+    CHECK(throws_with([&] { bt::flash_attention_forward(g, k, g, nullptr, 2, false, out); }, "K and V must be"));
+    Tensor f = Tensor::view(Device::GPU, dummy, 8, 256, Dtype::FP32);
+    CHECK(throws_with([&] { bt::flash_attention_forward(f, f, f, nullptr, 2, false, out); }, "dtype must be FP16 or BF16"));
+    CHECK(throws_with([&] { bt::flash_attention_windowed_forward(g, g, g, nullptr, 2, -1, out); }, "window must be >= 0"));
+    CHECK(throws_with([&] { dit::build_axial_rope_tables(4, 2, 2, 32, {8, 8, 8}); }, "must sum to head_dim"));
+    CHECK(throws_with([&] { dit::build_axial_rope_tables(4, 2, 2, 31, {15, 8, 8}); }, "head_dim must be even"));
+    Tensor Qr, Kr;
+    CHECK(throws_with([&] { dit::joint_attention(g, k, g, f, f, 128, 2, out, Qr, Kr); }, "Q/K/V must share shape"));
+    CHECK(throws_with([&] { g.row_view(4, 8); }, "rows out of range"));
+    Tensor v = g.row_view(2, 4);
+    CHECK(v.rows == 4 && v.data == reinterpret_cast<char*>(dummy) + 2 * 256 * 2);
+}
+
+static void gpu_checks() {
+    const int H = 2, d = 128, txt = 19, hp = 6, wp = 7, L = txt + hp * wp, D = H * d;
+    const std::vector<float> q = randn_bf16(7001, static_cast<size_t>(L) * D), k = randn_bf16(7002, static_cast<size_t>(L) * D),
+                             v = randn_bf16(7003, static_cast<size_t>(L) * D);
+    Tensor Q = upload_bf16(q, L, D), K = upload_bf16(k, L, D), V = upload_bf16(v, L, D);
+
+    {   // joint_attention: fused RoPE == checker's explicit RoPE (rounded to bf16) + exact attention
+        const std::vector<int> axes = {16, 56, 56};
+        dit::RopeTables tabs = dit::build_axial_rope_tables(txt, hp, wp, d, axes);
+        std::vector<float> oc(static_cast<size_t>(L) * d / 2), os(oc.size());
+        orc_build_axial_rope_tables(txt, hp, wp, d, axes.data(), 3, 10000.0f, oc.data(), os.data());
+        const std::vector<uint8_t> tc = tabs.cos.to_host_bytes();
+        CHECK(std::memcmp(tc.data(), oc.data(), tc.size()) == 0);      // same table builder arithmetic
+        Tensor out, Qr, Kr;
+        dit::joint_attention(Q, K, V, tabs.cos, tabs.sin, d, H, out, Qr, Kr);
+        std::vector<float> qr(q.size()), kr(k.size()), ref(q.size());
+        orc_rope_apply(q.data(), oc.data(), os.data(), L, H, d, 0, 1, qr.data());
+        orc_rope_apply(k.data(), oc.data(), os.data(), L, H, d, 0, 1, kr.data());
+        orc_sdpa(qr.data(), kr.data(), v.data(), L, L, H, d, -1.0, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr, 0,
+                 ref.data(), nullptr, 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("joint_attention       rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        // determinism: bit-exact across two calls (reference: tests/test_flux_blocks.cpp:241-247)
+        Tensor out2;
+        dit::joint_attention(Q, K, V, tabs.cos, tabs.sin, d, H, out2, Qr, Kr);
+        CHECK(out.to_host_bytes() == out2.to_host_bytes());
+        // stand-alone rope_apply + flash == fused
+        Tensor Qrot, Krot, out3;
+        bt::rope_apply(Q, tabs.cos, tabs.sin, d, H, Qrot);
+        bt::rope_apply(K, tabs.cos, tabs.sin, d, H, Krot);
+        bt::flash_attention_forward(Qrot, Krot, V, nullptr, H, false, out3);
+        CHECK(out.to_host_bytes() == out3.to_host_bytes());
+    }
+    {   // windowed causal vs checker
+        Tensor Qs = Q.row_view(10, 30), out;
+        bt::flash_attention_windowed_forward(Qs, K, V, nullptr, H, 0, out);
+        std::vector<int> lo(30), hi(30);
+        orc_rows_causal(30, L, L - 30, 0, lo.data(), hi.data());
+        std::vector<float> ref(static_cast<size_t>(30) * D);
+        orc_sdpa(q.data() + static_cast<size_t>(10) * D, k.data(), v.data(), 30, L, H, d, -1.0, nullptr, lo.data(), hi.data(), nullptr,
+                 nullptr, 0, 0, nullptr, 0, ref.data(), nullptr, 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("windowed causal       rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+    }
+    {   // block-causal in one launch == the reference's one call per segment, and cached == prefill rows
+        const int prefix = 21;                       // text prefix kept as "cache"
+        std::vector<dit::Segment> segs = {{dit::Segment::Kind::Text, prefix}, {dit::Segment::Kind::Image, L - prefix}};
+        Tensor out;
+        dit::block_causal_attention(Q, K, V, nullptr, nullptr, segs, 0, H, nullptr, nullptr, out);
+        Tensor o_text, o_img;
+        bt::flash_attention_windowed_forward(Q.row_view(0, prefix), K.row_view(0, prefix), V.row_view(0, prefix), nullptr, H, 0, o_text);
+        bt::flash_attention_forward(Q.row_view(prefix, L - prefix), K, V, nullptr, H, false, o_img);
+        const std::vector<uint8_t> all = out.to_host_bytes(), t = o_text.to_host_bytes(), im = o_img.to_host_bytes();
+        CHECK(std::memcmp(all.data(), t.data(), t.size()) == 0);
+        CHECK(std::memcmp(all.data() + t.size(), im.data(), im.size()) == 0);
+        // cached form: prefix K/V from a separate buffer, target rows only
+        Tensor kp = K.row_view(0, prefix), vp = V.row_view(0, prefix), o_cached;
+        dit::block_causal_attention(Q.row_view(prefix, L - prefix), K.row_view(prefix, L - prefix), V.row_view(prefix, L - prefix), &kp, &vp,
+                                    {{dit::Segment::Kind::Image, L - prefix}}, prefix, H, nullptr, nullptr, o_cached);
+        CHECK(o_cached.to_host_bytes() == im);
+        std::vector<int> sq = {prefix, L}, sk = {prefix, L}, sc = {1, 0}, lo(L), hi(L);
+        orc_rows_block_causal(L, L, 0, sq.data(), sk.data(), sc.data(), 2, lo.data(), hi.data());
+        std::vector<float> ref(q.size());
+        orc_sdpa(q.data(), k.data(), v.data(), L, L, H, d, -1.0, nullptr, lo.data(), hi.data(), nullptr, nullptr, 0, 0, nullptr, 0, ref.data(),
+                 nullptr, 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("block-causal          rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+    }
+    {   // ReLU linear attention, 70 x 32 (the reference's own head split) on a short sequence
+        const int Hl = 70, dl = 32, N = 96, Dl = Hl * dl;
+        const std::vector<float> ql = randn_bf16(7011, static_cast<size_t>(N) * Dl), kl = randn_bf16(7012, static_cast<size_t>(N) * Dl),
+                                 vl = randn_bf16(7013, static_cast<size_t>(N) * Dl);
+        Tensor Ql = upload_bf16(ql, N, Dl), Kl = upload_bf16(kl, N, Dl), Vl = upload_bf16(vl, N, Dl), state, out;
+        bt::linear_attention_relu_forward(Ql, Kl, Vl, Hl, 1e-15f, state, out);
+        std::vector<float> ref(ql.size());
+        orc_linear_attn_relu(ql.data(), kl.data(), vl.data(), N, Hl, dl, 1e-15f, ref.data(), nullptr, nullptr, 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("linear attention      rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        CHECK(state.rows == Hl && state.cols == dl * dl + dl);
+    }
+    {   // GPU-side error path: unsupported head_dim surfaces the C ABI's message
+        Tensor out;
+        CHECK(throws_with([&] { bt::flash_attention_forward(Q, K, V, nullptr, 8, false, out); }, "no kernel"));
+    }
+}
+
+int main(int argc, char** argv) {
+    const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
+    cpu_checks();
+    if (!cpu_only) gpu_checks();
+    if (g_failures == 0) std::printf("test_host_ops: OK\n");
+    return g_failures == 0 ? 0 : 1;
+}

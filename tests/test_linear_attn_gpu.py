@@ -1,0 +1,104 @@
+"""GPU parity of ReLU linear attention and stand-alone RoPE against the CPU checker (C ABI path)."""
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import assert_close, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("B,H,d,N", [(2, 20, 112, 256), (1, 70, 32, 200), (2, 3, 64, 333), (1, 2, 72, 1000),
+                                     (1, 2, 128, 130), (1, 1, 112, 1), (2, 2, 32, 63)])
+def test_linear_attention_parity(oracle, B, H, d, N):
+    dtype = "bf16"
+    q = randn(5011, (B, N, H * d), dtype); k = randn(5012, (B, N, H * d), dtype); v = randn(5013, (B, N, H * d), dtype)
+    ws = torch.empty(B * H * (d * d + d), dtype=torch.float32, device="cuda")
+    out = bd.linear_attention_relu_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, workspace=ws)
+    wsn = to_np(ws).reshape(B, H, d * d + d)
+    for b in range(B):
+        ref, S, z = oracle.linear_attn_relu(q[b], k[b], v[b], H, return_state=True)
+        assert_close(ref, to_np(out[b]), dtype, f"out b={b}")
+        # the FP32 state is what the reference captures at its identity seam (src/dit/sana.cpp:489-506)
+        Sg = wsn[b, :, :d * d].reshape(H, d, d); zg = wsn[b, :, d * d:]
+        assert np.max(np.abs(Sg - S)) <= 1e-4 * max(1.0, np.max(np.abs(S)))
+        assert np.max(np.abs(zg - z)) <= 1e-4 * max(1.0, np.max(np.abs(z)))
+
+
+def test_linear_attention_state_injection(oracle):
+    """accumulate_state adds this call's (S, z) to the workspace: attending over [anchor ; own] tokens
+    (the reference's inject form, src/dit/sana.cpp:498-505 with weight 1)."""
+    dtype, H, d, N = "bf16", 2, 112, 192
+    q = randn(5021, (N, H * d), dtype); k = randn(5022, (N, H * d), dtype); v = randn(5023, (N, H * d), dtype)
+    ka = randn(5024, (N, H * d), dtype); va = randn(5025, (N, H * d), dtype)
+    ws = torch.empty(H * (d * d + d), dtype=torch.float32, device="cuda")
+    bd.linear_attention_relu_forward(to_dev(q, dtype), to_dev(ka, dtype), to_dev(va, dtype), H, workspace=ws)
+    out = bd.linear_attention_relu_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, workspace=ws,
+                                           accumulate_state=True)
+    # reference: numerator and denominator over the concatenated keys, same queries
+    _, S1, z1 = oracle.linear_attn_relu(q, ka, va, H, return_state=True)
+    _, S2, z2 = oracle.linear_attn_relu(q, k, v, H, return_state=True)
+    S, z = S1.astype(np.float64) + S2, z1.astype(np.float64) + z2
+    qr = np.maximum(q, 0).reshape(N, H, d).astype(np.float64)
+    num = np.einsum("hij,nhj->nhi", S, qr); den = np.einsum("hj,nhj->nh", z, qr)
+    ref = (num / (den[..., None] + 1e-15)).reshape(N, H * d)
+    assert_close(ref, to_np(out), dtype)
+
+
+def test_linear_attention_zero_denominator():
+    dtype, H, d, N = "bf16", 1, 32, 64
+    q = -torch.ones((N, H * d), dtype=torch.bfloat16, device="cuda")
+    kv = torch.ones((N, H * d), dtype=torch.bfloat16, device="cuda")
+    out = bd.linear_attention_relu_forward(q, kv, kv, H)
+    assert not out.float().abs().max().item()
+
+
+def test_linear_attention_errors():
+    x = torch.zeros((64, 96), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="no kernel"):
+        bd.linear_attention_relu_forward(x, x, x, 2)                       # head_dim 48
+    with pytest.raises(RuntimeError, match="no kernel"):
+        bd.linear_attention_relu_forward(x.half(), x.half(), x.half(), 3)  # fp16 overflows S
+    with pytest.raises(RuntimeError, match="workspace"):
+        bd.linear_attention_relu_forward(x, x, x, 3, workspace=torch.zeros(8, device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("split_half", [False, True])
+@pytest.mark.parametrize("H,d,L", [(3, 128, 77), (2, 40, 130), (1, 72, 5)])
+def test_rope_apply(oracle, dtype, split_half, H, d, L):
+    x = randn(6001, (L, H * d), dtype)
+    rng = np.random.default_rng(3)
+    ang = rng.uniform(-3, 3, (L, d // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    out = bd.rope_apply(to_dev(x, dtype), torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), d, H,
+                        split_half=split_half)
+    ref = oracle.rope_apply(x, cos, sin, H, d, split_half=split_half)
+    got = to_np(out)
+    # one rounding to the storage dtype: half an ulp of the largest value
+    ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1.0)) <= ulp
+    # rotations preserve each pair's norm
+    gv, xv = got.reshape(L, H, d), x.reshape(L, H, d)
+    idx = [(p, p + d // 2) for p in range(d // 2)] if split_half else [(2 * p, 2 * p + 1) for p in range(d // 2)]
+    for i0, i1 in idx[:4]:
+        n0 = np.hypot(xv[..., i0], xv[..., i1]); n1 = np.hypot(gv[..., i0], gv[..., i1])
+        assert np.max(np.abs(n0 - n1)) <= 4 * ulp * max(1.0, n0.max())
+
+
+def test_rope_apply_perhead_and_inplace(oracle):
+    dtype, H, d, L = "bf16", 3, 64, 50
+    x = randn(6002, (L, H * d), dtype)
+    rng = np.random.default_rng(4)
+    ang = rng.uniform(-3, 3, (L * H, d // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    dx = to_dev(x, dtype)
+    out = bd.rope_apply_perhead(dx, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), d, H)
+    # per-head tables: row r*H + h rotates head h of token r (src/triposplat/flow_model.cpp:374)
+    ref = np.empty_like(x)
+    for h in range(H):
+        ref[:, h * d:(h + 1) * d] = oracle.rope_apply(x[:, h * d:(h + 1) * d].copy(), cos[h::H].copy(), sin[h::H].copy(), 1, d)
+    assert np.max(np.abs(to_np(out) - ref)) <= 2.0 ** -8 * max(1.0, np.abs(ref).max())
+    bd.rope_apply_perhead(dx, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda(), d, H, out=dx)
+    assert torch.equal(dx, out)
