@@ -16,10 +16,11 @@ from .ops import (  # noqa: F401
     rope_apply,
     rope_apply_perhead,
     sdpa_forward,
+    set_sdpa_kernel_choice,
 )
 
 __all__ = [
     "SdpaMask", "build_axial_rope_tables", "device_info", "flash_attention_forward",
     "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
-    "linear_attention_relu_forward", "rope_apply", "rope_apply_perhead", "sdpa_forward",
+    "linear_attention_relu_forward", "rope_apply", "rope_apply_perhead", "sdpa_forward", "set_sdpa_kernel_choice",
 ]

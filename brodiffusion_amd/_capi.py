@@ -20,7 +20,7 @@ MI_MAX_SEGMENTS = 32
 EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
-    "mi_sdpa_forward", "mi_sdpa_supported", "mi_rope_apply",
+    "mi_sdpa_forward", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
 ]
 
@@ -105,6 +105,7 @@ def lib() -> C.CDLL:
         L.mi_memset_async.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_void_p]
         L.mi_sdpa_forward.argtypes = [C.POINTER(MiSdpaArgs)]
         L.mi_sdpa_supported.argtypes = [C.c_int32, C.c_int32]
+        L.mi_sdpa_set_kernel_choice.argtypes = [C.c_int32]
         L.mi_rope_apply.argtypes = [C.POINTER(MiRopeArgs)]
         L.mi_linear_attn_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         L.mi_linear_attn_workspace_bytes.restype = C.c_size_t

@@ -22,6 +22,9 @@ FLAGS = [
     "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
     # packed-FP32 VALU forms are switched off for every kernel of this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # no NaN is ever produced on these paths (masked scores are -inf, guarded before subtraction), so
+    # max / compare need no signalling-NaN quieting moves; infinities keep their meaning
+    "-fno-honor-nans",
     "-Wall", "-Wno-unused-value", "-Wno-unknown-pragmas",
 ]
 

@@ -10,6 +10,7 @@ namespace mi {
 namespace {
 thread_local char g_err[512] = "";
 thread_local hipStream_t g_stream = nullptr;
+thread_local int g_kernel_choice = 0;
 }  // namespace
 
 int fail(const char* fmt, ...) {
@@ -21,6 +22,17 @@ int fail(const char* fmt, ...) {
 }
 void clear_error() { g_err[0] = '\0'; }
 hipStream_t resolve_stream(void* s) { return s ? static_cast<hipStream_t>(s) : g_stream; }
+int sdpa_kernel_choice() { return g_kernel_choice; }
+int device_cu_count() {
+    static thread_local int n = 0;
+    if (n == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+    }
+    return n;
+}
 
 namespace {
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -82,6 +94,13 @@ int mi_memcpy_d2d_async(void* dst, const void* src, size_t bytes, void* stream) 
 }
 int mi_memset_async(void* dst, int value, size_t bytes, void* stream) {
     mi::clear_error(); MI_HIP_CHECK(hipMemsetAsync(dst, value, bytes, mi::resolve_stream(stream))); return 0;
+}
+
+int mi_sdpa_set_kernel_choice(int32_t choice) {
+    mi::clear_error();
+    if (choice < 0 || choice > 2) return fail("mi_sdpa_set_kernel_choice: 0 (auto), 1 (128-row tiles) or 2 (256-row ping-pong)");
+    mi::g_kernel_choice = choice;
+    return 0;
 }
 
 int mi_sdpa_supported(int32_t dtype, int32_t head_dim) { return mi::sdpa_supported(dtype, head_dim) ? 1 : 0; }
@@ -163,10 +182,8 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
     for (const void* t : tabs)
         if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
     p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
-    p.n_q_tiles = (a->q_len + 127) / 128;
-    const long nb = static_cast<long>(a->batch) * a->num_heads * p.n_q_tiles;
+    const long nb = static_cast<long>(a->batch) * a->num_heads * ((a->q_len + 127) / 128);
     if (nb > 0x3fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
-    p.n_blocks = static_cast<int>(nb);
     return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
 }
 

@@ -13,6 +13,8 @@ namespace mi {
 int fail(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 void clear_error();
 hipStream_t resolve_stream(void* s);
+// Compute units of the current device (cached per thread; 256 if the query fails).
+int device_cu_count();
 
 #define MI_HIP_CHECK(expr)                                                          \
     do {                                                                            \
@@ -44,6 +46,9 @@ struct SdpaDev {
 // (stand-alone pass, Q load, K tile load) rounds identically: (a + ib)(c + is).
 __device__ __forceinline__ float rope_re(float a, float b, float c, float s) { return __builtin_fmaf(a, c, -(b * s)); }
 __device__ __forceinline__ float rope_im(float a, float b, float c, float s) { return __builtin_fmaf(a, s, b * c); }
+
+// 0 = pick by problem size, 1 = 128-row kernel, 2 = 256-row ping-pong kernel (mi_sdpa_set_kernel_choice).
+int sdpa_kernel_choice();
 
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 bool sdpa_supported(int dtype, int head_dim);

@@ -336,16 +336,6 @@ bool lin_supported(int dtype, int d) {
     return d == 32 || d == 64 || d == 72 || d == 112 || d == 128;
 }
 
-int cu_count() {
-    static thread_local int n = 0;
-    if (n == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-    }
-    return n;
-}
-
 }  // namespace
 }  // namespace mi
 
@@ -393,7 +383,7 @@ int mi_linear_attn_relu_forward(const mi_linear_attn_args* a) {
     p.ws = static_cast<float*>(a->workspace);
     p.tokens_per_group = 0;
     hipStream_t st = mi::resolve_stream(a->stream);
-    const int n_cu = mi::cu_count();
+    const int n_cu = mi::device_cu_count();
     return mi::launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, n_cu, st);
 }
 

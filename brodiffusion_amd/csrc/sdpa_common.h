@@ -1,0 +1,282 @@
+// Building blocks shared by the softmax-attention kernels for gfx950: MFMA wrappers, the LDS tile
+// geometry for a head dimension, the per-row visibility interval, Q fragment loading with RoPE, and
+// the three per-tile stages (S^T = K Q^T, online softmax, O^T += V^T P^T).
+//
+// Register layouts (v_mfma_f32_32x32x16, wave64; lq = lane % 32, lh = lane / 32):
+//   A operand: lane holds row lq, 8 consecutive contraction elements starting at 8*lh
+//   B operand: lane holds column lq, the same 8 contraction elements
+//   C/D:       lane holds column lq; acc[4b + i] is row 8b + 4*lh + i
+// The score tile is computed transposed (rows = keys, columns = queries), so a lane holds scores of
+// ONE query and the accumulator layout of P^T is directly the B operand of O^T += V^T P^T.
+#pragma once
+#include "internal.h"
+
+namespace mi {
+namespace sdpa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBN = 64;  // key rows per LDS tile
+constexpr float kNegInf = -__builtin_huge_valf();
+constexpr float kLazyLog2 = 8.0f;  // raise the softmax reference only when a tile exceeds it by 2^8
+
+template <typename T> struct Mma;
+template <> struct Mma<__bf16> {
+    using v8 = bf16x8;
+    static __device__ __forceinline__ f32x16 run(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mma<_Float16> {
+    using v8 = f16x8;
+    static __device__ __forceinline__ f32x16 run(v8 a, v8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// LDS geometry of one K/V tile for head dimension D.
+template <int D> struct HeadGeo {
+    static constexpr int DK = (D + 15) / 16 * 16;  // contraction extent of K Q^T (zero padded)
+    static constexpr int DV = (D + 31) / 32 * 32;  // output rows of V^T P^T
+    static constexpr int KC = DK / 16;
+    static constexpr int VB = DV / 32;
+    // K rows are read one row per lane with ds_read_b128: a stride of 16 * odd bytes puts 16
+    // consecutive rows on distinct banks.
+    static constexpr int K_STRIDE = DK * 2 + 16;
+    // V is read by ds_read_b64_tr_b16: 4 consecutive rows x 64 contiguous bytes per 32 lanes; a
+    // stride that is 64 mod 128 bytes puts those 4 rows on distinct bank groups.
+    static constexpr int V_STRIDE = ((DV * 2 + 63) / 128) * 128 + 64;
+    static constexpr int K_BYTES = kBN * K_STRIDE;
+    static constexpr int V_BYTES = kBN * V_STRIDE;
+    static constexpr int O_STRIDE = DK * 2 + 16;
+    static constexpr int CPR = D / 8;  // 16-byte chunks per row that hold data
+    static constexpr int NCH = kBN * CPR;
+};
+
+// v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 lanes of
+// its second; fed the same value twice it leaves (own, partner) in the lower half and
+// (partner, own) in the upper half, so max / sum of the two results is the reduction over lanes
+// l and l^32. (The results are copied to scalars before the bit cast: a bit cast applied to a
+// vector element expression reads element 0 for every index with this compiler.)
+__device__ __forceinline__ float exchange_max(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    const i32x2 r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    const int r0 = r[0], r1 = r[1];
+    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
+}
+__device__ __forceinline__ float exchange_sum(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    const i32x2 r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    const int r0 = r[0], r1 = r[1];
+    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+// Rotate the 4 adjacent pairs held in one 16-byte chunk, FP32 arithmetic, one rounding back to T.
+template <typename T>
+__device__ __forceinline__ u32x4 rope_chunk(u32x4 raw, f32x4 c, f32x4 s) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    t8 x = __builtin_bit_cast(t8, raw);
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const float a = static_cast<float>(x[2 * p]);
+        const float b = static_cast<float>(x[2 * p + 1]);
+        x[2 * p] = static_cast<T>(rope_re(a, b, c[p], s[p]));
+        x[2 * p + 1] = static_cast<T>(rope_im(a, b, c[p], s[p]));
+    }
+    return __builtin_bit_cast(u32x4, x);
+}
+
+// Visible key interval [lo, hi) of query row `qrow` (empty -> lo = hi = 0).
+__device__ __forceinline__ void row_interval(const SdpaDev& p, int b, int qrow, bool qvalid, int& lo, int& hi) {
+    lo = 0;
+    hi = p.Lk;
+    if (p.kv_valid_len) hi = min(hi, p.kv_valid_len[b]);
+    if (p.mask_mode == MI_MASK_CAUSAL) {
+        const int pos1 = p.q_offset + qrow + 1;
+        hi = min(hi, pos1);
+        if (p.window > 0) lo = max(0, pos1 - p.window);
+    } else if (p.mask_mode == MI_MASK_BLOCK_CAUSAL) {
+        // static indices only: the segment table stays in scalar registers
+        int sk = p.seg_k_end[0], sc = p.seg_causal[0];
+#pragma unroll
+        for (int s = 1; s < MI_MAX_SEGMENTS; ++s)
+            if (s < p.n_seg && qrow >= p.seg_q_end[s - 1]) { sk = p.seg_k_end[s]; sc = p.seg_causal[s]; }
+        hi = min(hi, sk);
+        if (sc) hi = min(hi, p.q_offset + qrow + 1);
+    }
+    if (!qvalid || hi <= lo) { lo = 0; hi = 0; }
+}
+
+// Extents of the 64 rows of a wavefront (each row is held by lanes l and l^32).
+struct WaveExtent { int lo_min, lo_max, hi_min, hi_max; };
+__device__ __forceinline__ WaveExtent wave_extent(int lo, int hi) {
+    WaveExtent w{hi > lo ? lo : 0x7fffffff, lo, hi, hi};
+#pragma unroll
+    for (int off = 16; off >= 1; off >>= 1) {
+        w.lo_min = min(w.lo_min, __shfl_xor(w.lo_min, off));
+        w.lo_max = max(w.lo_max, __shfl_xor(w.lo_max, off));
+        w.hi_min = min(w.hi_min, __shfl_xor(w.hi_min, off));
+        w.hi_max = max(w.hi_max, __shfl_xor(w.hi_max, off));
+    }
+    return w;
+}
+
+// Q fragments (B operand of K Q^T) of this lane's query row, RoPE applied on the way in.
+template <typename T, int D>
+__device__ __forceinline__ void load_q_frags(typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], const SdpaDev& p, const T* q_base,
+                                             int qrow, bool qvalid, int lh) {
+    using V8 = typename Mma<T>::v8;
+#pragma unroll
+    for (int c = 0; c < HeadGeo<D>::KC; ++c) {
+        const int d0 = 16 * c + 8 * lh;
+        u32x4 raw = u32x4{0, 0, 0, 0};
+        if (qvalid && d0 < D) {
+            raw = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + d0);
+            if (p.cos_q) {
+                const f32x4 cs = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
+                const f32x4 sn = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
+                raw = rope_chunk<T>(raw, cs, sn);
+            }
+        }
+        qf[c] = __builtin_bit_cast(V8, raw);
+    }
+}
+
+// S^T = K Q^T for one 64-key tile: 2 blocks of 32 keys.
+template <typename T, int D>
+__device__ __forceinline__ void qk_tile(const unsigned char* Ks, const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], int lq, int lh,
+                                        f32x16 (&sacc)[2]) {
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) {
+            const u32x4 a = *reinterpret_cast<const u32x4*>(Ks + (32 * kb + lq) * G::K_STRIDE + (16 * c + 8 * lh) * 2);
+            if (c == 0) {
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], zero);
+            } else {
+                sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], sacc[kb]);
+            }
+        }
+    }
+}
+
+// Online-softmax state of one lane (one query row, shared with lane l^32).
+// m is the reference the exponentials are taken against; it is raised only when a tile's maximum
+// exceeds it by more than 2^kLazyLog2, so most tiles skip the rescale of l and O. The result does
+// not depend on which reference is used.
+struct SoftmaxState {
+    float m = kNegInf;  // raw-score units
+    float mc = 0.f;     // m * scale_log2 (0 while m is -inf)
+    float l = 0.f;      // this lane's share of the denominator
+};
+
+// Masks (if MASKED), exponentiates and packs one score tile into the B operands of the PV product.
+template <typename T, int D, bool MASKED>
+__device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
+                                             SoftmaxState& st, float cl2, float lazy_raw, int j0, int lo, int hi, int lh,
+                                             const float* key_mask, int Lk) {
+    if constexpr (MASKED) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+                const int kbase = j0 + 32 * kb + 8 * bb + 4 * lh;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int key = kbase + i;
+                    bool vis = key >= lo && key < hi;
+                    if (key_mask) vis = vis && (key < Lk) && key_mask[key < Lk ? key : 0] != 0.f;
+                    if (!vis) sacc[kb][4 * bb + i] = kNegInf;
+                }
+            }
+    }
+    float mloc = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+    for (int e = 1; e < 16; ++e) mloc = fmaxf(mloc, fmaxf(sacc[0][e], sacc[1][e]));
+    mloc = exchange_max(mloc);
+    if (__any(mloc > st.m + lazy_raw)) {
+        const float m_new = fmaxf(st.m, mloc);
+        const float mc_new = (m_new == kNegInf) ? 0.f : m_new * cl2;
+        const float alpha = __builtin_amdgcn_exp2f(st.m * cl2 - mc_new);  // 1 where unchanged, 0 from -inf
+        st.m = m_new;
+        st.mc = mc_new;
+        st.l *= alpha;
+#pragma unroll
+        for (int vb = 0; vb < HeadGeo<D>::VB; ++vb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[vb][e] *= alpha;
+    }
+    float lsum0 = 0.f, lsum1 = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[0][e], cl2, -st.mc));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[1][e], cl2, -st.mc));
+        sacc[0][e] = p0;
+        sacc[1][e] = p1;
+        lsum0 += p0;
+        lsum1 += p1;
+    }
+    st.l += lsum0 + lsum1;
+    // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
+}
+
+// O^T += V^T P^T for one 64-key tile. V^T fragments come from the row-major V tile through LDS
+// transpose reads: within 16 lanes, lane j supplies the address of 4 consecutive head-dim elements
+// of key row j/4, and lane i receives 4 consecutive keys of head-dim column i.
+template <typename T, int D>
+__device__ __forceinline__ void pv_tile(const unsigned char* Vs, const typename Mma<T>::v8 (&pf)[4], int lane,
+                                        f32x16 (&oacc)[HeadGeo<D>::VB]) {
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    const int lh = lane >> 5;
+    const int trow = (lane & 15) >> 2;
+    const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) {
+#pragma unroll
+        for (int vb = 0; vb < G::VB; ++vb) {
+            const unsigned char* vptr = Vs + (16 * c4 + 4 * lh + trow) * G::V_STRIDE + (32 * vb + tcol) * 2;
+            const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
+            const s16x4 v_hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::V_STRIDE));
+            const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            oacc[vb] = Mma<T>::run(__builtin_bit_cast(V8, a), pf[c4], oacc[vb]);
+        }
+    }
+}
+
+// Normalised output rows of one wavefront into the LDS staging area (row-major, O_STRIDE).
+template <typename T, int D>
+__device__ __forceinline__ void stage_output(unsigned char* Os, int row, int lh, const f32x16 (&oacc)[HeadGeo<D>::VB], float inv) {
+    using G = HeadGeo<D>;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int vb = 0; vb < G::VB; ++vb)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+            const int d0 = 32 * vb + 8 * bb + 4 * lh;
+            if (d0 < D) {
+                t4 ov;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ov[i] = static_cast<T>(oacc[vb][4 * bb + i] * inv);
+                *reinterpret_cast<t4*>(Os + row * G::O_STRIDE + d0 * 2) = ov;
+            }
+        }
+}
+
+}  // namespace sdpa
+}  // namespace mi

@@ -1,129 +1,179 @@
-// Flash-style softmax attention forward for gfx950 (MI355X), hand-written.
+// Flash-style softmax attention forward for gfx950 (MI355X), hand-written. Two kernels share the
+// building blocks of sdpa_common.h:
 //
-// One work group = 4 wavefronts = 128 query rows of one (batch, head); each wavefront
-// owns 32 query rows for the whole key loop. Key/value tiles of 64 rows are staged in
-// LDS and shared by the 4 wavefronts.
+//   sdpa_fwd_pp_kernel   8 wavefronts = 256 query rows per work group, 2 wavefronts per SIMD. The two
+//                        wavefronts of a SIMD run half a tile apart: while one issues the MFMAs of
+//                        O += V^T P (tile t) and S = K Q^T (tile t+1), the other does the softmax of
+//                        its own tile on the VALU, so the matrix and vector pipes of the SIMD are busy
+//                        at the same time. The phase shift is set up once by one extra barrier for the
+//                        second group and kept by the two work-group barriers of every iteration.
+//   sdpa_fwd_kernel      4 wavefronts = 128 query rows per work group, 2 work groups per CU; used when
+//                        the problem has too few 256-row tiles to fill the chip.
 //
-// The score tile is computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16:
-//   A = K tile from LDS   (lane l: key row l%32, 8 contiguous head-dim elements at 8*(l/32))
-//   B = Q^T in registers  (lane l: query l%32,   same 8 head-dim elements)
-//   C = S^T               (lane l: query l%32;   acc[4b+i] is key 8b + 4*(l/32) + i)
-// so every lane holds scores of ONE query: the online-softmax row statistics need one
-// exchange between lanes l and l^32 (v_permlane32_swap) and no LDS. The accumulator layout
-// of P^T is already the B-operand layout of the second product O^T = V^T P^T (keys of a
-// 16-key chunk in the order acc[8c'..8c'+7]), so P never leaves registers. V^T comes from
-// the row-major V tile through ds_read_b64_tr_b16 (LDS transpose read), which hands each
-// lane 4 consecutive keys of one head-dim column.
-//
-// Not in HBM: scores, probabilities, rotated Q/K (RoPE is applied as Q and K are loaded),
-// the [prefix ; fresh] K/V concatenation (two source pointers), any mask tensor (per-row
-// visible-key intervals; key tiles outside every row's interval are skipped).
-#include "internal.h"
+// Key/value tiles of 64 rows are staged in LDS (double buffered, loaded one tile ahead through
+// registers). Not in HBM: scores, probabilities, rotated Q/K (RoPE is applied as Q and K are loaded),
+// the [prefix ; fresh] K/V concatenation (two source pointers), any mask tensor (per-row visible-key
+// intervals; key tiles outside every row's interval are skipped).
+#include "sdpa_common.h"
 
 namespace mi {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef int i32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+using namespace sdpa;
 
-constexpr int kBM = 128;      // query rows per work group
-constexpr int kBN = 64;       // key rows per LDS tile
-constexpr int kThreads = 256;
-constexpr float kNegInf = -__builtin_huge_valf();
-
-template <typename T> struct Mma;
-template <> struct Mma<__bf16> {
-    using v8 = bf16x8;
-    static __device__ __forceinline__ f32x16 run(v8 a, v8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct Mma<_Float16> {
-    using v8 = f16x8;
-    static __device__ __forceinline__ f32x16 run(v8 a, v8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-
-template <int D> struct Geo {
-    static constexpr int DK = (D + 15) / 16 * 16;  // contraction extent of K Q^T (zero padded)
-    static constexpr int DV = (D + 31) / 32 * 32;  // output rows of V^T P^T
-    static constexpr int KC = DK / 16;
-    static constexpr int VB = DV / 32;
-    // K rows are read one row per lane with ds_read_b128: a stride of 16 * odd bytes puts 16
-    // consecutive rows on distinct banks.
-    static constexpr int K_STRIDE = DK * 2 + 16;
-    // V is read by ds_read_b64_tr_b16: 4 consecutive rows x 64 contiguous bytes per 32 lanes; a
-    // stride that is 64 mod 128 bytes puts those 4 rows on distinct bank groups.
-    static constexpr int V_STRIDE = ((DV * 2 + 63) / 128) * 128 + 64;
-    static constexpr int K_BYTES = kBN * K_STRIDE;
-    static constexpr int V_BYTES = kBN * V_STRIDE;
-    static constexpr int M_BYTES = kBN * 4;
-    static constexpr int O_STRIDE = DK * 2 + 16;
-    static constexpr int O_BYTES = kBM * O_STRIDE;
-    static constexpr int KV_BYTES = K_BYTES + V_BYTES + M_BYTES;
-    static constexpr int LDS_BYTES = (KV_BYTES > O_BYTES ? KV_BYTES : O_BYTES);
-    static constexpr int CPR = D / 8;  // 16-byte chunks per row that hold data
-    static constexpr int NCH = kBN * CPR;
-    static constexpr int NLD = (NCH + kThreads - 1) / kThreads;
-};
-
-// v_permlane32_swap exchanges the upper 32 lanes of its first operand with the lower 32 lanes of
-// its second; fed the same value twice it leaves (own, partner) in the lower half and
-// (partner, own) in the upper half, so max / sum of the two results is the reduction over lanes
-// l and l^32. (The results are copied to scalars before the bit cast: a bit cast applied to a
-// vector element expression reads element 0 for every index with this compiler.)
-__device__ __forceinline__ float exchange_max(float x) {
-    const int xi = __builtin_bit_cast(int, x);
-    const i32x2 r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
-    const int r0 = r[0], r1 = r[1];
-    return fmaxf(__builtin_bit_cast(float, r0), __builtin_bit_cast(float, r1));
-}
-__device__ __forceinline__ float exchange_sum(float x) {
-    const int xi = __builtin_bit_cast(int, x);
-    const i32x2 r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
-    const int r0 = r[0], r1 = r[1];
-    return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+// Work-group id -> logical tile. Hardware deals consecutive work-group ids round-robin over the 8
+// XCDs; undo that so each XCD (one L2) gets a contiguous run of logical tiles, i.e. query tiles that
+// share the same K/V. Returns -1 for the padding groups of the last round.
+__device__ __forceinline__ int logical_block(int n_blocks) {
+    const int chunk = (n_blocks + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    return logical < n_blocks ? logical : -1;
 }
 
-// Rotate the 4 adjacent pairs held in one 16-byte chunk: (x0, x1) -> (x0 c - x1 s, x0 s + x1 c),
-// FP32 arithmetic, one rounding back to T.
-template <typename T>
-__device__ __forceinline__ u32x4 rope_chunk(u32x4 raw, f32x4 c, f32x4 s) {
-    typedef T t8 __attribute__((ext_vector_type(8)));
-    t8 x = __builtin_bit_cast(t8, raw);
+// Cooperative K/V tile movement for a work group of NT threads: global -> registers -> LDS.
+// kreg / vreg hold this thread's 16-byte chunks of one K tile and one V tile (possibly different tiles).
+template <typename T, int D, int NT, bool ROPE_K>
+struct TileMover {
+    using G = HeadGeo<D>;
+    static constexpr int NLD = (G::NCH + NT - 1) / NT;
+    static constexpr bool EXACT = (G::NCH % NT) == 0;
+    const SdpaDev& p;
+    const T* k_base; const T* v_base; const T* kp_base; const T* vp_base;
+    int tid, kv_stop;
+    u32x4 kreg[NLD], vreg[NLD];
+
+    // which: 0 = K tile into kreg, 1 = V tile into vreg
+    template <int WHICH>
+    __device__ __forceinline__ void issue(int j0) {
+        u32x4 (&reg)[NLD] = WHICH == 0 ? kreg : vreg;
+        const T* fresh = WHICH == 0 ? k_base : v_base;
+        const T* pre = WHICH == 0 ? kp_base : vp_base;
+        const long f_rs = WHICH == 0 ? p.k_rs : p.v_rs;
+        const long p_rs = WHICH == 0 ? p.kp_rs : p.vp_rs;
+        const bool in_prefix = j0 + kBN <= p.Lp;
+        const bool in_fresh = j0 >= p.Lp;
+        if ((in_prefix || in_fresh) && j0 + kBN <= kv_stop) {
+            // whole tile from one buffer: uniform base pointer plus a fixed per-thread byte offset
+            const unsigned char* base = in_fresh ? reinterpret_cast<const unsigned char*>(fresh + static_cast<long>(j0 - p.Lp) * f_rs)
+                                                 : reinterpret_cast<const unsigned char*>(pre + static_cast<long>(j0) * p_rs);
+            const unsigned rsb = static_cast<unsigned>(in_fresh ? f_rs : p_rs) * 2u;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const float a = static_cast<float>(x[2 * p]);
-        const float b = static_cast<float>(x[2 * p + 1]);
-        x[2 * p] = static_cast<T>(rope_re(a, b, c[p], s[p]));
-        x[2 * p + 1] = static_cast<T>(rope_im(a, b, c[p], s[p]));
+            for (int i = 0; i < NLD; ++i) {
+                const int idx = tid + NT * i;
+                const int row = idx / G::CPR;
+                const int cc = idx - row * G::CPR;
+                if (EXACT || idx < G::NCH) reg[i] = *reinterpret_cast<const u32x4*>(base + (static_cast<unsigned>(row) * rsb + cc * 16u));
+            }
+        } else {
+            // tile straddles the prefix / fresh boundary or the end of the visible keys
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int idx = tid + NT * i;
+                const int row = idx / G::CPR;
+                const int cc = idx - row * G::CPR;
+                const int j = j0 + row;
+                reg[i] = u32x4{0, 0, 0, 0};
+                if ((EXACT || idx < G::NCH) && j < kv_stop) {
+                    const T* r = j < p.Lp ? pre + static_cast<long>(j) * p_rs : fresh + static_cast<long>(j - p.Lp) * f_rs;
+                    reg[i] = *reinterpret_cast<const u32x4*>(r + cc * 8);
+                }
+            }
+        }
     }
-    return __builtin_bit_cast(u32x4, x);
+    __device__ __forceinline__ void store_k(int j0, unsigned char* Ks) {
+        // The rotation tables are fetched here rather than with the tile: they are L2 hits shared by
+        // every head, and holding them across the MFMA section would cost 8 registers per chunk
+        // exactly where pressure peaks. Prefix rows are stored already rotated.
+        f32x4 creg[ROPE_K ? NLD : 1], sreg[ROPE_K ? NLD : 1];
+        if constexpr (ROPE_K) {
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int idx = tid + NT * i;
+                const int row = idx / G::CPR;
+                const int cc = idx - row * G::CPR;
+                const int j = j0 + row;
+                creg[i] = f32x4{1.f, 1.f, 1.f, 1.f};
+                sreg[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if ((EXACT || idx < G::NCH) && j < kv_stop && j >= p.Lp) {
+                    const long jr = j - p.Lp;
+                    creg[i] = *reinterpret_cast<const f32x4*>(p.cos_k + jr * (D / 2) + cc * 4);
+                    sreg[i] = *reinterpret_cast<const f32x4*>(p.sin_k + jr * (D / 2) + cc * 4);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int idx = tid + NT * i;
+            const int row = idx / G::CPR;
+            const int cc = idx - row * G::CPR;
+            if (EXACT || idx < G::NCH) {
+                u32x4 kk = kreg[i];
+                if constexpr (ROPE_K) kk = rope_chunk<T>(kk, creg[i], sreg[i]);
+                *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = kk;
+            }
+        }
+    }
+    __device__ __forceinline__ void store_v(unsigned char* Vs) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int idx = tid + NT * i;
+            const int row = idx / G::CPR;
+            const int cc = idx - row * G::CPR;
+            if (EXACT || idx < G::NCH) *reinterpret_cast<u32x4*>(Vs + row * G::V_STRIDE + cc * 16) = vreg[i];
+        }
+    }
+};
+
+// Zero the LDS pad columns of `stages` K and V buffers once (tile stores never touch them).
+template <int D, int NT>
+__device__ __forceinline__ void zero_pads(unsigned char* kbuf0, unsigned char* vbuf0, int k_stage_bytes, int v_stage_bytes, int stages, int tid) {
+    using G = HeadGeo<D>;
+    for (int st = 0; st < stages; ++st) {
+        if constexpr (G::DK > D) {
+            for (int r = tid; r < kBN; r += NT)
+                *reinterpret_cast<u32x4*>(kbuf0 + st * k_stage_bytes + r * G::K_STRIDE + D * 2) = u32x4{0, 0, 0, 0};
+        }
+        if constexpr (G::DV > D) {
+            constexpr int PC = (G::DV - D) / 8;
+            for (int i = tid; i < kBN * PC; i += NT)
+                *reinterpret_cast<u32x4*>(vbuf0 + st * v_stage_bytes + (i / PC) * G::V_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
+        }
+    }
+}
+
+// Coalesced write-out of BM staged rows.
+template <typename T, int D, int NT>
+__device__ __forceinline__ void write_output(const unsigned char* Os, T* o_base, long o_rs, int q0, int Lq, int BM, int tid) {
+    using G = HeadGeo<D>;
+    for (int idx = tid; idx < BM * G::CPR; idx += NT) {
+        const int row = idx / G::CPR;
+        const int cc = idx - row * G::CPR;
+        if (q0 + row < Lq)
+            *reinterpret_cast<u32x4*>(o_base + static_cast<long>(q0 + row) * o_rs + cc * 8) =
+                *reinterpret_cast<const u32x4*>(Os + row * G::O_STRIDE + cc * 16);
+    }
+}
+
+// ───────────────────────────── 4-wavefront kernel ─────────────────────────────
+constexpr int kThreads4 = 256;
+template <int D> constexpr int lds_bytes_4() {
+    using G = HeadGeo<D>;
+    const int kv = 2 * (G::K_BYTES + G::V_BYTES);
+    const int o = 128 * G::O_STRIDE;
+    return kv > o ? kv : o;
 }
 
 template <typename T, int D, bool ROPE_K>
-__global__ void __launch_bounds__(kThreads, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(const SdpaDev p) {
-    using G = Geo<D>;
+__global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(const SdpaDev p) {
+    using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
+    constexpr int BM = 128;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    unsigned char* const Ks = smem;
-    unsigned char* const Vs = smem + G::K_BYTES;
-    float* const Ms = reinterpret_cast<float*>(smem + G::K_BYTES + G::V_BYTES);
     __shared__ int red[8];
+    constexpr int STAGE = G::K_BYTES + G::V_BYTES;
 
-    // Work-group id -> (batch, head, query tile). Hardware deals consecutive work-group ids
-    // round-robin over the 8 XCDs; undo that so each XCD (one L2) gets a contiguous run of
-    // logical tiles, i.e. query tiles that share the same K/V.
-    const int chunk = (p.n_blocks + 7) >> 3;
-    const int logical = (blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
-    if (logical >= p.n_blocks) return;
+    const int logical = logical_block(p.n_blocks);
+    if (logical < 0) return;
     int qt = logical % p.n_q_tiles;
     const int bh = logical / p.n_q_tiles;
     const int h = bh % p.H;
@@ -135,278 +185,242 @@ __global__ void __launch_bounds__(kThreads, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(c
     const int lane = tid & 63;
     const int lq = lane & 31;
     const int lh = lane >> 5;
-    const int q0 = qt * kBM;
+    const int q0 = qt * BM;
     const int qrow = q0 + wave * 32 + lq;
     const bool qvalid = qrow < p.Lq;
-
-    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     const int hk = h / p.kv_group;
-    const T* const k_base = static_cast<const T*>(p.k) + b * p.k_bs + hk * D;
-    const T* const v_base = static_cast<const T*>(p.v) + b * p.v_bs + hk * D;
-    const T* const kp_base = p.kp ? static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D : nullptr;
-    const T* const vp_base = p.vp ? static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D : nullptr;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+    const float* const key_mask = p.key_mask ? p.key_mask + b * p.key_mask_bs : nullptr;
 
-    // ── visible key interval [lo, hi) of this lane's query row ──
-    int lo = 0, hi = p.Lk;
-    if (p.kv_valid_len) hi = min(hi, p.kv_valid_len[b]);
-    if (p.mask_mode == MI_MASK_CAUSAL) {
-        const int pos1 = p.q_offset + qrow + 1;
-        hi = min(hi, pos1);
-        if (p.window > 0) lo = max(0, pos1 - p.window);
-    } else if (p.mask_mode == MI_MASK_BLOCK_CAUSAL) {
-        // static indices only: the segment table stays in scalar registers
-        int sk = p.seg_k_end[0], sc = p.seg_causal[0];
-#pragma unroll
-        for (int s = 1; s < MI_MAX_SEGMENTS; ++s)
-            if (s < p.n_seg && qrow >= p.seg_q_end[s - 1]) { sk = p.seg_k_end[s]; sc = p.seg_causal[s]; }
-        hi = min(hi, sk);
-        if (sc) hi = min(hi, p.q_offset + qrow + 1);
-    }
-    if (!qvalid || hi <= lo) { lo = 0; hi = 0; }
-    // wave-wide and group-wide extents
-    int w_lo_min = hi > lo ? lo : 0x7fffffff, w_hi_max = hi, w_hi_min = hi, w_lo_max = lo;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        w_lo_min = min(w_lo_min, __shfl_xor(w_lo_min, off));
-        w_hi_max = max(w_hi_max, __shfl_xor(w_hi_max, off));
-        w_hi_min = min(w_hi_min, __shfl_xor(w_hi_min, off));
-        w_lo_max = max(w_lo_max, __shfl_xor(w_lo_max, off));
-    }
-    if (lane == 0) { red[wave] = w_lo_min; red[4 + wave] = w_hi_max; }
-
-    // ── zero the LDS pad columns once (tile loads never touch them) ──
-    if constexpr (G::DK > D) {
-        for (int r = tid; r < kBN; r += kThreads)
-            *reinterpret_cast<u32x4*>(Ks + r * G::K_STRIDE + D * 2) = u32x4{0, 0, 0, 0};
-    }
-    if constexpr (G::DV > D) {
-        constexpr int PC = (G::DV - D) / 8;
-        for (int i = tid; i < kBN * PC; i += kThreads)
-            *reinterpret_cast<u32x4*>(Vs + (i / PC) * G::V_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
-    }
+    int lo, hi;
+    row_interval(p, b, qrow, qvalid, lo, hi);
+    const WaveExtent we = wave_extent(lo, hi);
+    if (lane == 0) { red[wave] = we.lo_min; red[4 + wave] = we.hi_max; }
+    zero_pads<D, kThreads4>(smem, smem + G::K_BYTES, STAGE, STAGE, 2, tid);
     __syncthreads();
     const int g_lo = min(min(red[0], red[1]), min(red[2], red[3]));
     const int kv_stop = max(max(red[4], red[5]), max(red[6], red[7]));
     const int kv_start = g_lo == 0x7fffffff ? 0 : (g_lo / kBN) * kBN;
 
-    // ── Q fragments (B operand of K Q^T), RoPE applied on the way in ──
     V8 qf[G::KC];
-#pragma unroll
-    for (int c = 0; c < G::KC; ++c) {
-        const int d0 = 16 * c + 8 * lh;
-        u32x4 raw = u32x4{0, 0, 0, 0};
-        if (qvalid && d0 < D) {
-            raw = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + d0);
-            if (p.cos_q) {
-                const f32x4 cs = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
-                const f32x4 sn = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
-                raw = rope_chunk<T>(raw, cs, sn);
-            }
-        }
-        qf[c] = __builtin_bit_cast(V8, raw);
-    }
+    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
 
     f32x16 oacc[G::VB];
 #pragma unroll
     for (int vb = 0; vb < G::VB; ++vb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
-    float m_run = kNegInf;  // running max of raw scores
-    float l_run = 0.f;      // this lane's share of the running denominator
+    SoftmaxState st;
     const float cl2 = p.scale_log2;
+    const float lazy_raw = kLazyLog2 / cl2;
 
-    // ── tile prefetch registers ──
-    u32x4 kreg[G::NLD], vreg[G::NLD];
-    float mreg = 1.f;
+    TileMover<T, D, kThreads4, ROPE_K> mv{p,
+                                          static_cast<const T*>(p.k) + b * p.k_bs + hk * D,
+                                          static_cast<const T*>(p.v) + b * p.v_bs + hk * D,
+                                          p.kp ? static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D : nullptr,
+                                          p.vp ? static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D : nullptr,
+                                          tid, kv_stop, {}, {}};
 
-    auto issue_loads = [&](int j0) {
-#pragma unroll
-        for (int i = 0; i < G::NLD; ++i) {
-            const int idx = tid + kThreads * i;
-            const int row = idx / G::CPR;
-            const int cc = idx - row * G::CPR;
-            const int j = j0 + row;
-            kreg[i] = u32x4{0, 0, 0, 0};
-            vreg[i] = u32x4{0, 0, 0, 0};
-            if (idx < G::NCH && j < kv_stop) {
-                if (j < p.Lp) {
-                    kreg[i] = *reinterpret_cast<const u32x4*>(kp_base + static_cast<long>(j) * p.kp_rs + cc * 8);
-                    vreg[i] = *reinterpret_cast<const u32x4*>(vp_base + static_cast<long>(j) * p.vp_rs + cc * 8);
-                } else {
-                    const long jr = j - p.Lp;
-                    kreg[i] = *reinterpret_cast<const u32x4*>(k_base + jr * p.k_rs + cc * 8);
-                    vreg[i] = *reinterpret_cast<const u32x4*>(v_base + jr * p.v_rs + cc * 8);
-                }
-            }
-        }
-        if (p.key_mask && tid < kBN) {
-            const int j = j0 + tid;
-            mreg = j < p.Lk ? p.key_mask[b * p.key_mask_bs + j] : 0.f;
-        }
-    };
-    auto store_tile = [&](int j0) {
-        // The rotation tables are fetched here rather than with the tile: they are L2 hits
-        // shared by every head, and holding them across the MFMA section would cost
-        // 8 registers per chunk exactly where pressure peaks. Prefix rows are stored rotated.
-        f32x4 creg[ROPE_K ? G::NLD : 1], sreg[ROPE_K ? G::NLD : 1];
-        if constexpr (ROPE_K) {
-#pragma unroll
-            for (int i = 0; i < G::NLD; ++i) {
-                const int idx = tid + kThreads * i;
-                const int row = idx / G::CPR;
-                const int cc = idx - row * G::CPR;
-                const int j = j0 + row;
-                creg[i] = f32x4{1.f, 1.f, 1.f, 1.f};
-                sreg[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if (idx < G::NCH && j < kv_stop && j >= p.Lp) {
-                    const long jr = j - p.Lp;
-                    creg[i] = *reinterpret_cast<const f32x4*>(p.cos_k + jr * (D / 2) + cc * 4);
-                    sreg[i] = *reinterpret_cast<const f32x4*>(p.sin_k + jr * (D / 2) + cc * 4);
-                }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < G::NLD; ++i) {
-            const int idx = tid + kThreads * i;
-            const int row = idx / G::CPR;
-            const int cc = idx - row * G::CPR;
-            if (idx < G::NCH) {
-                u32x4 kk = kreg[i];
-                if constexpr (ROPE_K) kk = rope_chunk<T>(kk, creg[i], sreg[i]);
-                *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = kk;
-                *reinterpret_cast<u32x4*>(Vs + row * G::V_STRIDE + cc * 16) = vreg[i];
-            }
-        }
-        if (p.key_mask && tid < kBN) Ms[tid] = mreg;
-    };
-
-    if (kv_start < kv_stop) issue_loads(kv_start);
-
+    // key loop, LDS double buffered: one barrier per tile
+    if (kv_start < kv_stop) {
+        mv.template issue<0>(kv_start);
+        mv.template issue<1>(kv_start);
+        mv.store_k(kv_start, smem);
+        mv.store_v(smem + G::K_BYTES);
+        if (kv_start + kBN < kv_stop) { mv.template issue<0>(kv_start + kBN); mv.template issue<1>(kv_start + kBN); }
+    }
+    __syncthreads();
+    int stage = 0;
     for (int j0 = kv_start; j0 < kv_stop; j0 += kBN) {
-        store_tile(j0);
-        __syncthreads();
-        if (j0 + kBN < kv_stop) issue_loads(j0 + kBN);
-
+        const unsigned char* Ks = smem + stage * STAGE;
+        const unsigned char* Vs = Ks + G::K_BYTES;
         // wavefronts none of whose rows can see this tile only help with the loads
-        if (j0 < w_hi_max && j0 + kBN > w_lo_min) {
-            // ── S^T = K Q^T : 2 blocks of 32 keys ──
+        if (j0 < we.hi_max && j0 + kBN > we.lo_min) {
             f32x16 sacc[2];
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
-#pragma unroll
-                for (int c = 0; c < G::KC; ++c) {
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(Ks + (32 * kb + lq) * G::K_STRIDE + (16 * c + 8 * lh) * 2);
-                    sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], sacc[kb]);
-                }
-            }
-            // ── visibility ──
-            const bool need_mask = (j0 + kBN > w_hi_min) || (j0 < w_lo_max) || (p.key_mask != nullptr);
-            if (need_mask) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int bb = 0; bb < 4; ++bb) {
-                        const int kbase = 32 * kb + 8 * bb + 4 * lh;
-                        f32x4 mv = {1.f, 1.f, 1.f, 1.f};
-                        if (p.key_mask) mv = *reinterpret_cast<const f32x4*>(Ms + kbase);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const int key = j0 + kbase + i;
-                            const bool vis = key >= lo && key < hi && mv[i] != 0.f;
-                            if (!vis) sacc[kb][4 * bb + i] = kNegInf;
-                        }
-                    }
-            }
-            // ── online softmax (base 2) ──
-            float mloc = kNegInf;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) mloc = fmaxf(mloc, sacc[kb][e]);
-            mloc = exchange_max(mloc);
-            const float m_new = fmaxf(m_run, mloc);
-            const float mc = (m_new == kNegInf) ? 0.f : m_new * cl2;
-            const float alpha = (m_run == kNegInf) ? 0.f : __builtin_amdgcn_exp2f(m_run * cl2 - mc);
-            m_run = m_new;
-            float lsum = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const float pe = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][e], cl2, -mc));
-                    sacc[kb][e] = pe;
-                    lsum += pe;
-                }
-            l_run = l_run * alpha + lsum;
-#pragma unroll
-            for (int vb = 0; vb < G::VB; ++vb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) oacc[vb][e] *= alpha;
-            // ── P^T as B operand: 16-key chunk c4 = acc[8*(c4%2) .. +7] of block c4/2 ──
             V8 pf[4];
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4)
-#pragma unroll
-                for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
-            // ── O^T += V^T P^T ──
-            const int trow = (lane & 15) >> 2;                     // key row inside a 4-key group
-            const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);  // head-dim column inside a 32 block
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) {
-#pragma unroll
-                for (int vb = 0; vb < G::VB; ++vb) {
-                    const unsigned char* vptr = Vs + (16 * c4 + 4 * lh + trow) * G::V_STRIDE + (32 * vb + tcol) * 2;
-                    const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4*)(vptr));
-                    const s16x4 v_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::V_STRIDE));
-                    const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    oacc[vb] = Mma<T>::run(__builtin_bit_cast(V8, a), pf[c4], oacc[vb]);
-                }
-            }
+            qk_tile<T, D>(Ks, qf, lq, lh, sacc);
+            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= we.hi_min) && (key_mask == nullptr);
+            if (interior) softmax_tile<T, D, false>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
+            else softmax_tile<T, D, true>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
+            pv_tile<T, D>(Vs, pf, lane, oacc);
         }
+        if (j0 + kBN < kv_stop) {
+            unsigned char* Kn = smem + (stage ^ 1) * STAGE;
+            mv.store_k(j0 + kBN, Kn);
+            mv.store_v(Kn + G::K_BYTES);
+        }
+        if (j0 + 2 * kBN < kv_stop) { mv.template issue<0>(j0 + 2 * kBN); mv.template issue<1>(j0 + 2 * kBN); }
         __syncthreads();
+        stage ^= 1;
     }
 
-    // ── epilogue: normalise, transpose through LDS, write full rows ──
-    const float l_tot = exchange_sum(l_run);
+    const float l_tot = exchange_sum(st.l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    unsigned char* const Os = smem;
-    typedef T t4 __attribute__((ext_vector_type(4)));
+    stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
+    __syncthreads();
+    write_output<T, D, kThreads4>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+}
+
+// ───────────────────────── 8-wavefront ping-pong kernel ─────────────────────────
+constexpr int kThreads8 = 512;
+template <int D> constexpr int lds_bytes_8() {
+    using G = HeadGeo<D>;
+    const int kv = 2 * (G::K_BYTES + G::V_BYTES);
+    const int o = 256 * G::O_STRIDE;
+    return kv > o ? kv : o;
+}
+
+// Time is counted in slots separated by work-group barriers. Group 0 (wavefronts 0-3) runs its MFMA
+// phase in even slots and its VALU phase in odd slots; group 1 (wavefronts 4-7, sharing the SIMDs of
+// 0-3) the other way round. With t = slot / 2:
+//   MFMA phase:  O += V_t^T P_t ;  S_{t+1} = K_{t+1} Q^T           (reads LDS tiles K_{t+1}, V_t)
+//   VALU phase:  P = softmax(S) of the tile just scored; store this thread's share of tiles
+//                K_{t+2}, V_{t+1} into the LDS buffers of K_t, V_{t-1}; issue the next global loads
+// Tiles K_{t+1}, V_t are complete in LDS before slot 2t and last read in slot 2t+1, and the buffers
+// they replace were last read in slot 2t-1, so two buffers per operand suffice.
+template <typename T, int D, bool ROPE_K>
+__global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev p) {
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    constexpr int BM = 256;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ int red[16];
+    unsigned char* const Kbuf = smem;                    // 2 x K tile
+    unsigned char* const Vbuf = smem + 2 * G::K_BYTES;   // 2 x V tile
+
+    const int logical = logical_block(p.n_blocks);
+    if (logical < 0) return;
+    int qt = logical % p.n_q_tiles;
+    const int bh = logical / p.n_q_tiles;
+    const int h = bh % p.H;
+    const int b = bh / p.H;
+    if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;  // longest key ranges first
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int grp = wave >> 2;      // phase group
+    const int lane = tid & 63;
+    const int lq = lane & 31;
+    const int lh = lane >> 5;
+    const int q0 = qt * BM;
+    const int qrow = q0 + wave * 32 + lq;
+    const bool qvalid = qrow < p.Lq;
+    const int hk = h / p.kv_group;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+    const float* const key_mask = p.key_mask ? p.key_mask + b * p.key_mask_bs : nullptr;
+
+    int lo, hi;
+    row_interval(p, b, qrow, qvalid, lo, hi);
+    const WaveExtent we = wave_extent(lo, hi);
+    if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    zero_pads<D, kThreads8>(Kbuf, Vbuf, G::K_BYTES, G::V_BYTES, 2, tid);
+    __syncthreads();
+    int g_lo = red[0], kv_stop = red[8];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) { g_lo = min(g_lo, red[w]); kv_stop = max(kv_stop, red[8 + w]); }
+    const int kv_start = g_lo == 0x7fffffff ? 0 : (g_lo / kBN) * kBN;
+    const int n_tiles = kv_stop > kv_start ? (kv_stop - kv_start + kBN - 1) / kBN : 0;
+
+    V8 qf[G::KC];
+    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
+
+    f32x16 oacc[G::VB];
 #pragma unroll
     for (int vb = 0; vb < G::VB; ++vb)
 #pragma unroll
-        for (int bb = 0; bb < 4; ++bb) {
-            const int d0 = 32 * vb + 8 * bb + 4 * lh;
-            if (d0 < D) {
-                t4 ov;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ov[i] = static_cast<T>(oacc[vb][4 * bb + i] * inv);
-                *reinterpret_cast<t4*>(Os + (wave * 32 + lq) * G::O_STRIDE + d0 * 2) = ov;
-            }
+        for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
+    SoftmaxState st;
+    const float cl2 = p.scale_log2;
+    const float lazy_raw = kLazyLog2 / cl2;
+
+    TileMover<T, D, kThreads8, ROPE_K> mv{p,
+                                          static_cast<const T*>(p.k) + b * p.k_bs + hk * D,
+                                          static_cast<const T*>(p.v) + b * p.v_bs + hk * D,
+                                          p.kp ? static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D : nullptr,
+                                          p.vp ? static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D : nullptr,
+                                          tid, kv_stop, {}, {}};
+    auto tile_j0 = [&](int t) { return kv_start + t * kBN; };
+    auto tile_active = [&](int t) { return t < n_tiles && tile_j0(t) < we.hi_max && tile_j0(t) + kBN > we.lo_min; };
+    // this thread's share of tiles K_kt, V_vt: registers -> LDS, then prefetch K_{kt+1}, V_{vt+1}
+    auto advance_tiles = [&](int kt, int vt) {
+        if (kt < n_tiles) mv.store_k(tile_j0(kt), Kbuf + (kt & 1) * G::K_BYTES);
+        if (vt < n_tiles) mv.store_v(Vbuf + (vt & 1) * G::V_BYTES);
+        if (kt + 1 < n_tiles) mv.template issue<0>(tile_j0(kt + 1));
+        if (vt + 1 < n_tiles) mv.template issue<1>(tile_j0(vt + 1));
+    };
+    f32x16 sacc[2];
+    V8 pf[4];
+    auto softmax_of = [&](int t) {
+        const int j0 = tile_j0(t);
+        const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= we.hi_min) && (key_mask == nullptr);
+        if (interior) softmax_tile<T, D, false>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
+        else softmax_tile<T, D, true>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
+    };
+
+    if (n_tiles > 0) {
+        // ── prologue, both groups in step: K_0 to LDS, score and exponentiate tile 0 ──
+        mv.template issue<0>(tile_j0(0));
+        mv.store_k(tile_j0(0), Kbuf);
+        if (n_tiles > 1) mv.template issue<0>(tile_j0(1));
+        mv.template issue<1>(tile_j0(0));
+        __syncthreads();
+        if (tile_active(0)) {
+            qk_tile<T, D>(Kbuf, qf, lq, lh, sacc);
+            softmax_of(0);
         }
-    __syncthreads();
-    for (int idx = tid; idx < kBM * G::CPR; idx += kThreads) {
-        const int row = idx / G::CPR;
-        const int cc = idx - row * G::CPR;
-        if (q0 + row < p.Lq)
-            *reinterpret_cast<u32x4*>(o_base + static_cast<long>(q0 + row) * p.o_rs + cc * 8) =
-                *reinterpret_cast<const u32x4*>(Os + row * G::O_STRIDE + cc * 16);
+        advance_tiles(1, 0);   // K_1, V_0 to LDS; registers now hold K_2, V_1
+        __syncthreads();
+        // ── group 1 falls one slot behind: its first slot only moves tiles ──
+        if (grp == 1) {
+            advance_tiles(2, 1);
+            __syncthreads();
+        }
+        for (int t = 0; t < n_tiles; ++t) {
+            // MFMA phase
+            __builtin_amdgcn_s_setprio(2);
+            if (tile_active(t)) pv_tile<T, D>(Vbuf + (t & 1) * G::V_BYTES, pf, lane, oacc);
+            if (tile_active(t + 1)) qk_tile<T, D>(Kbuf + ((t + 1) & 1) * G::K_BYTES, qf, lq, lh, sacc);
+            __builtin_amdgcn_s_setprio(0);
+            __syncthreads();
+            // VALU phase
+            if (tile_active(t + 1)) softmax_of(t + 1);
+            advance_tiles(t + 2 + grp, t + 1 + grp);
+            __syncthreads();
+        }
+        if (grp == 0) __syncthreads();
     }
+
+    const float l_tot = exchange_sum(st.l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
+    __syncthreads();
+    write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
 }
 
 template <typename T, int D>
-int launch_d(const SdpaDev& p, hipStream_t stream) {
+int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     const bool rope_k = p.cos_k != nullptr;
-    const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads);
-    const size_t lds = Geo<D>::LDS_BYTES;
-    if (rope_k) {
-        hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, true>), grid, block, lds, stream, p);
+    // 256-row tiles when they give every CU at least one work group; head_dim above 128 does not fit
+    // two wavefronts per SIMD and stays on the 128-row kernel.
+    const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
+    const int choice = sdpa_kernel_choice();
+    const bool pingpong = D <= 128 && (choice == 2 || (choice == 0 && tiles256 >= n_cu));
+    if (pingpong) {
+        p.n_q_tiles = (p.Lq + 255) / 256;
+        p.n_blocks = static_cast<int>(tiles256);
+        const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads8);
+        if constexpr (D <= 128) {
+            if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
+            else hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false>), grid, block, lds_bytes_8<D>(), stream, p);
+        }
     } else {
-        hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false>), grid, block, lds, stream, p);
+        p.n_q_tiles = (p.Lq + 127) / 128;
+        p.n_blocks = p.B * p.H * p.n_q_tiles;
+        const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads4);
+        if (rope_k) hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, true>), grid, block, lds_bytes_4<D>(), stream, p);
+        else hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false>), grid, block, lds_bytes_4<D>(), stream, p);
     }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("sdpa_fwd launch: %s", hipGetErrorString(e));
@@ -414,16 +428,16 @@ int launch_d(const SdpaDev& p, hipStream_t stream) {
 }
 
 template <typename T>
-int launch_t(const SdpaDev& p, int head_dim, hipStream_t stream) {
+int launch_t(const SdpaDev& p, int head_dim, int n_cu, hipStream_t stream) {
     switch (head_dim) {
-        case 40: return launch_d<T, 40>(p, stream);
-        case 64: return launch_d<T, 64>(p, stream);
-        case 72: return launch_d<T, 72>(p, stream);
-        case 80: return launch_d<T, 80>(p, stream);
-        case 96: return launch_d<T, 96>(p, stream);
-        case 112: return launch_d<T, 112>(p, stream);
-        case 128: return launch_d<T, 128>(p, stream);
-        case 160: return launch_d<T, 160>(p, stream);
+        case 40: return launch_d<T, 40>(p, n_cu, stream);
+        case 64: return launch_d<T, 64>(p, n_cu, stream);
+        case 72: return launch_d<T, 72>(p, n_cu, stream);
+        case 80: return launch_d<T, 80>(p, n_cu, stream);
+        case 96: return launch_d<T, 96>(p, n_cu, stream);
+        case 112: return launch_d<T, 112>(p, n_cu, stream);
+        case 128: return launch_d<T, 128>(p, n_cu, stream);
+        case 160: return launch_d<T, 160>(p, n_cu, stream);
         default: return fail("mi_sdpa_forward: head_dim %d has no kernel (40, 64, 72, 80, 96, 112, 128, 160)", head_dim);
     }
 }
@@ -439,8 +453,9 @@ bool sdpa_supported(int dtype, int head_dim) {
 }
 
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream) {
-    if (dtype == MI_DTYPE_BF16) return launch_t<__bf16>(p, head_dim, stream);
-    if (dtype == MI_DTYPE_F16) return launch_t<_Float16>(p, head_dim, stream);
+    const int n_cu = device_cu_count();
+    if (dtype == MI_DTYPE_BF16) return launch_t<__bf16>(p, head_dim, n_cu, stream);
+    if (dtype == MI_DTYPE_F16) return launch_t<_Float16>(p, head_dim, n_cu, stream);
     return fail("mi_sdpa_forward: dtype %d not supported (fp16 = 1, bf16 = 2)", dtype);
 }
 

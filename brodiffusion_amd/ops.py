@@ -83,6 +83,11 @@ def _as3(op: str, t: torch.Tensor, name: str):
     _fail(op, f"{name} must be (rows, cols) or (batch, rows, cols)")
 
 
+def set_sdpa_kernel_choice(choice: int) -> None:
+    """0 = by problem size, 1 = 128-row tiles, 2 = 256-row ping-pong kernel (see mi_sdpa_set_kernel_choice)."""
+    capi.check(capi.lib().mi_sdpa_set_kernel_choice(choice), "set_sdpa_kernel_choice")
+
+
 def device_info() -> dict:
     info = capi.MiDeviceInfo()
     capi.check(capi.lib().mi_device_info(C.byref(info)), "mi_device_info")

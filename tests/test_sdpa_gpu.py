@@ -11,6 +11,14 @@ from helpers import TOL, assert_close, randn, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["rows128", "rows256_pingpong"])
+def kernel_choice(request):
+    """Every case runs on both kernels: 4 wavefronts x 128 rows, and 8 wavefronts x 256 rows (ping-pong)."""
+    bd.set_sdpa_kernel_choice(1 if request.param == "rows128" else 2)
+    yield request.param
+    bd.set_sdpa_kernel_choice(0)
+
+
 def _oracle_batched(oracle, q, k, v, H, **kw):
     return np.stack([oracle.sdpa(q[b], k[b], v[b], H, **kw) for b in range(q.shape[0])])
 
