@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libmi_attention.so")
+# MI_ATTENTION_LIB points at an alternative build of the same library (kernel tuning experiments).
+LIB_PATH = os.environ.get("MI_ATTENTION_LIB") or os.path.join(HERE, "lib", "libmi_attention.so")
 
 MI_DTYPE_F16 = 1
 MI_DTYPE_BF16 = 2

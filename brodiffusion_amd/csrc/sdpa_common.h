@@ -103,11 +103,11 @@ __device__ __forceinline__ void row_interval(const SdpaDev& p, int b, int qrow, 
         hi = min(hi, pos1);
         if (p.window > 0) lo = max(0, pos1 - p.window);
     } else if (p.mask_mode == MI_MASK_BLOCK_CAUSAL) {
-        // static indices only: the segment table stays in scalar registers
+        // a scalar loop over the segment table (uniform index: scalar loads from the kernel arguments)
         int sk = p.seg_k_end[0], sc = p.seg_causal[0];
-#pragma unroll
-        for (int s = 1; s < MI_MAX_SEGMENTS; ++s)
-            if (s < p.n_seg && qrow >= p.seg_q_end[s - 1]) { sk = p.seg_k_end[s]; sc = p.seg_causal[s]; }
+#pragma unroll 1
+        for (int s = 1; s < p.n_seg; ++s)
+            if (qrow >= p.seg_q_end[s - 1]) { sk = p.seg_k_end[s]; sc = p.seg_causal[s]; }
         hi = min(hi, sk);
         if (sc) hi = min(hi, p.q_offset + qrow + 1);
     }
@@ -125,6 +125,11 @@ __device__ __forceinline__ WaveExtent wave_extent(int lo, int hi) {
         w.hi_min = min(w.hi_min, __shfl_xor(w.hi_min, off));
         w.hi_max = max(w.hi_max, __shfl_xor(w.hi_max, off));
     }
+    // identical in every lane now: move to scalar registers so tile decisions are scalar branches
+    w.lo_min = __builtin_amdgcn_readfirstlane(w.lo_min);
+    w.lo_max = __builtin_amdgcn_readfirstlane(w.lo_max);
+    w.hi_min = __builtin_amdgcn_readfirstlane(w.hi_min);
+    w.hi_max = __builtin_amdgcn_readfirstlane(w.hi_max);
     return w;
 }
 
@@ -149,23 +154,81 @@ __device__ __forceinline__ void load_q_frags(typename Mma<T>::v8 (&qf)[HeadGeo<D
     }
 }
 
-// S^T = K Q^T for one 64-key tile: 2 blocks of 32 keys.
-template <typename T, int D>
-__device__ __forceinline__ void qk_tile(const unsigned char* Ks, const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], int lq, int lh,
-                                        f32x16 (&sacc)[2]) {
+// The MFMA work of one step as a single software-pipelined stream: first O^T += V^T P^T for one
+// 64-key tile (if DO_PV), then S^T = K Q^T for one 64-key tile (if DO_QK). Every MFMA takes its A
+// operand from LDS; the LDS reads run kAhead operands ahead of the MFMA that consumes them so that
+// LDS latency hides behind the matrix pipe, and the order is pinned with scheduling barriers.
+//   PV operand (c4, vb): V^T fragment = head-dim block vb x 16-key chunk c4, through two LDS transpose
+//     reads (within 16 lanes, lane j supplies the address of 4 consecutive head-dim elements of key
+//     row j/4, and lane i receives 4 consecutive keys of head-dim column i).
+//   QK operand (kb, c):  K fragment = key block kb x 16 head-dim elements, one 16-byte read per lane.
+constexpr int kAhead = 4;
+#ifdef MI_EXPERIMENT_NO_SCHED_BARRIER
+#define MI_SCHED_BARRIER
+#else
+#define MI_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0);
+#endif
+
+// `mid` is called once, a few MFMAs into the stream: work placed there (tile movement) issues in
+// the shadow of the matrix pipe.
+struct NoMid { __device__ __forceinline__ void operator()() const {} };
+
+template <typename T, int D, bool DO_PV, bool DO_QK, typename Mid = NoMid>
+__device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsigned char* Ks, const typename Mma<T>::v8 (&pf)[4],
+                                            const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], f32x16 (&oacc)[HeadGeo<D>::VB],
+                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid()) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
+    constexpr int NPV = DO_PV ? 4 * G::VB : 0;
+    constexpr int NQK = DO_QK ? 2 * G::KC : 0;
+    constexpr int N = NPV + NQK;
+    if constexpr (N == 0) return;
+    const int lq = lane & 31;
+    const int lh = lane >> 5;
+    const int trow = (lane & 15) >> 2;
+    const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const unsigned char* const vlane = Vs + (4 * lh + trow) * G::V_STRIDE + tcol * 2;
+    const unsigned char* const klane = Ks + lq * G::K_STRIDE + 8 * lh * 2;
+    auto fetch = [&](int i) -> V8 {
+        if (i < NPV) {
+            const int c4 = i / G::VB, vb = i % G::VB;
+            const unsigned char* vptr = vlane + 16 * c4 * G::V_STRIDE + 32 * vb * 2;
+            const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
+            const s16x4 v_hi =
+                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::V_STRIDE));
+            const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(V8, a);
+        } else {
+            const int k = i - NPV;
+            const int kb = k / G::KC, c = k % G::KC;
+            const u32x4 a = *reinterpret_cast<const u32x4*>(klane + 32 * kb * G::K_STRIDE + 16 * c * 2);
+            return __builtin_bit_cast(V8, a);
+        }
+    };
+    V8 ring[kAhead];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int i = 0; i < kAhead && i < N; ++i) ring[i] = fetch(i);
 #pragma unroll
-        for (int c = 0; c < G::KC; ++c) {
-            const u32x4 a = *reinterpret_cast<const u32x4*>(Ks + (32 * kb + lq) * G::K_STRIDE + (16 * c + 8 * lh) * 2);
+    for (int i = 0; i < N; ++i) {
+        const V8 a = ring[i % kAhead];
+        if (i < NPV) {
+            const int c4 = i / G::VB, vb = i % G::VB;
+            oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
+        } else {
+            const int k = i - NPV;
+            const int kb = k / G::KC, c = k % G::KC;
             if (c == 0) {
                 const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], zero);
+                sacc[kb] = Mma<T>::run(a, qf[c], zero);
             } else {
-                sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], sacc[kb]);
+                sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
             }
+        }
+        if (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
+        MI_SCHED_BARRIER
+        if (i == (N > 8 ? 5 : 0)) {
+            mid();
+            MI_SCHED_BARRIER
         }
     }
 }
@@ -180,25 +243,38 @@ struct SoftmaxState {
     float l = 0.f;      // this lane's share of the denominator
 };
 
-// Masks (if MASKED), exponentiates and packs one score tile into the B operands of the PV product.
-template <typename T, int D, bool MASKED>
+// Masks (if `masked`, a wave-uniform flag), exponentiates and packs one score tile into the B operands
+// of the PV product. The mask step only touches the scores, so the two cases share every other
+// instruction and the accumulators are updated at one place only (separate masked / unmasked copies of
+// this function cost the register allocator ~70 registers in copies of O).
+template <typename T, int D>
 __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                             SoftmaxState& st, float cl2, float lazy_raw, int j0, int lo, int hi, int lh,
-                                             const float* key_mask, int Lk) {
-    if constexpr (MASKED) {
+                                             SoftmaxState& st, float cl2, float lazy_raw, bool masked, int j0, int lo, int hi,
+                                             int lh, const float* mask_tile) {
+    if (masked) {
+        // mask_tile: the 64 key-mask values of this tile staged in LDS (null when the call has no key mask)
+        if (mask_tile) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int bb = 0; bb < 4; ++bb) {
-                const int kbase = j0 + 32 * kb + 8 * bb + 4 * lh;
+                for (int bb = 0; bb < 4; ++bb) {
+                    const int kbase = 32 * kb + 8 * bb + 4 * lh;
+                    const f32x4 mk = *reinterpret_cast<const f32x4*>(mask_tile + kbase);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = kbase + i;
-                    bool vis = key >= lo && key < hi;
-                    if (key_mask) vis = vis && (key < Lk) && key_mask[key < Lk ? key : 0] != 0.f;
-                    if (!vis) sacc[kb][4 * bb + i] = kNegInf;
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = j0 + kbase + i;
+                        if (key < lo || key >= hi || mk[i] == 0.f) sacc[kb][4 * bb + i] = kNegInf;
+                    }
                 }
-            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                    if (key < lo || key >= hi) sacc[kb][e] = kNegInf;
+                }
+        }
     }
     float mloc = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
@@ -219,8 +295,13 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
     float lsum0 = 0.f, lsum1 = 0.f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
+#ifdef MI_EXPERIMENT_NO_EXP
+        const float p0 = __builtin_fmaf(sacc[0][e], cl2, -st.mc);
+        const float p1 = __builtin_fmaf(sacc[1][e], cl2, -st.mc);
+#else
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[0][e], cl2, -st.mc));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[1][e], cl2, -st.mc));
+#endif
         sacc[0][e] = p0;
         sacc[1][e] = p1;
         lsum0 += p0;
@@ -232,31 +313,6 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
     for (int c4 = 0; c4 < 4; ++c4)
 #pragma unroll
         for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
-}
-
-// O^T += V^T P^T for one 64-key tile. V^T fragments come from the row-major V tile through LDS
-// transpose reads: within 16 lanes, lane j supplies the address of 4 consecutive head-dim elements
-// of key row j/4, and lane i receives 4 consecutive keys of head-dim column i.
-template <typename T, int D>
-__device__ __forceinline__ void pv_tile(const unsigned char* Vs, const typename Mma<T>::v8 (&pf)[4], int lane,
-                                        f32x16 (&oacc)[HeadGeo<D>::VB]) {
-    using G = HeadGeo<D>;
-    using V8 = typename Mma<T>::v8;
-    const int lh = lane >> 5;
-    const int trow = (lane & 15) >> 2;
-    const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-#pragma unroll
-    for (int c4 = 0; c4 < 4; ++c4) {
-#pragma unroll
-        for (int vb = 0; vb < G::VB; ++vb) {
-            const unsigned char* vptr = Vs + (16 * c4 + 4 * lh + trow) * G::V_STRIDE + (32 * vb + tcol) * 2;
-            const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
-            const s16x4 v_hi =
-                __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::V_STRIDE));
-            const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            oacc[vb] = Mma<T>::run(__builtin_bit_cast(V8, a), pf[c4], oacc[vb]);
-        }
-    }
 }
 
 // Normalised output rows of one wavefront into the LDS staging area (row-major, O_STRIDE).

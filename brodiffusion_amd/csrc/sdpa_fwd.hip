@@ -30,6 +30,27 @@ __device__ __forceinline__ int logical_block(int n_blocks) {
     return logical < n_blocks ? logical : -1;
 }
 
+// The key axis is cut into 64-row tiles that never straddle the prefix / fresh boundary: prefix
+// tiles start at a multiple of 64 below prefix_len (the last one may be partial), fresh tiles start at
+// prefix_len + a multiple of 64. Rows of a tile at or beyond its segment's limit are zero in LDS and
+// masked in the scores.
+struct TilePlan {
+    int pre_lo, pre_hi, n_pre;  // prefix rows [pre_lo, pre_hi)
+    int fr_lo, fr_hi, n_tiles;  // all keys are numbered over [prefix ; fresh]
+    __device__ __forceinline__ TilePlan(int first_key, int stop_key, int Lp) {
+        pre_lo = first_key < Lp ? (first_key / kBN) * kBN : Lp;
+        pre_hi = min(stop_key, Lp);
+        n_pre = pre_hi > pre_lo ? (pre_hi - pre_lo + kBN - 1) / kBN : 0;
+        fr_lo = first_key > Lp ? Lp + ((first_key - Lp) / kBN) * kBN : Lp;
+        fr_hi = stop_key;
+        const int n_fr = fr_hi > fr_lo ? (fr_hi - fr_lo + kBN - 1) / kBN : 0;
+        n_tiles = n_pre + n_fr;
+    }
+    __device__ __forceinline__ bool in_prefix(int t) const { return t < n_pre; }
+    __device__ __forceinline__ int j0(int t) const { return t < n_pre ? pre_lo + t * kBN : fr_lo + (t - n_pre) * kBN; }
+    __device__ __forceinline__ int limit(int t) const { return t < n_pre ? pre_hi : fr_hi; }
+};
+
 // Cooperative K/V tile movement for a work group of NT threads: global -> registers -> LDS.
 // kreg / vreg hold this thread's 16-byte chunks of one K tile and one V tile (possibly different tiles).
 template <typename T, int D, int NT, bool ROPE_K>
@@ -38,66 +59,69 @@ struct TileMover {
     static constexpr int NLD = (G::NCH + NT - 1) / NT;
     static constexpr bool EXACT = (G::NCH % NT) == 0;
     const SdpaDev& p;
-    const T* k_base; const T* v_base; const T* kp_base; const T* vp_base;
-    int tid, kv_stop;
+    const TilePlan& plan;
+    const unsigned char* k_base; const unsigned char* v_base; const unsigned char* kp_base; const unsigned char* vp_base;
+    int tid;
     u32x4 kreg[NLD], vreg[NLD];
+    float mreg;   // key-mask value of key row `tid` of the K tile in kreg (threads 0..63, 4-wavefront kernel)
 
-    // which: 0 = K tile into kreg, 1 = V tile into vreg
-    template <int WHICH>
-    __device__ __forceinline__ void issue(int j0) {
-        u32x4 (&reg)[NLD] = WHICH == 0 ? kreg : vreg;
-        const T* fresh = WHICH == 0 ? k_base : v_base;
-        const T* pre = WHICH == 0 ? kp_base : vp_base;
-        const long f_rs = WHICH == 0 ? p.k_rs : p.v_rs;
-        const long p_rs = WHICH == 0 ? p.kp_rs : p.vp_rs;
-        const bool in_prefix = j0 + kBN <= p.Lp;
-        const bool in_fresh = j0 >= p.Lp;
-        if ((in_prefix || in_fresh) && j0 + kBN <= kv_stop) {
-            // whole tile from one buffer: uniform base pointer plus a fixed per-thread byte offset
-            const unsigned char* base = in_fresh ? reinterpret_cast<const unsigned char*>(fresh + static_cast<long>(j0 - p.Lp) * f_rs)
-                                                 : reinterpret_cast<const unsigned char*>(pre + static_cast<long>(j0) * p_rs);
-            const unsigned rsb = static_cast<unsigned>(in_fresh ? f_rs : p_rs) * 2u;
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-                const int idx = tid + NT * i;
-                const int row = idx / G::CPR;
-                const int cc = idx - row * G::CPR;
-                if (EXACT || idx < G::NCH) reg[i] = *reinterpret_cast<const u32x4*>(base + (static_cast<unsigned>(row) * rsb + cc * 16u));
-            }
-        } else {
-            // tile straddles the prefix / fresh boundary or the end of the visible keys
-#pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-                const int idx = tid + NT * i;
-                const int row = idx / G::CPR;
-                const int cc = idx - row * G::CPR;
-                const int j = j0 + row;
-                reg[i] = u32x4{0, 0, 0, 0};
-                if ((EXACT || idx < G::NCH) && j < kv_stop) {
-                    const T* r = j < p.Lp ? pre + static_cast<long>(j) * p_rs : fresh + static_cast<long>(j - p.Lp) * f_rs;
-                    reg[i] = *reinterpret_cast<const u32x4*>(r + cc * 8);
-                }
-            }
+    // key-mask values travel with the K tile: one float per key row, staged next to the tile in LDS
+    __device__ __forceinline__ void issue_mask(int t, const float* key_mask) {
+        if (tid < kBN) {
+            const int j = plan.j0(t) + tid;
+            mreg = j < plan.limit(t) ? key_mask[j] : 0.f;
         }
     }
-    __device__ __forceinline__ void store_k(int j0, unsigned char* Ks) {
+    __device__ __forceinline__ void store_mask(float* Ms) {
+        if (tid < kBN) Ms[tid] = mreg;
+    }
+
+    // WHICH: 0 = K tile t into kreg, 1 = V tile t into vreg
+    template <int WHICH>
+    __device__ __forceinline__ void issue(int t) {
+        u32x4 (&reg)[NLD] = WHICH == 0 ? kreg : vreg;
+        const bool pre = plan.in_prefix(t);
+        const int j0 = plan.j0(t);
+        const int nvalid = plan.limit(t) - j0;   // rows of this tile that exist
+        // uniform base pointer of the tile plus a fixed per-thread byte offset
+        const unsigned rsb = static_cast<unsigned>(pre ? (WHICH == 0 ? p.kp_rs : p.vp_rs) : (WHICH == 0 ? p.k_rs : p.v_rs)) * 2u;
+        const unsigned char* base = pre ? (WHICH == 0 ? kp_base : vp_base) + static_cast<unsigned long>(j0) * rsb
+                                        : (WHICH == 0 ? k_base : v_base) + static_cast<unsigned long>(j0 - p.Lp) * rsb;
+        // Rows past the end of the segment are read from its last row (always valid memory) and
+        // replaced by zeros when the tile is written to LDS: no branch and no register
+        // initialisation stands between the loads, so they all go out back to back.
+        const int last = min(nvalid, kBN) - 1;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int idx = tid + NT * i;
+            const int row = min(idx / G::CPR, last);
+            const int cc = idx % G::CPR;
+            if (EXACT || idx < G::NCH) reg[i] = *reinterpret_cast<const u32x4*>(base + (static_cast<unsigned>(row) * rsb + cc * 16u));
+        }
+    }
+    __device__ __forceinline__ void store_k(int t, unsigned char* Ks) {
         // The rotation tables are fetched here rather than with the tile: they are L2 hits shared by
         // every head, and holding them across the MFMA section would cost 8 registers per chunk
         // exactly where pressure peaks. Prefix rows are stored already rotated.
         f32x4 creg[ROPE_K ? NLD : 1], sreg[ROPE_K ? NLD : 1];
+        const int nvalid_k = plan.limit(t) - plan.j0(t);
+        bool rot = false;
         if constexpr (ROPE_K) {
+            rot = !plan.in_prefix(t);
+            if (rot) {
+                const int jr0 = plan.j0(t) - p.Lp;
+                const int nvalid = plan.limit(t) - plan.j0(t);
 #pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-                const int idx = tid + NT * i;
-                const int row = idx / G::CPR;
-                const int cc = idx - row * G::CPR;
-                const int j = j0 + row;
-                creg[i] = f32x4{1.f, 1.f, 1.f, 1.f};
-                sreg[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-                if ((EXACT || idx < G::NCH) && j < kv_stop && j >= p.Lp) {
-                    const long jr = j - p.Lp;
-                    creg[i] = *reinterpret_cast<const f32x4*>(p.cos_k + jr * (D / 2) + cc * 4);
-                    sreg[i] = *reinterpret_cast<const f32x4*>(p.sin_k + jr * (D / 2) + cc * 4);
+                for (int i = 0; i < NLD; ++i) {
+                    const int idx = tid + NT * i;
+                    const int row = idx / G::CPR;
+                    const int cc = idx - row * G::CPR;
+                    creg[i] = f32x4{1.f, 1.f, 1.f, 1.f};
+                    sreg[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    if ((EXACT || idx < G::NCH) && row < nvalid) {
+                        creg[i] = *reinterpret_cast<const f32x4*>(p.cos_k + static_cast<long>(jr0 + row) * (D / 2) + cc * 4);
+                        sreg[i] = *reinterpret_cast<const f32x4*>(p.sin_k + static_cast<long>(jr0 + row) * (D / 2) + cc * 4);
+                    }
                 }
             }
         }
@@ -108,18 +132,21 @@ struct TileMover {
             const int cc = idx - row * G::CPR;
             if (EXACT || idx < G::NCH) {
                 u32x4 kk = kreg[i];
-                if constexpr (ROPE_K) kk = rope_chunk<T>(kk, creg[i], sreg[i]);
+                if constexpr (ROPE_K) { if (rot) kk = rope_chunk<T>(kk, creg[i], sreg[i]); }
+                if (row >= nvalid_k) kk = u32x4{0, 0, 0, 0};
                 *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = kk;
             }
         }
     }
-    __device__ __forceinline__ void store_v(unsigned char* Vs) {
+    __device__ __forceinline__ void store_v(int t, unsigned char* Vs) {
+        const int nvalid = plan.limit(t) - plan.j0(t);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int idx = tid + NT * i;
             const int row = idx / G::CPR;
             const int cc = idx - row * G::CPR;
-            if (EXACT || idx < G::NCH) *reinterpret_cast<u32x4*>(Vs + row * G::V_STRIDE + cc * 16) = vreg[i];
+            if (EXACT || idx < G::NCH)
+                *reinterpret_cast<u32x4*>(Vs + row * G::V_STRIDE + cc * 16) = row < nvalid ? vreg[i] : u32x4{0, 0, 0, 0};
         }
     }
 };
@@ -158,7 +185,7 @@ __device__ __forceinline__ void write_output(const unsigned char* Os, T* o_base,
 constexpr int kThreads4 = 256;
 template <int D> constexpr int lds_bytes_4() {
     using G = HeadGeo<D>;
-    const int kv = 2 * (G::K_BYTES + G::V_BYTES);
+    const int kv = 2 * (G::K_BYTES + G::V_BYTES + kBN * 4);
     const int o = 128 * G::O_STRIDE;
     return kv > o ? kv : o;
 }
@@ -170,7 +197,7 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     constexpr int BM = 128;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int red[8];
-    constexpr int STAGE = G::K_BYTES + G::V_BYTES;
+    constexpr int STAGE = G::K_BYTES + G::V_BYTES + kBN * 4;   // K tile, V tile, 64 key-mask floats
 
     const int logical = logical_block(p.n_blocks);
     if (logical < 0) return;
@@ -181,7 +208,7 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;  // longest key ranges first
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
     const int lane = tid & 63;
     const int lq = lane & 31;
     const int lh = lane >> 5;
@@ -199,9 +226,9 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     if (lane == 0) { red[wave] = we.lo_min; red[4 + wave] = we.hi_max; }
     zero_pads<D, kThreads4>(smem, smem + G::K_BYTES, STAGE, STAGE, 2, tid);
     __syncthreads();
-    const int g_lo = min(min(red[0], red[1]), min(red[2], red[3]));
-    const int kv_stop = max(max(red[4], red[5]), max(red[6], red[7]));
-    const int kv_start = g_lo == 0x7fffffff ? 0 : (g_lo / kBN) * kBN;
+    const int g_lo = __builtin_amdgcn_readfirstlane(min(min(red[0], red[1]), min(red[2], red[3])));
+    const int kv_stop = __builtin_amdgcn_readfirstlane(max(max(red[4], red[5]), max(red[6], red[7])));
+    const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
 
     V8 qf[G::KC];
     load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
@@ -215,44 +242,56 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     const float cl2 = p.scale_log2;
     const float lazy_raw = kLazyLog2 / cl2;
 
-    TileMover<T, D, kThreads4, ROPE_K> mv{p,
-                                          static_cast<const T*>(p.k) + b * p.k_bs + hk * D,
-                                          static_cast<const T*>(p.v) + b * p.v_bs + hk * D,
-                                          p.kp ? static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D : nullptr,
-                                          p.vp ? static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D : nullptr,
-                                          tid, kv_stop, {}, {}};
+    TileMover<T, D, kThreads4, ROPE_K> mv{p, plan,
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D),
+                                          tid, {}, {}, 1.f};
 
     // key loop, LDS double buffered: one barrier per tile
-    if (kv_start < kv_stop) {
-        mv.template issue<0>(kv_start);
-        mv.template issue<1>(kv_start);
-        mv.store_k(kv_start, smem);
-        mv.store_v(smem + G::K_BYTES);
-        if (kv_start + kBN < kv_stop) { mv.template issue<0>(kv_start + kBN); mv.template issue<1>(kv_start + kBN); }
+    const int n_tiles = plan.n_tiles;
+    if (n_tiles > 0) {
+        mv.template issue<0>(0);
+        mv.template issue<1>(0);
+        if (key_mask) mv.issue_mask(0, key_mask);
+        mv.store_k(0, smem);
+        mv.store_v(0, smem + G::K_BYTES);
+        if (key_mask) mv.store_mask(reinterpret_cast<float*>(smem + G::K_BYTES + G::V_BYTES));
+        if (n_tiles > 1) {
+            mv.template issue<0>(1);
+            mv.template issue<1>(1);
+            if (key_mask) mv.issue_mask(1, key_mask);
+        }
     }
     __syncthreads();
-    int stage = 0;
-    for (int j0 = kv_start; j0 < kv_stop; j0 += kBN) {
-        const unsigned char* Ks = smem + stage * STAGE;
+    for (int t = 0; t < n_tiles; ++t) {
+        const unsigned char* Ks = smem + (t & 1) * STAGE;
         const unsigned char* Vs = Ks + G::K_BYTES;
+        const float* Ms = key_mask ? reinterpret_cast<const float*>(Vs + G::V_BYTES) : nullptr;
+        const int j0 = plan.j0(t);
+        const int lim = plan.limit(t);
         // wavefronts none of whose rows can see this tile only help with the loads
         if (j0 < we.hi_max && j0 + kBN > we.lo_min) {
             f32x16 sacc[2];
             V8 pf[4];
-            qk_tile<T, D>(Ks, qf, lq, lh, sacc);
-            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= we.hi_min) && (key_mask == nullptr);
-            if (interior) softmax_tile<T, D, false>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
-            else softmax_tile<T, D, true>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
-            pv_tile<T, D>(Vs, pf, lane, oacc);
+            mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
+            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim)) && (key_mask == nullptr);
+            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, Ms);
+            mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
         }
-        if (j0 + kBN < kv_stop) {
-            unsigned char* Kn = smem + (stage ^ 1) * STAGE;
-            mv.store_k(j0 + kBN, Kn);
-            mv.store_v(Kn + G::K_BYTES);
+        if (t + 1 < n_tiles) {
+            unsigned char* Kn = smem + ((t + 1) & 1) * STAGE;
+            mv.store_k(t + 1, Kn);
+            mv.store_v(t + 1, Kn + G::K_BYTES);
+            if (key_mask) mv.store_mask(reinterpret_cast<float*>(Kn + G::K_BYTES + G::V_BYTES));
         }
-        if (j0 + 2 * kBN < kv_stop) { mv.template issue<0>(j0 + 2 * kBN); mv.template issue<1>(j0 + 2 * kBN); }
+        if (t + 2 < n_tiles) {
+            mv.template issue<0>(t + 2);
+            mv.template issue<1>(t + 2);
+            if (key_mask) mv.issue_mask(t + 2, key_mask);
+        }
         __syncthreads();
-        stage ^= 1;
     }
 
     const float l_tot = exchange_sum(st.l);
@@ -273,12 +312,14 @@ template <int D> constexpr int lds_bytes_8() {
 
 // Time is counted in slots separated by work-group barriers. Group 0 (wavefronts 0-3) runs its MFMA
 // phase in even slots and its VALU phase in odd slots; group 1 (wavefronts 4-7, sharing the SIMDs of
-// 0-3) the other way round. With t = slot / 2:
-//   MFMA phase:  O += V_t^T P_t ;  S_{t+1} = K_{t+1} Q^T           (reads LDS tiles K_{t+1}, V_t)
-//   VALU phase:  P = softmax(S) of the tile just scored; store this thread's share of tiles
-//                K_{t+2}, V_{t+1} into the LDS buffers of K_t, V_{t-1}; issue the next global loads
-// Tiles K_{t+1}, V_t are complete in LDS before slot 2t and last read in slot 2t+1, and the buffers
-// they replace were last read in slot 2t-1, so two buffers per operand suffice.
+// 0-3) the other way round. With t = slot / 2 (the first iteration, t = -1, has no P yet and only
+// scores tile 0):
+//   MFMA phase:  O += V_t^T P_t ;  S_{t+1} = K_{t+1} Q^T   (reads LDS tiles V_t, K_{t+1}); in its
+//                shadow the wavefront stores its share of tiles K_{t+2}, V_{t+1} into the LDS buffers
+//                of K_t, V_{t-1} and issues the global loads of K_{t+3}, V_{t+2}
+//   VALU phase:  P_{t+1} = softmax(S_{t+1})
+// Tiles K_{t+1}, V_t are complete in LDS before slot 2t and last read in slot 2t+1; the buffers
+// written in slots 2t and 2t+1 were last read in slot 2t-1, so two buffers per operand suffice.
 template <typename T, int D, bool ROPE_K>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev p) {
     using G = HeadGeo<D>;
@@ -298,7 +339,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;  // longest key ranges first
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
     const int grp = wave >> 2;      // phase group
     const int lane = tid & 63;
     const int lq = lane & 31;
@@ -309,19 +350,23 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     const int hk = h / p.kv_group;
     const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
-    const float* const key_mask = p.key_mask ? p.key_mask + b * p.key_mask_bs : nullptr;
 
     int lo, hi;
     row_interval(p, b, qrow, qvalid, lo, hi);
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    // K pad columns must be zero; the V buffers are zeroed whole because the first pass through the
+    // MFMA stream multiplies a zero P with whatever the second V buffer holds
     zero_pads<D, kThreads8>(Kbuf, Vbuf, G::K_BYTES, G::V_BYTES, 2, tid);
+    for (int i = tid; i < 2 * G::V_BYTES / 16; i += kThreads8) *reinterpret_cast<u32x4*>(Vbuf + i * 16) = u32x4{0, 0, 0, 0};
     __syncthreads();
     int g_lo = red[0], kv_stop = red[8];
 #pragma unroll
     for (int w = 1; w < 8; ++w) { g_lo = min(g_lo, red[w]); kv_stop = max(kv_stop, red[8 + w]); }
-    const int kv_start = g_lo == 0x7fffffff ? 0 : (g_lo / kBN) * kBN;
-    const int n_tiles = kv_stop > kv_start ? (kv_stop - kv_start + kBN - 1) / kBN : 0;
+    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
+    kv_stop = __builtin_amdgcn_readfirstlane(kv_stop);
+    const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
+    const int n_tiles = plan.n_tiles;
 
     V8 qf[G::KC];
     load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
@@ -335,60 +380,115 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     const float cl2 = p.scale_log2;
     const float lazy_raw = kLazyLog2 / cl2;
 
-    TileMover<T, D, kThreads8, ROPE_K> mv{p,
-                                          static_cast<const T*>(p.k) + b * p.k_bs + hk * D,
-                                          static_cast<const T*>(p.v) + b * p.v_bs + hk * D,
-                                          p.kp ? static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D : nullptr,
-                                          p.vp ? static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D : nullptr,
-                                          tid, kv_stop, {}, {}};
-    auto tile_j0 = [&](int t) { return kv_start + t * kBN; };
-    auto tile_active = [&](int t) { return t < n_tiles && tile_j0(t) < we.hi_max && tile_j0(t) + kBN > we.lo_min; };
+    TileMover<T, D, kThreads8, ROPE_K> mv{p, plan,
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D),
+                                          tid, {}, {}, 1.f};
+    auto tile_active = [&](int t) {
+        if (t < 0 || t >= n_tiles) return false;
+        const int j0 = plan.j0(t);
+        return j0 < we.hi_max && j0 + kBN > we.lo_min;
+    };
     // this thread's share of tiles K_kt, V_vt: registers -> LDS, then prefetch K_{kt+1}, V_{vt+1}
+#ifdef MI_EXPERIMENT_TIMING
+    unsigned long long tmv[4] = {0, 0, 0, 0};
+#endif
     auto advance_tiles = [&](int kt, int vt) {
-        if (kt < n_tiles) mv.store_k(tile_j0(kt), Kbuf + (kt & 1) * G::K_BYTES);
-        if (vt < n_tiles) mv.store_v(Vbuf + (vt & 1) * G::V_BYTES);
-        if (kt + 1 < n_tiles) mv.template issue<0>(tile_j0(kt + 1));
-        if (vt + 1 < n_tiles) mv.template issue<1>(tile_j0(vt + 1));
+#ifdef MI_EXPERIMENT_TIMING
+        unsigned long long a0 = __builtin_readcyclecounter();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned long long a1 = __builtin_readcyclecounter();
+#endif
+#ifndef MI_EXPERIMENT_NO_LDS_STORE
+        if (kt < n_tiles) mv.store_k(kt, Kbuf + (kt & 1) * G::K_BYTES);
+        if (vt < n_tiles) mv.store_v(vt, Vbuf + (vt & 1) * G::V_BYTES);
+#endif
+#ifdef MI_EXPERIMENT_TIMING
+        unsigned long long a2 = __builtin_readcyclecounter();
+#endif
+#ifndef MI_EXPERIMENT_NO_GLOBAL_LOAD
+        if (kt + 1 < n_tiles) mv.template issue<0>(kt + 1);
+        if (vt + 1 < n_tiles) mv.template issue<1>(vt + 1);
+#endif
+#ifdef MI_EXPERIMENT_TIMING
+        unsigned long long a3 = __builtin_readcyclecounter();
+        tmv[0] += a1 - a0; tmv[1] += a2 - a1; tmv[2] += a3 - a2;
+#endif
     };
     f32x16 sacc[2];
     V8 pf[4];
-    auto softmax_of = [&](int t) {
-        const int j0 = tile_j0(t);
-        const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= we.hi_min) && (key_mask == nullptr);
-        if (interior) softmax_tile<T, D, false>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
-        else softmax_tile<T, D, true>(sacc, pf, oacc, st, cl2, lazy_raw, j0, lo, hi, lh, key_mask, p.Lk);
-    };
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
 
     if (n_tiles > 0) {
-        // ── prologue, both groups in step: K_0 to LDS, score and exponentiate tile 0 ──
-        mv.template issue<0>(tile_j0(0));
-        mv.store_k(tile_j0(0), Kbuf);
-        if (n_tiles > 1) mv.template issue<0>(tile_j0(1));
-        mv.template issue<1>(tile_j0(0));
+        // ── prologue: K_0 into LDS; registers then hold K_1, V_0 ──
+        mv.template issue<0>(0);
+        mv.store_k(0, Kbuf);
+        if (n_tiles > 1) mv.template issue<0>(1);
+        mv.template issue<1>(0);
         __syncthreads();
-        if (tile_active(0)) {
-            qk_tile<T, D>(Kbuf, qf, lq, lh, sacc);
-            softmax_of(0);
-        }
-        advance_tiles(1, 0);   // K_1, V_0 to LDS; registers now hold K_2, V_1
-        __syncthreads();
-        // ── group 1 falls one slot behind: its first slot only moves tiles ──
-        if (grp == 1) {
-            advance_tiles(2, 1);
-            __syncthreads();
-        }
-        for (int t = 0; t < n_tiles; ++t) {
+        // ── group 1 falls one slot behind ──
+        if (grp == 1) __syncthreads();
+#ifdef MI_EXPERIMENT_TIMING
+        unsigned long long tm[6] = {0, 0, 0, 0, 0, 0}, tc0, tc1;
+#define MI_TICK(i) tc1 = __builtin_readcyclecounter(); tm[i] += tc1 - tc0; tc0 = tc1;
+        tc0 = __builtin_readcyclecounter();
+#else
+#define MI_TICK(i)
+#endif
+        // iteration -1 only scores tile 0 (there is no P yet)
+        for (int t = -1; t < n_tiles; ++t) {
             // MFMA phase
+#ifndef MI_EXPERIMENT_NO_SETPRIO
             __builtin_amdgcn_s_setprio(2);
-            if (tile_active(t)) pv_tile<T, D>(Vbuf + (t & 1) * G::V_BYTES, pf, lane, oacc);
-            if (tile_active(t + 1)) qk_tile<T, D>(Kbuf + ((t + 1) & 1) * G::K_BYTES, qf, lq, lh, sacc);
+#endif
+#ifndef MI_EXPERIMENT_NO_MFMA
+            // Always the full stream: at t = -1 P is zero and the (zero-filled) V buffer adds nothing;
+            // after the last tile the extra scores are never read. This wavefront's share of the tile
+            // movement rides along in the stream, where the VALU and memory ports are otherwise idle.
+            mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
+#ifdef MI_EXPERIMENT_NO_TILE_MOVES
+                                          NoMid());
+#else
+                                          [&]() { advance_tiles(t + 2, t + 1); });
+#endif
+#endif
+#ifndef MI_EXPERIMENT_NO_SETPRIO
             __builtin_amdgcn_s_setprio(0);
+#endif
+            MI_TICK(0)
             __syncthreads();
+            MI_TICK(1)
             // VALU phase
-            if (tile_active(t + 1)) softmax_of(t + 1);
-            advance_tiles(t + 2 + grp, t + 1 + grp);
+#ifndef MI_EXPERIMENT_NO_SOFTMAX
+            if (tile_active(t + 1)) {
+                const int j0 = plan.j0(t + 1);
+                const int lim = plan.limit(t + 1);
+                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
+                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
+            } else {
+                // nothing visible to this wavefront in that tile: the next PV pass must add zero
+#pragma unroll
+                for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+            }
+#endif
+            MI_TICK(2)
+            MI_TICK(3)
             __syncthreads();
+            MI_TICK(4)
         }
+#ifdef MI_EXPERIMENT_TIMING
+        if (lane == 0 && blockIdx.x < 64) {
+            unsigned long long* dbg = reinterpret_cast<unsigned long long*>(const_cast<float*>(p.cos_k));  // experiment only: buffer passed in the cos_k slot
+            for (int i = 0; i < 6; ++i) dbg[(blockIdx.x * 8 + wave) * 8 + i] = tm[i];
+            dbg[(blockIdx.x * 8 + wave) * 8 + 6] = n_tiles + 1;
+            dbg[(blockIdx.x * 8 + wave) * 8 + 3] = tmv[0];   // wait for the loads
+            dbg[(blockIdx.x * 8 + wave) * 8 + 5] = tmv[1];   // LDS stores
+            dbg[(blockIdx.x * 8 + wave) * 8 + 7] = tmv[2];   // issue
+        }
+#endif
         if (grp == 0) __syncthreads();
     }
 
@@ -401,12 +501,17 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
 
 template <typename T, int D>
 int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
+#ifdef MI_EXPERIMENT_TIMING
+    const bool rope_k = false;  // the cos_k slot carries the timing buffer in this build
+#else
     const bool rope_k = p.cos_k != nullptr;
+#endif
     // 256-row tiles when they give every CU at least one work group; head_dim above 128 does not fit
     // two wavefronts per SIMD and stays on the 128-row kernel.
     const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int choice = sdpa_kernel_choice();
-    const bool pingpong = D <= 128 && (choice == 2 || (choice == 0 && tiles256 >= n_cu));
+    // calls with a key mask stay on the 128-row kernel, which stages the mask tile in LDS
+    const bool pingpong = D <= 128 && p.key_mask == nullptr && (choice == 2 || (choice == 0 && tiles256 >= n_cu));
     if (pingpong) {
         p.n_q_tiles = (p.Lq + 255) / 256;
         p.n_blocks = static_cast<int>(tiles256);
