@@ -51,6 +51,7 @@ class MiSdpaArgs(C.Structure):
         ("seg_q_end", C.c_int32 * MI_MAX_SEGMENTS), ("seg_k_end", C.c_int32 * MI_MAX_SEGMENTS),
         ("seg_causal", C.c_int32 * MI_MAX_SEGMENTS),
         ("rope_cos_q", C.c_void_p), ("rope_sin_q", C.c_void_p), ("rope_cos_k", C.c_void_p), ("rope_sin_k", C.c_void_p),
+        ("rope_k_scratch", C.c_void_p),
         ("stream", C.c_void_p),
     ]
 

@@ -98,7 +98,8 @@ int mi_memset_async(void* dst, int value, size_t bytes, void* stream) {
 
 int mi_sdpa_set_kernel_choice(int32_t choice) {
     mi::clear_error();
-    if (choice < 0 || choice > 2) return fail("mi_sdpa_set_kernel_choice: 0 (auto), 1 (128-row tiles) or 2 (256-row ping-pong)");
+    if (choice < 0 || choice > 3)
+        return fail("mi_sdpa_set_kernel_choice: 0 (auto), 1 (128-row tiles), 2 (256-row ping-pong) or 3 (ping-pong, register-staged tiles)");
     mi::g_kernel_choice = choice;
     return 0;
 }
@@ -182,6 +183,27 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
     for (const void* t : tabs)
         if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
     p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
+    if (p.cos_k && a->rope_k_scratch && a->kv_len > 0) {
+        // K is rotated once into the caller's scratch (a pure HBM pass) and the attention kernel reads the
+        // rotated copy: the LDS-DMA tile path stays usable and no work group repeats the rotation.
+        if (!mi::aligned16(a->rope_k_scratch)) return fail("mi_sdpa_forward: rope_k_scratch must be 16-byte aligned");
+        const size_t esz = 2;
+        for (int b = 0; b < a->batch; ++b) {
+            mi_rope_args r;
+            std::memset(&r, 0, sizeof(r));
+            r.struct_size = sizeof(r);
+            r.dtype = a->dtype;
+            r.x = static_cast<const char*>(a->k) + static_cast<size_t>(b) * p.k_bs * esz;
+            r.out = static_cast<char*>(a->rope_k_scratch) + static_cast<size_t>(b) * a->kv_len * Dkv * esz;
+            r.cos = p.cos_k; r.sin = p.sin_k;
+            r.rows = a->kv_len; r.num_heads = Hkv; r.head_dim = a->head_dim;
+            r.x_row_stride = p.k_rs; r.out_row_stride = Dkv;
+            r.stream = mi::resolve_stream(a->stream);
+            if (mi_rope_apply(&r) != 0) return -1;
+        }
+        p.k = a->rope_k_scratch; p.k_rs = Dkv; p.k_bs = Dkv * a->kv_len;
+        p.cos_k = nullptr; p.sin_k = nullptr;
+    }
     const long nb = static_cast<long>(a->batch) * a->num_heads * ((a->q_len + 127) / 128);
     if (nb > 0x3fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
     return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));

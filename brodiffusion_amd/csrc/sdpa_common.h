@@ -163,11 +163,7 @@ __device__ __forceinline__ void load_q_frags(typename Mma<T>::v8 (&qf)[HeadGeo<D
 //     row j/4, and lane i receives 4 consecutive keys of head-dim column i).
 //   QK operand (kb, c):  K fragment = key block kb x 16 head-dim elements, one 16-byte read per lane.
 constexpr int kAhead = 4;
-#ifdef MI_EXPERIMENT_NO_SCHED_BARRIER
-#define MI_SCHED_BARRIER
-#else
 #define MI_SCHED_BARRIER __builtin_amdgcn_sched_barrier(0);
-#endif
 
 // `mid` is called once, a few MFMAs into the stream: work placed there (tile movement) issues in
 // the shadow of the matrix pipe.
@@ -295,13 +291,8 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
     float lsum0 = 0.f, lsum1 = 0.f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-#ifdef MI_EXPERIMENT_NO_EXP
-        const float p0 = __builtin_fmaf(sacc[0][e], cl2, -st.mc);
-        const float p1 = __builtin_fmaf(sacc[1][e], cl2, -st.mc);
-#else
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[0][e], cl2, -st.mc));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[1][e], cl2, -st.mc));
-#endif
         sacc[0][e] = p0;
         sacc[1][e] = p1;
         lsum0 += p0;

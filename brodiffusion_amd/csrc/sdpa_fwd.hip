@@ -14,6 +14,8 @@
 // registers). Not in HBM: scores, probabilities, rotated Q/K (RoPE is applied as Q and K are loaded),
 // the [prefix ; fresh] K/V concatenation (two source pointers), any mask tensor (per-row visible-key
 // intervals; key tiles outside every row's interval are skipped).
+#include <type_traits>
+
 #include "sdpa_common.h"
 
 namespace mi {
@@ -392,30 +394,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         return j0 < we.hi_max && j0 + kBN > we.lo_min;
     };
     // this thread's share of tiles K_kt, V_vt: registers -> LDS, then prefetch K_{kt+1}, V_{vt+1}
-#ifdef MI_EXPERIMENT_TIMING
-    unsigned long long tmv[4] = {0, 0, 0, 0};
-#endif
     auto advance_tiles = [&](int kt, int vt) {
-#ifdef MI_EXPERIMENT_TIMING
-        unsigned long long a0 = __builtin_readcyclecounter();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        unsigned long long a1 = __builtin_readcyclecounter();
-#endif
-#ifndef MI_EXPERIMENT_NO_LDS_STORE
         if (kt < n_tiles) mv.store_k(kt, Kbuf + (kt & 1) * G::K_BYTES);
         if (vt < n_tiles) mv.store_v(vt, Vbuf + (vt & 1) * G::V_BYTES);
-#endif
-#ifdef MI_EXPERIMENT_TIMING
-        unsigned long long a2 = __builtin_readcyclecounter();
-#endif
-#ifndef MI_EXPERIMENT_NO_GLOBAL_LOAD
         if (kt + 1 < n_tiles) mv.template issue<0>(kt + 1);
         if (vt + 1 < n_tiles) mv.template issue<1>(vt + 1);
-#endif
-#ifdef MI_EXPERIMENT_TIMING
-        unsigned long long a3 = __builtin_readcyclecounter();
-        tmv[0] += a1 - a0; tmv[1] += a2 - a1; tmv[2] += a3 - a2;
-#endif
     };
     f32x16 sacc[2];
     V8 pf[4];
@@ -431,38 +414,18 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         __syncthreads();
         // ── group 1 falls one slot behind ──
         if (grp == 1) __syncthreads();
-#ifdef MI_EXPERIMENT_TIMING
-        unsigned long long tm[6] = {0, 0, 0, 0, 0, 0}, tc0, tc1;
-#define MI_TICK(i) tc1 = __builtin_readcyclecounter(); tm[i] += tc1 - tc0; tc0 = tc1;
-        tc0 = __builtin_readcyclecounter();
-#else
-#define MI_TICK(i)
-#endif
         // iteration -1 only scores tile 0 (there is no P yet)
         for (int t = -1; t < n_tiles; ++t) {
             // MFMA phase
-#ifndef MI_EXPERIMENT_NO_SETPRIO
             __builtin_amdgcn_s_setprio(2);
-#endif
-#ifndef MI_EXPERIMENT_NO_MFMA
             // Always the full stream: at t = -1 P is zero and the (zero-filled) V buffer adds nothing;
             // after the last tile the extra scores are never read. This wavefront's share of the tile
             // movement rides along in the stream, where the VALU and memory ports are otherwise idle.
             mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
-#ifdef MI_EXPERIMENT_NO_TILE_MOVES
-                                          NoMid());
-#else
                                           [&]() { advance_tiles(t + 2, t + 1); });
-#endif
-#endif
-#ifndef MI_EXPERIMENT_NO_SETPRIO
             __builtin_amdgcn_s_setprio(0);
-#endif
-            MI_TICK(0)
             __syncthreads();
-            MI_TICK(1)
             // VALU phase
-#ifndef MI_EXPERIMENT_NO_SOFTMAX
             if (tile_active(t + 1)) {
                 const int j0 = plan.j0(t + 1);
                 const int lim = plan.limit(t + 1);
@@ -473,22 +436,276 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
             }
-#endif
-            MI_TICK(2)
-            MI_TICK(3)
             __syncthreads();
-            MI_TICK(4)
         }
-#ifdef MI_EXPERIMENT_TIMING
-        if (lane == 0 && blockIdx.x < 64) {
-            unsigned long long* dbg = reinterpret_cast<unsigned long long*>(const_cast<float*>(p.cos_k));  // experiment only: buffer passed in the cos_k slot
-            for (int i = 0; i < 6; ++i) dbg[(blockIdx.x * 8 + wave) * 8 + i] = tm[i];
-            dbg[(blockIdx.x * 8 + wave) * 8 + 6] = n_tiles + 1;
-            dbg[(blockIdx.x * 8 + wave) * 8 + 3] = tmv[0];   // wait for the loads
-            dbg[(blockIdx.x * 8 + wave) * 8 + 5] = tmv[1];   // LDS stores
-            dbg[(blockIdx.x * 8 + wave) * 8 + 7] = tmv[2];   // issue
+        if (grp == 0) __syncthreads();
+    }
+
+    const float l_tot = exchange_sum(st.l);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
+    __syncthreads();
+    write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+}
+
+// ─────────────── 8-wavefront ping-pong kernel, head_dim 128, tiles by LDS DMA ───────────────
+// Same schedule as sdpa_fwd_pp_kernel, but K/V tiles go from global memory straight into LDS
+// (global_load_lds_dwordx4: lane i of a wavefront deposits its 16 bytes at base + 16*i), so tile
+// movement costs no registers, no LDS store instructions and no wait inside the MFMA stream.
+// A DMA instruction writes 1024 contiguous bytes = 4 unpadded 256-byte rows, so bank conflicts are
+// avoided by an XOR swizzle instead of row padding: 16-byte chunk c of row r lives at chunk position
+// c ^ f(r), f(r) = 4*(r%4) + (r/4)%4. The swizzle is applied for free on the global side (each lane
+// fetches the chunk that belongs in its LDS slot) and undone in the LDS read addresses:
+//   K reads (one row per lane, 16 consecutive rows): f takes 16 distinct values -> 16 distinct slots
+//   V transpose reads (4 rows x 64 bytes per 32 lanes): rows r%4 = 0..3 land in distinct 64-byte windows
+// Tiles are ring-buffered three deep: the loads of K_{t+3}, V_{t+2} are issued during MFMA phase t
+// and awaited at the end of the following VALU phase, two phases later. The key loop is unrolled by
+// three so that every LDS offset is an instruction immediate.
+// A wavefront issues at most one instruction every 4 clocks, so instruction count is what the phases
+// cost: tile pointers advance incrementally in scalar registers, and the four DMA instructions of a
+// step are spread between the first MFMAs instead of being issued in one lump.
+// Rows past the end of a segment are fetched from its last row (valid memory); their scores are masked.
+constexpr int kDmaStages = 3;
+constexpr int kRowBytes128 = 256;
+constexpr int kTileBytes128 = kBN * kRowBytes128;   // 16 KB per operand tile
+constexpr int kVbufOff128 = kDmaStages * kTileBytes128;
+constexpr int lds_bytes_dma() {
+    const int kv = 2 * kDmaStages * kTileBytes128;
+    const int o = 256 * HeadGeo<128>::O_STRIDE;
+    return kv > o ? kv : o;
+}
+
+__device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2) & 3); }
+
+// Walks the tiles of one operand (K or V) in order, keeping the tile's base pointer, row stride and
+// the number of rows left in the current segment (prefix, then fresh) in scalar registers.
+struct TileCursor {
+    const unsigned char* ptr;     // first row of the current tile
+    unsigned rsb;                 // row stride in bytes
+    int rows_left;                // rows of the segment from the current tile on
+    int t;                        // index of the current tile
+    // fresh segment, entered when t reaches n_pre
+    const unsigned char* fresh_ptr;
+    unsigned fresh_rsb;
+    int fresh_rows, n_pre;
+    __device__ __forceinline__ void init(const TilePlan& plan, const unsigned char* pre_base, unsigned pre_rsb,
+                                         const unsigned char* fr_base, unsigned fr_rsb, int Lp) {
+        fresh_ptr = fr_base + static_cast<unsigned long>(plan.fr_lo - Lp) * fr_rsb;
+        fresh_rsb = fr_rsb;
+        fresh_rows = plan.fr_hi - plan.fr_lo;
+        n_pre = plan.n_pre;
+        t = 0;
+        if (n_pre > 0) { ptr = pre_base + static_cast<unsigned long>(plan.pre_lo) * pre_rsb; rsb = pre_rsb; rows_left = plan.pre_hi - plan.pre_lo; }
+        else { ptr = fresh_ptr; rsb = fresh_rsb; rows_left = fresh_rows; }
+    }
+    __device__ __forceinline__ void next() {
+        ++t;
+        if (t == n_pre) { ptr = fresh_ptr; rsb = fresh_rsb; rows_left = fresh_rows; }
+        else { ptr += kBN * rsb; rows_left -= kBN; }
+    }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const SdpaDev p) {
+    constexpr int D = 128;
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    constexpr int BM = 256;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ int red[16];
+
+    const int logical = logical_block(p.n_blocks);
+    if (logical < 0) return;
+    int qt = logical % p.n_q_tiles;
+    const int bh = logical / p.n_q_tiles;
+    const int h = bh % p.H;
+    const int b = bh / p.H;
+    if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2;
+    const int lane = tid & 63;
+    const int lq = lane & 31;
+    const int lh = lane >> 5;
+    const int q0 = qt * BM;
+    const int qrow = q0 + wave * 32 + lq;
+    const bool qvalid = qrow < p.Lq;
+    const int hk = h / p.kv_group;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+
+    int lo, hi;
+    row_interval(p, b, qrow, qvalid, lo, hi);
+    const WaveExtent we = wave_extent(lo, hi);
+    if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    // the first pass through the MFMA stream multiplies a zero P with the last V buffer
+    for (int i = tid; i < kTileBytes128 / 16; i += kThreads8)
+        *reinterpret_cast<u32x4*>(smem + kVbufOff128 + (kDmaStages - 1) * kTileBytes128 + i * 16) = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    int g_lo = red[0], kv_stop = red[8];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) { g_lo = min(g_lo, red[w]); kv_stop = max(kv_stop, red[8 + w]); }
+    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
+    kv_stop = __builtin_amdgcn_readfirstlane(kv_stop);
+    const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
+    const int n_tiles = plan.n_tiles;
+
+    V8 qf[G::KC];
+    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
+    f32x16 oacc[G::VB];
+#pragma unroll
+    for (int vb = 0; vb < G::VB; ++vb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
+    SoftmaxState st;
+    const float cl2 = p.scale_log2;
+    const float lazy_raw = kLazyLog2 / cl2;
+
+    // ── DMA source geometry of this lane: LDS slot (row 4*wave + lane/16 [+32], position lane%16) ──
+    TileCursor kc, vc;
+    kc.init(plan, reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D), static_cast<unsigned>(p.kp_rs) * 2u,
+            reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D), static_cast<unsigned>(p.k_rs) * 2u, p.Lp);
+    vc.init(plan, reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D), static_cast<unsigned>(p.vp_rs) * 2u,
+            reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D), static_cast<unsigned>(p.v_rs) * 2u, p.Lp);
+    const int drow = 4 * wave + (lane >> 4);
+    const unsigned dchunk = ((lane & 15) ^ swz(drow)) * 16u;   // chunk this slot must receive (same for row + 32)
+    // One DMA instruction: rows (drow + 32*half) of the cursor's tile into LDS at lds_off + 1024*wave + 8192*half.
+    // Written as inline assembly on purpose: for the compiler's builtin every later LDS read may alias
+    // the DMA's LDS write, so it waits for the load to land (vmcnt(0)) before the next ds_read and the
+    // whole memory latency ends up inside the MFMA stream. The tiles written here are never read before
+    // the explicit wait + barrier at the end of the following VALU phase.
+    const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)smem));
+    auto dma = [&](const TileCursor& c, int half, int lds_off) {
+        const int row = min(drow + 32 * half, min(c.rows_left, kBN) - 1);
+        const unsigned voff = static_cast<unsigned>(row) * c.rsb + dchunk;
+        const unsigned dst = lds_base + lds_off + wave * 1024 + half * 8192;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory");
+    };
+
+    // ── LDS read addresses in the swizzled layout (stage and block offsets are immediates) ──
+    // K fragment (kb, c): row 32kb + lq, chunk 2c + lh  ->  position (2c + lh) ^ f(lq)
+    const int fk = swz(lq);
+    unsigned kaddr[G::KC];
+#pragma unroll
+    for (int c = 0; c < G::KC; ++c) kaddr[c] = lq * kRowBytes128 + (((2 * c + lh) ^ fk) << 4);
+    // V fragment (c4, vb), halves hh = 0, 1: key row 16c4 + 4lh + 8hh + trow, 8 bytes at head-dim 32vb + tcol
+    const int trow = (lane & 15) >> 2;
+    const int j4 = lane & 3;
+    const int g1 = (lane >> 4) & 1;
+    unsigned vaddr[G::VB][2];
+#pragma unroll
+    for (int vb = 0; vb < G::VB; ++vb)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const int row = 4 * lh + 8 * hh + trow;
+            const int chunk = 4 * vb + 2 * g1 + (j4 >> 1);
+            vaddr[vb][hh] = kVbufOff128 + row * kRowBytes128 + ((chunk ^ swz(row)) << 4) + 8 * (j4 & 1);
         }
-#endif
+
+    f32x16 sacc[2];
+    V8 pf[4];
+#pragma unroll
+    for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+
+    auto tile_active = [&](int t) {
+        if (t < 0 || t >= n_tiles) return false;
+        const int j0 = plan.j0(t);
+        return j0 < we.hi_max && j0 + kBN > we.lo_min;
+    };
+
+    // One step t of the loop with S = (t + 1) % 3 known at compile time:
+    //   reads K_{t+1} from K stage S and V_t from V stage (S + 2) % 3,
+    //   loads K_{t+3} into K stage (S + 2) % 3 and V_{t+2} into V stage (S + 1) % 3.
+    auto step = [&](auto stage_tag, int t) {
+        constexpr int S = decltype(stage_tag)::value;
+        constexpr int KS = S * kTileBytes128, VS = ((S + 2) % 3) * kTileBytes128;
+        constexpr int KD = ((S + 2) % 3) * kTileBytes128, VD = kVbufOff128 + ((S + 1) % 3) * kTileBytes128;
+        const bool load_k = t + 3 < n_tiles, load_v = t + 2 < n_tiles;
+        // ── MFMA phase ──
+        __builtin_amdgcn_s_setprio(2);
+        {
+            constexpr int NPV = 4 * G::VB, N = NPV + 2 * G::KC;
+            auto fetch = [&](int i) -> V8 {
+                if (i < NPV) {
+                    const int c4 = i / G::VB, vb = i % G::VB;
+                    const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * kRowBytes128 + vaddr[vb][0]));
+                    const s16x4 v_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * kRowBytes128 + vaddr[vb][1]));
+                    const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    return __builtin_bit_cast(V8, a);
+                } else {
+                    const int k = i - NPV;
+                    const int kb = k / G::KC, c = k % G::KC;
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * kRowBytes128 + kaddr[c]);
+                    return __builtin_bit_cast(V8, a);
+                }
+            };
+            V8 ring[kAhead];
+#pragma unroll
+            for (int i = 0; i < kAhead; ++i) ring[i] = fetch(i);
+#pragma unroll
+            for (int i = 0; i < N; ++i) {
+                const V8 a = ring[i % kAhead];
+                if (i < NPV) {
+                    const int c4 = i / G::VB, vb = i % G::VB;
+                    oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
+                } else {
+                    const int k = i - NPV;
+                    const int kb = k / G::KC, c = k % G::KC;
+                    if (c == 0) {
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        sacc[kb] = Mma<T>::run(a, qf[c], zero);
+                    } else {
+                        sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
+                    }
+                }
+                if (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
+                MI_SCHED_BARRIER
+                // the four DMA instructions of this step, one behind each of MFMAs 1, 3, 5, 7
+                if (i == 1 && load_k) dma(kc, 0, KD);
+                if (i == 3 && load_k) dma(kc, 1, KD);
+                if (i == 5 && load_v) dma(vc, 0, VD);
+                if (i == 7 && load_v) dma(vc, 1, VD);
+                if (i == 1 || i == 3 || i == 5 || i == 7) { MI_SCHED_BARRIER }
+            }
+        }
+        __builtin_amdgcn_s_setprio(0);
+        if (load_k) kc.next();
+        if (load_v) vc.next();
+        __syncthreads();
+        // ── VALU phase ──
+        if (tile_active(t + 1)) {
+            const int j0 = plan.j0(t + 1);
+            const int lim = plan.limit(t + 1);
+            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
+            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
+        } else {
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's tile loads have landed
+        __syncthreads();
+    };
+
+    if (n_tiles > 0) {
+        // prologue: K_0, K_1, V_0 (the loop loads K_{t+3}, V_{t+2} from t = -1 on); cursors end at K_2, V_1
+        dma(kc, 0, 0); dma(kc, 1, 0);
+        if (n_tiles > 1) { kc.next(); dma(kc, 0, kTileBytes128); dma(kc, 1, kTileBytes128); }
+        if (n_tiles > 2) kc.next();
+        dma(vc, 0, kVbufOff128); dma(vc, 1, kVbufOff128);
+        if (n_tiles > 1) vc.next();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (grp == 1) __syncthreads();   // group 1 falls one slot behind
+        for (int t = -1; t < n_tiles; t += 3) {
+            step(std::integral_constant<int, 0>{}, t);
+            if (t + 1 >= n_tiles) break;
+            step(std::integral_constant<int, 1>{}, t + 1);
+            if (t + 2 >= n_tiles) break;
+            step(std::integral_constant<int, 2>{}, t + 2);
+        }
         if (grp == 0) __syncthreads();
     }
 
@@ -501,23 +718,20 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
 
 template <typename T, int D>
 int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
-#ifdef MI_EXPERIMENT_TIMING
-    const bool rope_k = false;  // the cos_k slot carries the timing buffer in this build
-#else
     const bool rope_k = p.cos_k != nullptr;
-#endif
     // 256-row tiles when they give every CU at least one work group; head_dim above 128 does not fit
     // two wavefronts per SIMD and stays on the 128-row kernel.
     const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int choice = sdpa_kernel_choice();
     // calls with a key mask stay on the 128-row kernel, which stages the mask tile in LDS
-    const bool pingpong = D <= 128 && p.key_mask == nullptr && (choice == 2 || (choice == 0 && tiles256 >= n_cu));
+    const bool pingpong = D <= 128 && p.key_mask == nullptr && (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
     if (pingpong) {
         p.n_q_tiles = (p.Lq + 255) / 256;
         p.n_blocks = static_cast<int>(tiles256);
         const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads8);
         if constexpr (D <= 128) {
             if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
+            else if (D == 128 && sdpa_kernel_choice() != 3) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T>), grid, block, lds_bytes_dma(), stream, p);
             else hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false>), grid, block, lds_bytes_8<D>(), stream, p);
         }
     } else {

@@ -167,7 +167,7 @@ RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, co
 }
 
 void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin, int head_dim,
-                     int num_heads, Tensor& out, Tensor& /*Qr*/, Tensor& /*Kr*/) {
+                     int num_heads, Tensor& out, Tensor& /*Qr*/, Tensor& Kr) {
     const char* op = "joint_attention";
     if (head_dim <= 0 || num_heads <= 0 || Q.cols != head_dim * num_heads) fail(std::string(op) + ": D must equal head_dim * num_heads");
     if (K.rows != Q.rows || V.rows != Q.rows || K.cols != Q.cols || V.cols != Q.cols) fail(std::string(op) + ": Q/K/V must share shape (L, D)");
@@ -175,11 +175,13 @@ void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Te
     init_args(a, op, Q, K, V, num_heads, num_heads, out);
     set_rope(a, op, &cos, &sin, Q.rows, true);
     set_rope(a, op, &cos, &sin, K.rows, false);
+    Kr.resize(K.rows, K.cols, K.dtype, K.device);  // receives RoPE(K), as in the reference
+    a.rope_k_scratch = Kr.data;
     check(op, mi_sdpa_forward(&a));
 }
 
 void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin, int head_dim,
-                          int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out, Tensor& /*Qr*/, Tensor& /*Kr*/,
+                          int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out, Tensor& /*Qr*/, Tensor& Kr,
                           Tensor& /*Krep*/, Tensor& /*Vrep*/) {
     const char* op = "gqa_attention_masked";
     if (num_kv_heads <= 0 || num_q_heads <= 0 || num_q_heads % num_kv_heads != 0)
@@ -190,6 +192,10 @@ void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, con
     a.key_mask = d_mask;
     set_rope(a, op, cos, sin, Q.rows, true);
     set_rope(a, op, cos, sin, K.rows, false);
+    if (cos) {
+        Kr.resize(K.rows, K.cols, K.dtype, K.device);
+        a.rope_k_scratch = Kr.data;
+    }
     check(op, mi_sdpa_forward(&a));
 }
 

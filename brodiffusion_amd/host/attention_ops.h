@@ -39,8 +39,9 @@ struct RopeTables {
 RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const std::vector<int>& axes_dims_rope,
                                    float theta = 10000.0f);
 
-// RoPE on Q and K, then full-bidirectional attention. The rotation is applied while Q and K are
-// loaded; Qr / Kr (the reference's scratch) are accepted and left untouched.
+// RoPE on Q and K, then full-bidirectional attention. Q is rotated while it is loaded; K is rotated
+// into Kr (resized to K's shape, holds RoPE(K) afterwards as in the reference) and read from there.
+// Qr is accepted and left untouched.
 void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin,
                      int head_dim, int num_heads, Tensor& out, Tensor& Qr, Tensor& Kr);
 

@@ -101,9 +101,10 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
                  scale: Optional[float] = None, mask: Optional[SdpaMask] = None,
                  kv_valid_len: Optional[torch.Tensor] = None, key_mask: Optional[torch.Tensor] = None,
                  rope_q: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                 rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, op: str = "sdpa_forward") -> torch.Tensor:
+                 rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 rope_k_scratch: Optional[torch.Tensor] = None, op: str = "sdpa_forward") -> torch.Tensor:
     """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None)."""
-    _dev(op, q, k, v, out, k_prefix, v_prefix, kv_valid_len, key_mask)
+    _dev(op, q, k, v, out, k_prefix, v_prefix, kv_valid_len, key_mask, rope_k_scratch)
     dt = _dtype_code(op, q)
     if k.dtype != q.dtype or v.dtype != q.dtype:
         _fail(op, "Q, K, V must share one dtype")
@@ -181,6 +182,12 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
             a.rope_cos_q, a.rope_sin_q = cs.data_ptr(), sn.data_ptr()
         else:
             a.rope_cos_k, a.rope_sin_k = cs.data_ptr(), sn.data_ptr()
+    if rope_k_scratch is not None:
+        if rope_k is None:
+            _fail(op, "rope_k_scratch given without rope_k tables")
+        if rope_k_scratch.dtype != q.dtype or not rope_k_scratch.is_contiguous() or rope_k_scratch.numel() < k.numel():
+            _fail(op, "rope_k_scratch must be contiguous, of Q's dtype and at least as large as K")
+        a.rope_k_scratch = rope_k_scratch.data_ptr()
     a.stream = _stream()
     capi.check(capi.lib().mi_sdpa_forward(C.byref(a)), op)
     return out
@@ -245,18 +252,21 @@ def rope_apply_perhead(X, cos, sin, head_dim: int, num_heads: int, out: Optional
 def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
                     Qr: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
     """Full-bidirectional joint attention with RoPE on Q and K (include/brodiffusion/dit/common.h:74-88).
-    The rotation happens while Q and K are loaded; the Qr / Kr scratch tensors of the reference
-    signature are accepted and left untouched."""
+    Q is rotated while it is loaded. With a Kr scratch (K's shape and dtype) K is rotated into it by one
+    pass and, as in the reference, Kr holds RoPE(K) afterwards; without one K is rotated tile by tile
+    inside the attention kernel (slower). Qr is accepted and left untouched."""
     op = "joint_attention"
     if Q.dim() != 2 or Q.shape[1] != head_dim * num_heads:
         _fail(op, "D must equal head_dim * num_heads")
     if K.shape != Q.shape or V.shape != Q.shape:
         _fail(op, "Q/K/V must share shape (L, D)")
-    return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), op=op)
+    if Kr is not None and (Kr.shape != K.shape or Kr.dtype != K.dtype):
+        _fail(op, "Kr must have K's shape and dtype")
+    return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), rope_k_scratch=Kr, op=op)
 
 
 def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num_kv_heads: int, d_mask,
-                         out: Optional[torch.Tensor] = None):
+                         out: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
     """Bidirectional grouped-query attention with optional RoPE and key-padding mask
     (include/brodiffusion/dit/common.h:131-153). K/V heads are indexed in place, not widened."""
     op = "gqa_attention_masked"
@@ -266,7 +276,7 @@ def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num
         _fail(op, "cos and sin must be given together")
     rope = (cos, sin) if cos is not None else None
     return sdpa_forward(Q, K, V, num_q_heads, num_kv_heads=num_kv_heads, out=out, key_mask=d_mask,
-                        rope_q=rope, rope_k=rope, op=op)
+                        rope_q=rope, rope_k=rope, rope_k_scratch=Kr if rope is not None else None, op=op)
 
 
 def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,

@@ -82,8 +82,9 @@ MI_API int mi_memset_async(void* dst, int value, size_t bytes, void* stream);
  *   - k_prefix/v_prefix: leading key rows read from a second buffer, so the cached
  *     prefix K/V of the Qwen-Image step (src/dit/qwenimage21_forward.cpp:599-649) is
  *     consumed in place instead of being copied into [cache ; fresh];
- *   - rope_*: RoPE applied to Q and to the rows of `k` as they are loaded, replacing the
- *     two bt::rope_apply passes of dit::joint_attention (src/dit/common.cpp:188-196).
+ *   - rope_*: RoPE applied to Q as it is loaded and to the rows of `k` (as they are loaded, or by
+ *     one pass into rope_k_scratch when the caller lends one), replacing the two bt::rope_apply
+ *     passes of dit::joint_attention (src/dit/common.cpp:188-196).
  *     Adjacent-pair convention (x[2p], x[2p+1]); prefix rows are taken as already rotated
  *     (the reference caches post-RoPE K, qwenimage21_forward.cpp:587-597);
  *   - block-causal segments: the per-segment calls of the prefill form
@@ -135,13 +136,18 @@ typedef struct mi_sdpa_args {
     const float* rope_sin_q;
     const float* rope_cos_k;     /* device FP32 (kv_len, head_dim/2) or NULL; rows of `k` only */
     const float* rope_sin_k;
+    void* rope_k_scratch;        /* device (batch, kv_len, kv_heads*head_dim) of `dtype`, dense, or NULL. With rope_cos_k:
+                                    K is rotated into it by one bandwidth-bound pass and attention reads the rotated copy
+                                    (fastest form); afterwards it holds RoPE(K) like the Kr scratch of dit::joint_attention
+                                    (src/dit/common.cpp:193). NULL: K is rotated tile by tile as it is loaded */
     void* stream;                /* hipStream_t; NULL = library current stream */
 } mi_sdpa_args;
 
 MI_API int mi_sdpa_forward(const mi_sdpa_args* args);
 /* Tuning / testing knob for the calling thread: 0 = choose the kernel by problem size (default),
  * 1 = always the 4-wavefront kernel (128 query rows per work group), 2 = always the 8-wavefront
- * ping-pong kernel (256 rows; head_dim <= 128). Results agree to rounding; no reference counterpart. */
+ * ping-pong kernel (256 rows; head_dim <= 128), 3 = as 2 but with register-staged tiles where the
+ * default would use LDS DMA (head_dim 128). Results agree to rounding; no reference counterpart. */
 MI_API int mi_sdpa_set_kernel_choice(int32_t choice);
 /* 1 if (dtype, head_dim) has a compiled kernel, else 0. */
 MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);

@@ -155,7 +155,10 @@ static void gpu_checks() {
         Tensor kp = K.row_view(0, prefix), vp = V.row_view(0, prefix), o_cached;
         dit::block_causal_attention(Q.row_view(prefix, L - prefix), K.row_view(prefix, L - prefix), V.row_view(prefix, L - prefix), &kp, &vp,
                                     {{dit::Segment::Kind::Image, L - prefix}}, prefix, H, nullptr, nullptr, o_cached);
-        CHECK(o_cached.to_host_bytes() == im);
+        // the key tiles restart at the prefix boundary, so the summation order differs from the one-buffer call
+        const Err ec = compare(download_bf16(o_img), download_bf16(o_cached));
+        std::printf("cached vs prefill     rel_l2=%.3e max_abs=%.3e\n", ec.rel_l2, ec.max_abs);
+        CHECK(within_bf16(ec));
         std::vector<int> sq = {prefix, L}, sk = {prefix, L}, sc = {1, 0}, lo(L), hi(L);
         orc_rows_block_causal(L, L, 0, sq.data(), sk.data(), sc.data(), 2, lo.data(), hi.data());
         std::vector<float> ref(q.size());

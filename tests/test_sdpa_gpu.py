@@ -11,10 +11,11 @@ from helpers import TOL, assert_close, randn, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["rows128", "rows256_pingpong"])
+@pytest.fixture(autouse=True, params=["rows128", "rows256_pingpong", "rows256_pingpong_regs"])
 def kernel_choice(request):
-    """Every case runs on both kernels: 4 wavefronts x 128 rows, and 8 wavefronts x 256 rows (ping-pong)."""
-    bd.set_sdpa_kernel_choice(1 if request.param == "rows128" else 2)
+    """Every case runs on all kernels: 4 wavefronts x 128 rows; 8 wavefronts x 256 rows (ping-pong) with
+    LDS-DMA tiles where available (head_dim 128) and with register-staged tiles."""
+    bd.set_sdpa_kernel_choice({"rows128": 1, "rows256_pingpong": 2, "rows256_pingpong_regs": 3}[request.param])
     yield request.param
     bd.set_sdpa_kernel_choice(0)
 
@@ -187,6 +188,30 @@ def test_joint_attention_fused_rope(oracle, dtype, d, axes):
     dkr = bd.rope_apply(to_dev(k, dtype), cos, sin, d, H)
     out2 = bd.flash_attention_forward(dqr, dkr, to_dev(v, dtype), None, H, False)
     assert torch.equal(out, out2)
+    # with the Kr scratch of the reference signature: K rotated by one pass, Kr holds RoPE(K) afterwards
+    Kr = torch.zeros_like(dkr)
+    out3 = bd.joint_attention(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), cos, sin, d, H, Kr=Kr)
+    assert torch.equal(Kr, dkr) and torch.equal(out3, out2)
+
+
+def test_rope_k_scratch_batched_strided(oracle):
+    """The scratch form with batch > 1 and a strided K (K cut out of a fused QKV projection)."""
+    dtype, B, H, d, L = "bf16", 2, 2, 128, 200
+    qkv = randn(105, (B, L, 3 * H * d), dtype)
+    dqkv = to_dev(qkv, dtype)
+    dq, dk, dv = dqkv[..., :H * d], dqkv[..., H * d:2 * H * d], dqkv[..., 2 * H * d:]
+    ocos, osin = oracle.build_axial_rope_tables(8, 12, 16, d, (16, 56, 56))
+    cos, sin = torch.from_numpy(ocos).cuda(), torch.from_numpy(osin).cuda()
+    Kr = torch.empty((B, L, H * d), dtype=dq.dtype, device="cuda")
+    out = bd.sdpa_forward(dq, dk, dv, H, rope_q=(cos, sin), rope_k=(cos, sin), rope_k_scratch=Kr)
+    fused = bd.sdpa_forward(dq, dk, dv, H, rope_q=(cos, sin), rope_k=(cos, sin))
+    assert torch.equal(out, fused)
+    for b in range(B):
+        q, k, v = qkv[b, :, :H * d], qkv[b, :, H * d:2 * H * d], qkv[b, :, 2 * H * d:]
+        qr = oracle.rope_apply(q, ocos, osin, H, d, round_to_dtype=dtype)
+        kr = oracle.rope_apply(k, ocos, osin, H, d, round_to_dtype=dtype)
+        assert_close(oracle.sdpa(qr, kr, v, H), to_np(out[b]), dtype)
+        assert_close(kr, to_np(Kr[b]), dtype)
 
 
 def test_rope_on_fresh_keys_only_with_prefix(oracle):
