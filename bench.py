@@ -25,9 +25,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, published
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured.
-TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --traffic-probe`: (69290 KiB x 2.00 calibration) fetched + 27648 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (69290 * 2 + 27648) * 1024
 
 
 def parse():
@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="few launches of the headline step plus one 256 MiB tensor copy; run under rocprofv3 --pmc "
+                         "FETCH_SIZE (or WRITE_SIZE): the copy calibrates the counter, the step gives HBM bytes per launch")
     return ap.parse_args()
 
 
@@ -167,6 +170,15 @@ def main():
     def step():
         bd.joint_attention(q, k, v, cos, sin, d, H, out=out, Kr=kr)
 
+    if args.traffic_probe:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+            step()
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": "3 x (256 MiB copy, headline step)"}))
+        return
     preheat(torch, step)
     for _ in range(args.warmup):
         step()
