@@ -312,16 +312,18 @@ template <int D> constexpr int lds_bytes_8() {
     return kv > o ? kv : o;
 }
 
-// Time is counted in slots separated by work-group barriers. Group 0 (wavefronts 0-3) runs its MFMA
-// phase in even slots and its VALU phase in odd slots; group 1 (wavefronts 4-7, sharing the SIMDs of
-// 0-3) the other way round. With t = slot / 2 (the first iteration, t = -1, has no P yet and only
-// scores tile 0):
-//   MFMA phase:  O += V_t^T P_t ;  S_{t+1} = K_{t+1} Q^T   (reads LDS tiles V_t, K_{t+1}); in its
-//                shadow the wavefront stores its share of tiles K_{t+2}, V_{t+1} into the LDS buffers
-//                of K_t, V_{t-1} and issues the global loads of K_{t+3}, V_{t+2}
-//   VALU phase:  P_{t+1} = softmax(S_{t+1})
-// Tiles K_{t+1}, V_t are complete in LDS before slot 2t and last read in slot 2t+1; the buffers
-// written in slots 2t and 2t+1 were last read in slot 2t-1, so two buffers per operand suffice.
+// Eight wavefronts, 32 query rows each; wavefronts w and w + 4 share a SIMD. One work-group barrier per
+// key tile. Between two barriers (step t; step -1 has no P yet and only scores tile 0) every wavefront runs
+//   the MFMA stream:  O += V_t^T P_t ;  S_{t+1} = K_{t+1} Q^T   (reads LDS tiles V_t, K_{t+1}), and
+//   one softmax:      P = softmax(S) of the scores it holds,
+// in opposite order in the two groups: group 0 (wavefronts 0-3) streams first and then turns S_{t+1} into
+// P_{t+1}; group 1 first turns S_t (scored in the previous step) into P_t and then streams. So on every SIMD
+// one wavefront feeds the matrix pipe while the other is in its VALU part, and neither waits for the other
+// before the end of the step: a barrier between the two halves (strict ping-pong) makes each stream run
+// alone with its LDS and dependency latencies exposed and was measured ~1.6x slower.
+// In the shadow of the stream the wavefront stores its share of tiles K_{t+2}, V_{t+1} into the LDS buffers
+// of K_t, V_{t-1} (last read in step t-1) and issues the global loads of K_{t+3}, V_{t+2}; two buffers per
+// operand suffice.
 template <typename T, int D, bool ROPE_K>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev p) {
     using G = HeadGeo<D>;
@@ -412,23 +414,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         if (n_tiles > 1) mv.template issue<0>(1);
         mv.template issue<1>(0);
         __syncthreads();
-        // ── group 1 falls one slot behind ──
-        if (grp == 1) __syncthreads();
-        // iteration -1 only scores tile 0 (there is no P yet)
-        for (int t = -1; t < n_tiles; ++t) {
-            // MFMA phase
-            __builtin_amdgcn_s_setprio(2);
-            // Always the full stream: at t = -1 P is zero and the (zero-filled) V buffer adds nothing;
-            // after the last tile the extra scores are never read. This wavefront's share of the tile
-            // movement rides along in the stream, where the VALU and memory ports are otherwise idle.
-            mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
-                                          [&]() { advance_tiles(t + 2, t + 1); });
-            __builtin_amdgcn_s_setprio(0);
-            __syncthreads();
-            // VALU phase
-            if (tile_active(t + 1)) {
-                const int j0 = plan.j0(t + 1);
-                const int lim = plan.limit(t + 1);
+        auto softmax_of = [&](int tt) {
+            if (tile_active(tt)) {
+                const int j0 = plan.j0(tt);
+                const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
                 softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
             } else {
@@ -436,9 +425,24 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
 #pragma unroll
                 for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
             }
+        };
+        // step -1 only scores tile 0 (there is no P yet)
+        for (int t = -1; t < n_tiles; ++t) {
+            if (grp == 1) {
+                softmax_of(t);
+                MI_SCHED_BARRIER
+            }
+            // Always the full stream: at t = -1 P is zero and the (zero-filled) V buffer adds nothing;
+            // after the last tile the extra scores are never read. This wavefront's share of the tile
+            // movement rides along in the stream.
+            mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
+                                          [&]() { advance_tiles(t + 2, t + 1); });
+            if (grp == 0) {
+                MI_SCHED_BARRIER
+                softmax_of(t + 1);
+            }
             __syncthreads();
         }
-        if (grp == 0) __syncthreads();
     }
 
     const float l_tot = exchange_sum(st.l);
@@ -451,19 +455,16 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
 // ─────────────── 8-wavefront ping-pong kernel, head_dim 128, tiles by LDS DMA ───────────────
 // Same schedule as sdpa_fwd_pp_kernel, but K/V tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4: lane i of a wavefront deposits its 16 bytes at base + 16*i), so tile
-// movement costs no registers, no LDS store instructions and no wait inside the MFMA stream.
+// movement costs no registers and no LDS store instructions.
 // A DMA instruction writes 1024 contiguous bytes = 4 unpadded 256-byte rows, so bank conflicts are
 // avoided by an XOR swizzle instead of row padding: 16-byte chunk c of row r lives at chunk position
 // c ^ f(r), f(r) = 4*(r%4) + (r/4)%4. The swizzle is applied for free on the global side (each lane
 // fetches the chunk that belongs in its LDS slot) and undone in the LDS read addresses:
 //   K reads (one row per lane, 16 consecutive rows): f takes 16 distinct values -> 16 distinct slots
 //   V transpose reads (4 rows x 64 bytes per 32 lanes): rows r%4 = 0..3 land in distinct 64-byte windows
-// Tiles are ring-buffered three deep: the loads of K_{t+3}, V_{t+2} are issued during MFMA phase t
-// and awaited at the end of the following VALU phase, two phases later. The key loop is unrolled by
-// three so that every LDS offset is an instruction immediate.
-// A wavefront issues at most one instruction every 4 clocks, so instruction count is what the phases
-// cost: tile pointers advance incrementally in scalar registers, and the four DMA instructions of a
-// step are spread between the first MFMAs instead of being issued in one lump.
+// Tiles are ring-buffered three deep: the loads of K_{t+3}, V_{t+2} are issued in step t, awaited at
+// the end of step t+1 and read in step t+2. The key loop is unrolled by three so that every LDS offset
+// is an instruction immediate; tile pointers advance incrementally in scalar registers.
 // Rows past the end of a segment are fetched from its last row (valid memory); their scores are masked.
 constexpr int kDmaStages = 3;
 constexpr int kRowBytes128 = 256;
@@ -622,8 +623,34 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         constexpr int KS = S * kTileBytes128, VS = ((S + 2) % 3) * kTileBytes128;
         constexpr int KD = ((S + 2) % 3) * kTileBytes128, VD = kVbufOff128 + ((S + 1) % 3) * kTileBytes128;
         const bool load_k = t + 3 < n_tiles, load_v = t + 2 < n_tiles;
-        // ── MFMA phase ──
-        __builtin_amdgcn_s_setprio(2);
+        auto softmax_of = [&](int tt) {
+            if (tile_active(tt)) {
+                const int j0 = plan.j0(tt);
+                const int lim = plan.limit(tt);
+                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
+                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
+            } else {
+                // nothing visible to this wavefront in that tile: the next PV pass must add zero
+#pragma unroll
+                for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+            }
+        };
+        // An LDS read issued behind an LDS-DMA load does not return before that load has landed (measured: the
+        // read takes the full memory latency), so the four DMA instructions of a step go where the wavefront
+        // has no LDS access ahead of it for a long time: right before its softmax.
+        auto issue_dma = [&]() {
+            if (load_k) { dma(kc, 0, KD); dma(kc, 1, KD); }
+            if (load_v) { dma(vc, 0, VD); dma(vc, 1, VD); }
+            if (load_k) kc.next();
+            if (load_v) vc.next();
+        };
+        // group 1 turns the scores of its previous step into P first, so that its MFMA stream meets group 0's softmax
+        if (grp == 1) {
+            issue_dma();
+            MI_SCHED_BARRIER
+            softmax_of(t);
+            MI_SCHED_BARRIER
+        }
         {
             constexpr int NPV = 4 * G::VB, N = NPV + 2 * G::KC;
             auto fetch = [&](int i) -> V8 {
@@ -663,29 +690,19 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 }
                 if (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
                 MI_SCHED_BARRIER
-                // the four DMA instructions of this step, one behind each of MFMAs 1, 3, 5, 7
-                if (i == 1 && load_k) dma(kc, 0, KD);
-                if (i == 3 && load_k) dma(kc, 1, KD);
-                if (i == 5 && load_v) dma(vc, 0, VD);
-                if (i == 7 && load_v) dma(vc, 1, VD);
-                if (i == 1 || i == 3 || i == 5 || i == 7) { MI_SCHED_BARRIER }
             }
         }
-        __builtin_amdgcn_s_setprio(0);
-        if (load_k) kc.next();
-        if (load_v) vc.next();
-        __syncthreads();
-        // ── VALU phase ──
-        if (tile_active(t + 1)) {
-            const int j0 = plan.j0(t + 1);
-            const int lim = plan.limit(t + 1);
-            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
-        } else {
-#pragma unroll
-            for (int c4 = 0; c4 < 4; ++c4) pf[c4] = __builtin_bit_cast(V8, u32x4{0, 0, 0, 0});
+        if (grp == 0) {
+            MI_SCHED_BARRIER
+            issue_dma();
+            MI_SCHED_BARRIER
+            softmax_of(t + 1);
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's tile loads have landed
+        // The tiles loaded in the PREVIOUS step are read in the next one: wait for those only (this step's
+        // loads stay in flight; loads complete in order), then meet the other wavefronts.
+        if (load_k) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if (load_v) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     };
 
@@ -698,7 +715,6 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         if (n_tiles > 1) vc.next();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (grp == 1) __syncthreads();   // group 1 falls one slot behind
         for (int t = -1; t < n_tiles; t += 3) {
             step(std::integral_constant<int, 0>{}, t);
             if (t + 1 >= n_tiles) break;
@@ -706,7 +722,6 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             if (t + 2 >= n_tiles) break;
             step(std::integral_constant<int, 2>{}, t + 2);
         }
-        if (grp == 0) __syncthreads();
     }
 
     const float l_tot = exchange_sum(st.l);
