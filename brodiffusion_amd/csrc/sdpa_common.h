@@ -79,17 +79,26 @@ __device__ __forceinline__ float exchange_sum(float x) {
 }
 
 // Rotate the 4 adjacent pairs held in one 16-byte chunk, FP32 arithmetic, one rounding back to T.
+// (post_scale multiplies the rotated value before the rounding; 1 leaves it bit-identical to the stand-alone pass.)
 template <typename T>
-__device__ __forceinline__ u32x4 rope_chunk(u32x4 raw, f32x4 c, f32x4 s) {
+__device__ __forceinline__ u32x4 rope_chunk(u32x4 raw, f32x4 c, f32x4 s, float post_scale = 1.f) {
     typedef T t8 __attribute__((ext_vector_type(8)));
     t8 x = __builtin_bit_cast(t8, raw);
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         const float a = static_cast<float>(x[2 * p]);
         const float b = static_cast<float>(x[2 * p + 1]);
-        x[2 * p] = static_cast<T>(rope_re(a, b, c[p], s[p]));
-        x[2 * p + 1] = static_cast<T>(rope_im(a, b, c[p], s[p]));
+        x[2 * p] = static_cast<T>(rope_re(a, b, c[p], s[p]) * post_scale);
+        x[2 * p + 1] = static_cast<T>(rope_im(a, b, c[p], s[p]) * post_scale);
     }
+    return __builtin_bit_cast(u32x4, x);
+}
+template <typename T>
+__device__ __forceinline__ u32x4 scale_chunk(u32x4 raw, float f) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    t8 x = __builtin_bit_cast(t8, raw);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = static_cast<T>(static_cast<float>(x[e]) * f);
     return __builtin_bit_cast(u32x4, x);
 }
 
@@ -133,25 +142,53 @@ __device__ __forceinline__ WaveExtent wave_extent(int lo, int hi) {
     return w;
 }
 
-// Q fragments (B operand of K Q^T) of this lane's query row, RoPE applied on the way in.
+// The Q tile of a work group goes through LDS once. A lane needs the 16-byte pieces of ONE query row (B operand of
+// K Q^T), so direct loads would touch one cache line per lane and instruction, and the RoPE tables twice as many;
+// instead the rows are fetched with full-row coalescing (consecutive threads take consecutive 16-byte chunks of a row,
+// of Q and of the cos / sin tables), rotated in registers and stored row-major at stride O_STRIDE (the layout the
+// output staging uses later). All loads are issued before the first is used: out-of-range rows and the zero-pad
+// chunk are fetched from a clamped address and blanked at the store.
+// q_scale != 1 folds a factor (softmax scale times log2 e) into Q before its single rounding to T.
+template <typename T, int D, int NT, int ROWS>
+__device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p, const T* q_base, int q0, int tid, float q_scale = 1.f) {
+    using G = HeadGeo<D>;
+    constexpr int CPRK = G::DK / 8;            // chunks per staged row (data chunks, then the zero pad)
+    constexpr int NCH = ROWS * CPRK;
+    constexpr int NI = (NCH + NT - 1) / NT;
+    const int last_row = p.Lq - 1;
+    const bool rope = p.cos_q != nullptr;
+    u32x4 raw[NI];
+    f32x4 cs[NI], sn[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int idx = min(tid + NT * i, NCH - 1);
+        const int row = idx / CPRK, cc = min(idx - row * CPRK, G::CPR - 1);
+        const int qrow = min(q0 + row, last_row);
+        raw[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + cc * 8);
+        if (rope) {
+            cs[i] = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
+            sn[i] = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int idx = tid + NT * i;
+        const int row = idx / CPRK, cc = idx - row * CPRK;
+        u32x4 v = raw[i];
+        if (rope) v = rope_chunk<T>(v, cs[i], sn[i], q_scale);
+        else if (q_scale != 1.f) v = scale_chunk<T>(v, q_scale);
+        if (q0 + row > last_row || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
+        if (idx < NCH) *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
+    }
+}
+
+// Q fragments of this lane's query row (tile row `trow`) from the staged tile.
 template <typename T, int D>
-__device__ __forceinline__ void load_q_frags(typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], const SdpaDev& p, const T* q_base,
-                                             int qrow, bool qvalid, int lh) {
+__device__ __forceinline__ void read_q_frags(typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], const unsigned char* Qs, int trow, int lh) {
     using V8 = typename Mma<T>::v8;
 #pragma unroll
-    for (int c = 0; c < HeadGeo<D>::KC; ++c) {
-        const int d0 = 16 * c + 8 * lh;
-        u32x4 raw = u32x4{0, 0, 0, 0};
-        if (qvalid && d0 < D) {
-            raw = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + d0);
-            if (p.cos_q) {
-                const f32x4 cs = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
-                const f32x4 sn = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + d0 / 2);
-                raw = rope_chunk<T>(raw, cs, sn);
-            }
-        }
-        qf[c] = __builtin_bit_cast(V8, raw);
-    }
+    for (int c = 0; c < HeadGeo<D>::KC; ++c)
+        qf[c] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Qs + trow * HeadGeo<D>::O_STRIDE + (16 * c + 8 * lh) * 2));
 }
 
 // The MFMA work of one step as a single software-pipelined stream: first O^T += V^T P^T for one
@@ -172,7 +209,7 @@ struct NoMid { __device__ __forceinline__ void operator()() const {} };
 template <typename T, int D, bool DO_PV, bool DO_QK, typename Mid = NoMid>
 __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsigned char* Ks, const typename Mma<T>::v8 (&pf)[4],
                                             const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid()) {
+                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid(), const f32x16* s_init = nullptr) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
     constexpr int NPV = DO_PV ? 4 * G::VB : 0;
@@ -214,8 +251,9 @@ __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsig
             const int k = i - NPV;
             const int kb = k / G::KC, c = k % G::KC;
             if (c == 0) {
+                // the score accumulator starts from zero, or from the caller's vector (minus the row's softmax reference)
                 const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                sacc[kb] = Mma<T>::run(a, qf[c], zero);
+                sacc[kb] = Mma<T>::run(a, qf[c], s_init ? *s_init : zero);
             } else {
                 sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
             }
@@ -304,6 +342,78 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
     for (int c4 = 0; c4 < 4; ++c4)
 #pragma unroll
         for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
+}
+
+// Softmax step for scores that leave the matrix pipe in exponent units and relative to the row's reference: Q carries
+// scale * log2(e), and the first K Q^T MFMA of a key block starts from an accumulator filled with -ref (`neg_ref`, the
+// same value in all 16 slots), so P = exp2(S) needs no further arithmetic and the usual tile maximum is not computed at
+// all. Per 64-key tile and lane that is 32 v_exp, 32 adds and 16 packs instead of ~150 VALU instructions.
+//   * The reference of a row is the maximum of its first tile with a visible key (then its largest term is 1, so the
+//     denominator stays >= 1), and is raised to a later tile's maximum only when that tile's terms get large (lane sum
+//     above 2^10, or overflow). Any reference gives the same softmax; these two rules keep every term within FP32 / T range.
+//   * Both cases, and rows that have not seen a key yet, take the slow path below (wave-uniform branch): row maximum,
+//     shift of l, O and the scores, new exponentials. Lanes l and l^32 share a row and decide from row-wide values only.
+struct RelSoftmaxState {
+    float l = 0.f;          // this lane's share of the denominator
+    bool started = false;   // the row has a reference (it has seen a visible key)
+};
+constexpr float kRelSumMax = 1024.f;
+
+template <typename T, int D>
+__device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
+                                                 RelSoftmaxState& st, f32x16& neg_ref, bool masked, bool dead_row, int j0, int lo,
+                                                 int hi, int lh) {
+    if (masked) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                if (key < lo || key >= hi) sacc[kb][e] = kNegInf;
+            }
+    }
+    auto exponentiate = [&]() -> float {
+        float s0 = 0.f, s1 = 0.f;
+        // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
+#pragma unroll
+        for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+            for (int t = 0; t < 8; t += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t]);
+                const float p1 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t + 1]);
+                pf[c4][t] = static_cast<T>(p0);
+                pf[c4][t + 1] = static_cast<T>(p1);
+                s0 += p0;
+                s1 += p1;
+            }
+        return s0 + s1;
+    };
+    float ls = exponentiate();
+    const bool fine = (st.started || dead_row) && ls < kRelSumMax;   // false also for inf / nan sums
+    if (__any(!fine)) {
+        float mloc = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mloc = fmaxf(mloc, fmaxf(sacc[0][e], sacc[1][e]));
+        mloc = exchange_max(mloc);
+        const bool visible = mloc > kNegInf;
+        // a started row only ever moves its reference up (its terms then stay <= 1)
+        const float shift = !visible ? 0.f : (st.started ? fmaxf(mloc, 0.f) : mloc);
+        const float alpha = st.started ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // nothing accumulated before the first key
+        st.started = st.started || visible;
+        st.l *= alpha;
+#pragma unroll
+        for (int vb = 0; vb < HeadGeo<D>::VB; ++vb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[vb][e] *= alpha;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            sacc[0][e] -= shift;
+            sacc[1][e] -= shift;
+            neg_ref[e] -= shift;
+        }
+        ls = exponentiate();
+    }
+    st.l += ls;
 }
 
 // Normalised output rows of one wavefront into the LDS staging area (row-major, O_STRIDE).

@@ -226,14 +226,16 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     row_interval(p, b, qrow, qvalid, lo, hi);
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[4 + wave] = we.hi_max; }
+    V8 qf[G::KC];
+    stage_q_tile<T, D, kThreads4, BM>(smem, p, q_base, q0, tid);
+    __syncthreads();
+    read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
+    __syncthreads();
     zero_pads<D, kThreads4>(smem, smem + G::K_BYTES, STAGE, STAGE, 2, tid);
     __syncthreads();
     const int g_lo = __builtin_amdgcn_readfirstlane(min(min(red[0], red[1]), min(red[2], red[3])));
     const int kv_stop = __builtin_amdgcn_readfirstlane(max(max(red[4], red[5]), max(red[6], red[7])));
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
-
-    V8 qf[G::KC];
-    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
 
     f32x16 oacc[G::VB];
 #pragma unroll
@@ -359,6 +361,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     row_interval(p, b, qrow, qvalid, lo, hi);
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    V8 qf[G::KC];
+    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid, p.scale_log2);   // Q carries scale * log2(e)
+    __syncthreads();
+    read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
+    __syncthreads();
     // K pad columns must be zero; the V buffers are zeroed whole because the first pass through the
     // MFMA stream multiplies a zero P with whatever the second V buffer holds
     zero_pads<D, kThreads8>(Kbuf, Vbuf, G::K_BYTES, G::V_BYTES, 2, tid);
@@ -372,17 +379,16 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
     const int n_tiles = plan.n_tiles;
 
-    V8 qf[G::KC];
-    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
-
     f32x16 oacc[G::VB];
 #pragma unroll
     for (int vb = 0; vb < G::VB; ++vb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
-    SoftmaxState st;
-    const float cl2 = p.scale_log2;
-    const float lazy_raw = kLazyLog2 / cl2;
+    RelSoftmaxState st;
+    const bool dead_row = hi <= lo;
+    f32x16 neg_ref;   // minus the row's softmax reference in all 16 slots: accumulator start of every score block
+#pragma unroll
+    for (int e = 0; e < 16; ++e) neg_ref[e] = 0.f;
 
     TileMover<T, D, kThreads8, ROPE_K> mv{p, plan,
                                           reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D),
@@ -419,7 +425,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -436,7 +442,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
             // after the last tile the extra scores are never read. This wavefront's share of the tile
             // movement rides along in the stream.
             mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
-                                          [&]() { advance_tiles(t + 2, t + 1); });
+                                          [&]() { advance_tiles(t + 2, t + 1); }, &neg_ref);
             if (grp == 0) {
                 MI_SCHED_BARRIER
                 softmax_of(t + 1);
@@ -540,6 +546,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     row_interval(p, b, qrow, qvalid, lo, hi);
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    V8 qf[G::KC];
+    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid, p.scale_log2);   // Q carries scale * log2(e)
+    __syncthreads();
+    read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
+    __syncthreads();
     // the first pass through the MFMA stream multiplies a zero P with the last V buffer
     for (int i = tid; i < kTileBytes128 / 16; i += kThreads8)
         *reinterpret_cast<u32x4*>(smem + kVbufOff128 + (kDmaStages - 1) * kTileBytes128 + i * 16) = u32x4{0, 0, 0, 0};
@@ -552,16 +563,16 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
     const int n_tiles = plan.n_tiles;
 
-    V8 qf[G::KC];
-    load_q_frags<T, D>(qf, p, q_base, qrow, qvalid, lh);
     f32x16 oacc[G::VB];
 #pragma unroll
     for (int vb = 0; vb < G::VB; ++vb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
-    SoftmaxState st;
-    const float cl2 = p.scale_log2;
-    const float lazy_raw = kLazyLog2 / cl2;
+    RelSoftmaxState st;
+    const bool dead_row = hi <= lo;
+    f32x16 neg_ref;   // minus the row's softmax reference in all 16 slots: accumulator start of every score block
+#pragma unroll
+    for (int e = 0; e < 16; ++e) neg_ref[e] = 0.f;
 
     // ── DMA source geometry of this lane: LDS slot (row 4*wave + lane/16 [+32], position lane%16) ──
     TileCursor kc, vc;
@@ -628,7 +639,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, nullptr);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -682,8 +693,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                     const int k = i - NPV;
                     const int kb = k / G::KC, c = k % G::KC;
                     if (c == 0) {
-                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                        sacc[kb] = Mma<T>::run(a, qf[c], zero);
+                        sacc[kb] = Mma<T>::run(a, qf[c], neg_ref);
                     } else {
                         sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
                     }

@@ -11,6 +11,18 @@ from helpers import TOL, assert_close, randn, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
+def assert_same(a: torch.Tensor, b: torch.Tensor, exact: bool, what: str = ""):
+    """Two routes to the same result: bit-identical where both run the same arithmetic in the same order,
+    else equal to rounding: each is within one unit in the last place of the exact value, so they differ by
+    at most two (2^-7 of the magnitude in bf16, 2^-10 in fp16)."""
+    if exact:
+        assert torch.equal(a, b), what
+    else:
+        ulp2 = 2.0 ** -7 if a.dtype == torch.bfloat16 else 2.0 ** -10
+        err = (a.float() - b.float()).abs().max().item()
+        assert err <= ulp2 * max(1.0, b.float().abs().max().item()), f"{what}: max abs diff {err}"
+
+
 @pytest.fixture(autouse=True, params=["rows128", "rows256_pingpong", "rows256_pingpong_regs"])
 def kernel_choice(request):
     """Every case runs on all kernels: 4 wavefronts x 128 rows; 8 wavefronts x 256 rows (ping-pong) with
@@ -74,7 +86,7 @@ def test_causal_rows_without_keys_are_zero(oracle):
 
 
 @pytest.mark.parametrize("dtype,d", [("bf16", 72), ("fp16", 40), ("bf16", 128)])
-def test_key_mask_equals_trimmed(oracle, dtype, d):
+def test_key_mask_equals_trimmed(oracle, kernel_choice, dtype, d):
     """Key padding three ways (kv_valid_len, 0/1 d_mask, trimmed K/V) must agree: the reference handles
     padding by trimming to the valid rows (src/pipeline.cpp:391-414)."""
     B, H, Lq, Lk = 2, 2, 130, 300
@@ -92,7 +104,9 @@ def test_key_mask_equals_trimmed(oracle, dtype, d):
         assert_close(ref, to_np(o_len[b]), dtype, "kv_valid_len")
         assert_close(ref, to_np(o_mask[b]), dtype, "d_mask")
         o_trim = bd.flash_attention_forward(dq[b], dk[b, :valid[b]], dv[b, :valid[b]], None, H, False)
-        assert torch.equal(o_trim, o_len[b]) and torch.equal(o_trim, o_mask[b])
+        # calls with a 0/1 mask always run on the 128-row kernel, the others on the chosen one
+        assert_same(o_trim, o_len[b], True, "trimmed vs kv_valid_len")
+        assert_same(o_trim, o_mask[b], kernel_choice == "rows128", "trimmed vs d_mask")
 
 
 def test_scattered_key_mask_and_empty_mask(oracle):
@@ -143,7 +157,7 @@ def test_block_causal_prefix_kv(oracle, kernel_choice, prefix, blocks):
         s = e
 
 
-def test_block_causal_with_text_segments(oracle):
+def test_block_causal_with_text_segments(oracle, kernel_choice):
     """Prefill form with causal text runs and bidirectional image blocks in one launch
     (src/dit/qwenimage21_forward.cpp:650-676)."""
     dtype, H, d = "bf16", 2, 128
@@ -166,12 +180,14 @@ def test_block_causal_with_text_segments(oracle):
             seg = bd.flash_attention_windowed_forward(dq[s:e], dk[:e], dv[:e], None, H, 0)
         else:
             seg = bd.flash_attention_forward(dq[s:e], dk[:e], dv[:e], None, H, False)
-        assert torch.equal(seg, out[s:e])
+        # rows of several segments share a wavefront in the one-launch form, and a wavefront re-references
+        # its softmax as a whole: same values to rounding, bit-identical on the kernel that keeps exact row maxima
+        assert_same(seg, out[s:e], kernel_choice == "rows128", "per-segment call vs one launch")
         s = e
 
 
 @pytest.mark.parametrize("dtype,d,axes", [("bf16", 128, (16, 56, 56)), ("fp16", 64, (16, 24, 24)), ("bf16", 40, (8, 16, 16))])
-def test_joint_attention_fused_rope(oracle, dtype, d, axes):
+def test_joint_attention_fused_rope(oracle, kernel_choice, dtype, d, axes):
     H, txt, hp, wp = 2, 37, 9, 11
     L = txt + hp * wp
     q = randn(101, (L, H * d), dtype); k = randn(102, (L, H * d), dtype); v = randn(103, (L, H * d), dtype)
@@ -187,11 +203,13 @@ def test_joint_attention_fused_rope(oracle, dtype, d, axes):
     dqr = bd.rope_apply(to_dev(q, dtype), cos, sin, d, H)
     dkr = bd.rope_apply(to_dev(k, dtype), cos, sin, d, H)
     out2 = bd.flash_attention_forward(dqr, dkr, to_dev(v, dtype), None, H, False)
-    assert torch.equal(out, out2)
+    # the 256-row kernels fold the softmax scale into Q before its rounding: one rounding when fused, two when not
+    assert_same(out, out2, kernel_choice == "rows128", "fused vs stand-alone RoPE")
     # with the Kr scratch of the reference signature: K rotated by one pass, Kr holds RoPE(K) afterwards
     Kr = torch.zeros_like(dkr)
     out3 = bd.joint_attention(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), cos, sin, d, H, Kr=Kr)
-    assert torch.equal(Kr, dkr) and torch.equal(out3, out2)
+    assert torch.equal(Kr, dkr)
+    assert_same(out3, out2, kernel_choice == "rows128", "Kr scratch form vs stand-alone RoPE")
 
 
 def test_rope_k_scratch_batched_strided(oracle):
