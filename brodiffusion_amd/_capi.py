@@ -22,7 +22,7 @@ EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
     "mi_sdpa_forward", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply",
-    "mi_linear_attn_workspace_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
+    "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
 ]
 
 
@@ -76,7 +76,8 @@ class MiLinearAttnArgs(C.Structure):
         ("v_row_stride", C.c_int64), ("v_batch_stride", C.c_int64),
         ("o_row_stride", C.c_int64), ("o_batch_stride", C.c_int64),
         ("eps", C.c_float), ("accumulate_state", C.c_int32),
-        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("stream", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("stream", C.c_void_p),
     ]
 
 
@@ -111,6 +112,8 @@ def lib() -> C.CDLL:
         L.mi_rope_apply.argtypes = [C.POINTER(MiRopeArgs)]
         L.mi_linear_attn_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         L.mi_linear_attn_workspace_bytes.restype = C.c_size_t
+        L.mi_linear_attn_scratch_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
+        L.mi_linear_attn_scratch_bytes.restype = C.c_size_t
         L.mi_linear_attn_relu_forward.argtypes = [C.POINTER(MiLinearAttnArgs)]
         L.mi_linear_attn_supported.argtypes = [C.c_int32, C.c_int32]
         _lib = L

@@ -12,6 +12,7 @@
 //                 global memory; the denominator is an exact FP32 dot of z with the lane's own Q
 //                 values plus one exchange between lanes l and l^32.
 #include <algorithm>
+#include <cstdlib>
 
 #include "internal.h"
 
@@ -50,7 +51,12 @@ struct LinDev {
     long q_rs, q_bs, k_rs, k_bs, v_rs, v_bs, o_rs, o_bs;
     float eps;
     float* ws;      // per (b,h): D*D floats of S (row = value channel), then D floats of z
+    float* part;    // partial states of the token chunks: [(b,h)][chunk][D*D + D], or null
+    int n_part;     // chunks per (b,h) in `part`
+    int add_to_state;   // no partials: this group's (S, z) is added to the state instead of replacing it
     int tokens_per_group;
+    int n_chunks;   // token chunks per (batch, head)
+    int n_blocks;   // work groups with work = B * H * n_chunks
 };
 
 template <int D> struct LGeo {
@@ -58,8 +64,9 @@ template <int D> struct LGeo {
     static constexpr int NB = DP / 32;
     static constexpr int KC = DP / 16;
     static constexpr int T_STRIDE = ((DP * 2 + 63) / 128) * 128 + 64;  // tiles read by transpose reads
-    static constexpr int S_STRIDE = DP * 2 + 16;                       // S rows read by ds_read_b128
+    static constexpr int S_STRIDE = DP * 2 + 16;                       // rows read one per lane by ds_read_b128
     static constexpr int CPR = D / 8;
+    static constexpr int CPRP = DP / 8;
     static constexpr int NCH = kTN * CPR;
     static constexpr int NLD = (NCH + kThreads - 1) / kThreads;
     static constexpr int WS_FLOATS = D * D + D;
@@ -74,75 +81,113 @@ __device__ __forceinline__ u32x4 relu8(u32x4 raw) {
     return __builtin_bit_cast(u32x4, x);
 }
 
-__global__ void __launch_bounds__(256) fill_zero_kernel(float* p, long n) {
-    for (long i = blockIdx.x * 256L + threadIdx.x; i < n; i += gridDim.x * 256L) p[i] = 0.f;
+__global__ void __launch_bounds__(256) fill_zero_kernel(f32x4* p, long n4) {
+    for (long i = blockIdx.x * 256L + threadIdx.x; i < n4; i += gridDim.x * 256L) p[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// Work group -> (batch*head, token chunk). Hardware work-group ids go round the 8 XCDs, each with its own L2: the
+// logical index is arranged so that one XCD gets a contiguous range of heads with all their chunks. Then the heads
+// whose 2*D-byte row segments share cache lines (a token row holds all heads side by side) meet in the same L2,
+// and so do the work groups that read the same (S, z).
+__device__ __forceinline__ bool lin_block(const LinDev& p, int& bh, int& chunk) {
+    const int per_xcd = (p.n_blocks + 7) >> 3;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.n_blocks) return false;
+    bh = logical / p.n_chunks;
+    chunk = logical - bh * p.n_chunks;
+    return true;
 }
 
 // ── state: (S, z) += over this group's token chunk ──
-template <typename T, int D>
-__global__ void __launch_bounds__(kThreads) linattn_state_kernel(const LinDev p) {
-    using G = LGeo<D>;
-    using V8 = typename Mma<T>::v8;
-    __shared__ __attribute__((aligned(16))) unsigned char Ks[kTN * G::T_STRIDE];
-    __shared__ __attribute__((aligned(16))) unsigned char Vs[kTN * G::T_STRIDE];
+// The pass is a stream of K and V rows with little arithmetic, so what matters is bytes in flight: a work group has
+// 16 wavefronts, each owning at most one 32x32 block of S (16 accumulator registers), which leaves registers for a
+// 128-token tile in flight per group on top of the one being multiplied. Loads are branch-free (rows past the end of
+// the chunk are fetched from its last row and K is blanked at the LDS store, which removes their contribution to S
+// and z) and all issued before the first is used. z comes from the same K fragments against an all-ones A operand.
+// At the end the wavefronts add their blocks into an FP32 image of (S, z) in LDS (several wavefronts share a block
+// when S has fewer than 16 of them), which then goes out in full rows with plain stores: to the state itself when the
+// group covers the whole (batch, head), else to the group's slot among the partial states that a small reduction
+// kernel adds up afterwards (atomic adds from several groups to one address are executed at the memory side on this
+// multi-die GPU and were measured to cost far more than the whole pass).
+constexpr int kStateThreads = 1024;
+constexpr int kMaxStateSplit = 8;   // most token chunks per (batch, head) whose partial states the workspace can hold
+constexpr int kStateTile = 128;
 
-    const int bh = blockIdx.y;
+template <int D> struct StateGeo {
+    using G = LGeo<D>;
+    static constexpr int NBLK = G::NB * G::NB;                                   // 32x32 blocks of S
+    static constexpr int NTS = NBLK >= 16 ? 1 : (16 / NBLK > 8 ? 8 : 16 / NBLK); // wavefronts sharing a block (token split)
+    static constexpr int KSTEPS = (kStateTile / 16) / NTS;                       // 16-token steps per wavefront and tile
+    static constexpr int NCH = kStateTile * G::CPR;
+    static constexpr int NLD = (NCH + kStateThreads - 1) / kStateThreads;
+    static constexpr int TILE_BYTES = kStateTile * G::T_STRIDE;
+    static constexpr int S_FLOATS = G::DP * G::DP + G::DP;
+    static constexpr int LDS_BYTES = 2 * TILE_BYTES > S_FLOATS * 4 ? 2 * TILE_BYTES : S_FLOATS * 4;
+};
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinDev p) {
+    using G = LGeo<D>;
+    using SG = StateGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    unsigned char* const Ks = lds;
+    unsigned char* const Vs = lds + SG::TILE_BYTES;
+
+    int bh, chunk;
+    if (!lin_block(p, bh, chunk)) return;
     const int b = bh / p.H, h = bh % p.H;
-    const int n_begin = blockIdx.x * p.tokens_per_group;
+    const int n_begin = chunk * p.tokens_per_group;
     const int n_end = min(p.N, n_begin + p.tokens_per_group);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int lq = lane & 31, lh = lane >> 5;
     const T* const k_base = static_cast<const T*>(p.k) + b * p.k_bs + h * D;
     const T* const v_base = static_cast<const T*>(p.v) + b * p.v_bs + h * D;
 
-    // wave -> (row block of S, share of the 4 k-steps of a tile)
-    constexpr int NTS = G::NB >= 3 ? 1 : 4 / G::NB;  // token splits
-    constexpr int KSTEPS = 4 / NTS;
-    const int rb = wave % G::NB;
-    const int ts = wave / G::NB;
-    const bool active = wave < G::NB * NTS;
+    // wave -> (block of S, share of the k-steps of a tile)
+    const int blk = wave % SG::NBLK;
+    const int ts = wave / SG::NBLK;
+    const int rb = blk / G::NB, cb = blk % G::NB;
+    const bool active = ts < SG::NTS;
     const bool does_z = active && rb == 0;
 
     if constexpr (G::DP > D) {  // pad columns stay zero for the whole kernel
         constexpr int PC = (G::DP - D) / 8;
-        for (int i = tid; i < kTN * PC; i += kThreads) {
+        for (int i = tid; i < kStateTile * PC; i += kStateThreads) {
             const int off = (i / PC) * G::T_STRIDE + D * 2 + (i % PC) * 16;
             *reinterpret_cast<u32x4*>(Ks + off) = u32x4{0, 0, 0, 0};
             *reinterpret_cast<u32x4*>(Vs + off) = u32x4{0, 0, 0, 0};
         }
     }
 
-    f32x16 acc[G::NB], zacc[G::NB];
+    f32x16 acc, zacc;
 #pragma unroll
-    for (int cb = 0; cb < G::NB; ++cb)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) { acc[cb][e] = 0.f; zacc[cb][e] = 0.f; }
+    for (int e = 0; e < 16; ++e) { acc[e] = 0.f; zacc[e] = 0.f; }
     V8 ones;
 #pragma unroll
     for (int t = 0; t < 8; ++t) ones[t] = static_cast<T>(1.f);
 
-    u32x4 kreg[G::NLD], vreg[G::NLD];
+    u32x4 kreg[SG::NLD], vreg[SG::NLD];
+    const int last = n_end - 1;
     auto issue_loads = [&](int n0) {
 #pragma unroll
-        for (int i = 0; i < G::NLD; ++i) {
-            const int idx = tid + kThreads * i;
-            const int row = idx / G::CPR, cc = idx - (idx / G::CPR) * G::CPR;
-            const int n = n0 + row;
-            kreg[i] = u32x4{0, 0, 0, 0};
-            vreg[i] = u32x4{0, 0, 0, 0};
-            if (idx < G::NCH && n < n_end) {
-                kreg[i] = *reinterpret_cast<const u32x4*>(k_base + static_cast<long>(n) * p.k_rs + cc * 8);
-                vreg[i] = *reinterpret_cast<const u32x4*>(v_base + static_cast<long>(n) * p.v_rs + cc * 8);
-            }
+        for (int i = 0; i < SG::NLD; ++i) {
+            const int idx = min(tid + kStateThreads * i, SG::NCH - 1);
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            const long n = min(n0 + row, last);
+            kreg[i] = *reinterpret_cast<const u32x4*>(k_base + n * p.k_rs + cc * 8);
+            vreg[i] = *reinterpret_cast<const u32x4*>(v_base + n * p.v_rs + cc * 8);
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](int n0) {
 #pragma unroll
-        for (int i = 0; i < G::NLD; ++i) {
-            const int idx = tid + kThreads * i;
-            const int row = idx / G::CPR, cc = idx - (idx / G::CPR) * G::CPR;
-            if (idx < G::NCH) {
-                *reinterpret_cast<u32x4*>(Ks + row * G::T_STRIDE + cc * 16) = relu8<T>(kreg[i]);
+        for (int i = 0; i < SG::NLD; ++i) {
+            const int idx = tid + kStateThreads * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < SG::NCH) {
+                u32x4 kv = relu8<T>(kreg[i]);
+                if (n0 + row > last) kv = u32x4{0, 0, 0, 0};
+                *reinterpret_cast<u32x4*>(Ks + row * G::T_STRIDE + cc * 16) = kv;
                 *reinterpret_cast<u32x4*>(Vs + row * G::T_STRIDE + cc * 16) = vreg[i];
             }
         }
@@ -150,67 +195,94 @@ __global__ void __launch_bounds__(kThreads) linattn_state_kernel(const LinDev p)
 
     const int trow = (lane & 15) >> 2;
     const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    if (n_begin < n_end) issue_loads(n_begin);
-    for (int n0 = n_begin; n0 < n_end; n0 += kTN) {
-        store_tile();
+    issue_loads(n_begin);
+    for (int n0 = n_begin; n0 < n_end; n0 += kStateTile) {
+        store_tile(n0);
         __syncthreads();
-        if (n0 + kTN < n_end) issue_loads(n0 + kTN);
+        if (n0 + kStateTile < n_end) issue_loads(n0 + kStateTile);
         if (active) {
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) {
-                const int ks = ts * KSTEPS + s;
-                const int trow0 = 16 * ks + 4 * lh + trow;
+            for (int s = 0; s < SG::KSTEPS; ++s) {
+                const int trow0 = 16 * (ts * SG::KSTEPS + s) + 4 * lh + trow;
                 const unsigned char* vptr = Vs + trow0 * G::T_STRIDE + (32 * rb + tcol) * 2;
+                const unsigned char* kptr = Ks + trow0 * G::T_STRIDE + (32 * cb + tcol) * 2;
                 const s16x4 a_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
                 const s16x4 a_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::T_STRIDE));
+                const s16x4 b_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(kptr));
+                const s16x4 b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4*)(kptr + 8 * G::T_STRIDE));
                 const V8 a = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-#pragma unroll
-                for (int cb = 0; cb < G::NB; ++cb) {
-                    const unsigned char* kptr = Ks + trow0 * G::T_STRIDE + (32 * cb + tcol) * 2;
-                    const s16x4 b_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(kptr));
-                    const s16x4 b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4*)(kptr + 8 * G::T_STRIDE));
-                    const V8 bk = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                    acc[cb] = Mma<T>::run(a, bk, acc[cb]);
-                    if (does_z) zacc[cb] = Mma<T>::run(ones, bk, zacc[cb]);
-                }
+                const V8 bk = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                acc = Mma<T>::run(a, bk, acc);
+                if (does_z) zacc = Mma<T>::run(ones, bk, zacc);
             }
         }
         __syncthreads();
     }
 
+    // blocks -> FP32 image of (S, z) in LDS (rows of DP floats, then z), reusing the tile space
+    float* const Sl = reinterpret_cast<float*>(lds);
+    for (int i = tid; i < SG::S_FLOATS; i += kStateThreads) Sl[i] = 0.f;
+    __syncthreads();
     if (active) {
-        float* const S = p.ws + static_cast<long>(bh) * G::WS_FLOATS;
-        float* const z = S + D * D;
+        const int j = 32 * cb + lq;
 #pragma unroll
-        for (int cb = 0; cb < G::NB; ++cb) {
-            const int j = 32 * cb + lq;
-            if (j < D) {
+        for (int bb = 0; bb < 4; ++bb)
 #pragma unroll
-                for (int bb = 0; bb < 4; ++bb)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int i = 32 * rb + 8 * bb + 4 * lh + e;
-                        if (i < D) atomicAdd(S + i * D + j, acc[cb][4 * bb + e]);
-                    }
-                if (does_z && lh == 0) atomicAdd(z + j, zacc[cb][0]);
+            for (int e = 0; e < 4; ++e) {
+                const int i = 32 * rb + 8 * bb + 4 * lh + e;
+                if constexpr (SG::NTS > 1) atomicAdd(Sl + i * G::DP + j, acc[4 * bb + e]);
+                else Sl[i * G::DP + j] = acc[4 * bb + e];
             }
+        if (does_z && lh == 0) {
+            if constexpr (SG::NTS > 1) atomicAdd(Sl + G::DP * G::DP + j, zacc[0]);
+            else Sl[G::DP * G::DP + j] = zacc[0];
         }
+    }
+    __syncthreads();
+    // this group's (S, z): straight into the state when it covers the whole (batch, head), else into its partial slot
+    float* const S = p.part ? p.part + (static_cast<long>(bh) * p.n_part + chunk) * G::WS_FLOATS
+                            : p.ws + static_cast<long>(bh) * G::WS_FLOATS;
+    for (int idx = tid; idx < (D + 1) * (D / 4); idx += kStateThreads) {
+        const int i = idx / (D / 4), j = (idx - i * (D / 4)) * 4;     // i == D: the z row, kept behind the DP rows of S
+        f32x4 v = *reinterpret_cast<const f32x4*>(Sl + (i < D ? i : G::DP) * G::DP + j);
+        if (p.add_to_state) v += *reinterpret_cast<const f32x4*>(S + i * D + j);   // the only group of this (batch, head)
+        *reinterpret_cast<f32x4*>(S + i * D + j) = v;
+    }
+}
+
+// state (+)= sum of the partial states of the token chunks, one element per thread and step.
+__global__ void __launch_bounds__(256) linattn_reduce_kernel(float* ws, const float* part, int n_part, long ws_floats4, long total4,
+                                                             int accumulate) {
+    for (long i = blockIdx.x * 256L + threadIdx.x; i < total4; i += gridDim.x * 256L) {
+        const long bh = i / ws_floats4, off = i - bh * ws_floats4;
+        f32x4 v = accumulate ? reinterpret_cast<const f32x4*>(ws)[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int c = 0; c < n_part; ++c) v += reinterpret_cast<const f32x4*>(part)[(bh * n_part + c) * ws_floats4 + off];
+        reinterpret_cast<f32x4*>(ws)[i] = v;
     }
 }
 
 // ── apply: O = (S relu(Q)) / (z . relu(Q) + eps) ──
+// S sits in LDS as 16-bit A operand for the whole group. Tokens go through in tiles of 128 (32 per wavefront, one per
+// lane pair): the Q rows are fetched with full-row coalescing (the next tile is in flight in registers), ReLU'd and
+// staged in LDS, where each lane picks the B-operand fragments of its own token; the denominator is an exact FP32
+// dot of z with those values plus one exchange between lanes l and l^32. Results leave through the same LDS tile so
+// that the stores are full 16-byte chunks of contiguous row segments.
 template <typename T, int D>
 __global__ void __launch_bounds__(kThreads) linattn_apply_kernel(const LinDev p) {
     using G = LGeo<D>;
     using V8 = typename Mma<T>::v8;
+    constexpr int TM = 128;                       // tokens per tile
+    constexpr int NQ = (TM * G::CPR + kThreads - 1) / kThreads;
     __shared__ __attribute__((aligned(16))) unsigned char Ss[G::DP * G::S_STRIDE];
+    __shared__ __attribute__((aligned(16))) unsigned char Qs[TM * G::S_STRIDE];
     __shared__ __attribute__((aligned(16))) float Zs[G::DP];
 
-    const int bh = blockIdx.y;
+    int bh, chunk;
+    if (!lin_block(p, bh, chunk)) return;
     const int b = bh / p.H, h = bh % p.H;
-    const int n_begin = blockIdx.x * p.tokens_per_group;
+    const int n_begin = chunk * p.tokens_per_group;
     const int n_end = min(p.N, n_begin + p.tokens_per_group);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int lq = lane & 31, lh = lane >> 5;
@@ -218,33 +290,66 @@ __global__ void __launch_bounds__(kThreads) linattn_apply_kernel(const LinDev p)
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
     const float* const S = p.ws + static_cast<long>(bh) * G::WS_FLOATS;
     const float* const z = S + D * D;
+    const int last = n_end - 1;
 
-    // stage S (FP32 -> T) and z (FP32) in LDS; pad rows/columns are zero
-    for (int idx = tid; idx < G::DP * (G::DP / 4); idx += kThreads) {
-        const int i = idx / (G::DP / 4);
-        const int j = (idx - i * (G::DP / 4)) * 4;
-        f32x4 sv = {0.f, 0.f, 0.f, 0.f};
-        if (i < D && j < D) sv = *reinterpret_cast<const f32x4*>(S + i * D + j);
-        typedef T t4 __attribute__((ext_vector_type(4)));
-        t4 tv;
+    u32x4 qreg[NQ];
+    auto issue_q = [&](int n0) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) tv[e] = static_cast<T>(sv[e]);
-        *reinterpret_cast<t4*>(Ss + i * G::S_STRIDE + j * 2) = tv;
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = min(tid + kThreads * i, TM * G::CPR - 1);
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            qreg[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(min(n0 + row, last)) * p.q_rs + cc * 8);
+        }
+    };
+    issue_q(n_begin);
+
+    // stage S (FP32 -> T) and z (FP32) in LDS; pad rows/columns are zero. All loads are issued before the first
+    // conversion (pad positions read a clamped address and are blanked).
+    {
+        constexpr int NS = (G::DP * (G::DP / 4) + kThreads - 1) / kThreads;
+        f32x4 sv[NS];
+#pragma unroll
+        for (int t = 0; t < NS; ++t) {
+            const int idx = min(tid + kThreads * t, G::DP * (G::DP / 4) - 1);
+            const int i = idx / (G::DP / 4), j = (idx - i * (G::DP / 4)) * 4;
+            sv[t] = *reinterpret_cast<const f32x4*>(S + min(i, D - 1) * D + min(j, D - 4));
+        }
+#pragma unroll
+        for (int t = 0; t < NS; ++t) {
+            const int idx = tid + kThreads * t;
+            const int i = idx / (G::DP / 4), j = (idx - i * (G::DP / 4)) * 4;
+            typedef T t4 __attribute__((ext_vector_type(4)));
+            t4 tv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tv[e] = (i < D && j < D) ? static_cast<T>(sv[t][e]) : static_cast<T>(0.f);
+            if (idx < G::DP * (G::DP / 4)) *reinterpret_cast<t4*>(Ss + i * G::S_STRIDE + j * 2) = tv;
+        }
     }
     for (int j = tid; j < G::DP; j += kThreads) Zs[j] = j < D ? z[j] : 0.f;
-    __syncthreads();
+    if constexpr (G::DP > D) {  // pad chunks of the Q tile stay zero
+        constexpr int PC = (G::DP - D) / 8;
+        for (int i = tid; i < TM * PC; i += kThreads)
+            *reinterpret_cast<u32x4*>(Qs + (i / PC) * G::S_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
+    }
 
-    for (int n0 = n_begin + wave * 32; n0 < n_end; n0 += 4 * 32) {
-        const int n = n0 + lq;
-        const bool valid = n < n_end;
+    for (int n0 = n_begin; n0 < n_end; n0 += TM) {
+        // Q tile: registers -> LDS (ReLU on the way), then the next tile's loads
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = tid + kThreads * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < TM * G::CPR) *reinterpret_cast<u32x4*>(Qs + row * G::S_STRIDE + cc * 16) = relu8<T>(qreg[i]);
+        }
+        __syncthreads();
+        if (n0 + TM < n_end) issue_q(n0 + TM);
+
+        const int trow = wave * 32 + lq;          // this lane's token within the tile
         V8 qf[G::KC];
         float den = 0.f;
 #pragma unroll
         for (int c = 0; c < G::KC; ++c) {
             const int d0 = 16 * c + 8 * lh;
-            u32x4 raw = {0, 0, 0, 0};
-            if (valid && d0 < D) raw = relu8<T>(*reinterpret_cast<const u32x4*>(q_base + static_cast<long>(n) * p.q_rs + d0));
-            qf[c] = __builtin_bit_cast(V8, raw);
+            qf[c] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Qs + trow * G::S_STRIDE + d0 * 2));
             const f32x4 z0 = *reinterpret_cast<const f32x4*>(Zs + d0);
             const f32x4 z1 = *reinterpret_cast<const f32x4*>(Zs + d0 + 4);
 #pragma unroll
@@ -264,6 +369,7 @@ __global__ void __launch_bounds__(kThreads) linattn_apply_kernel(const LinDev p)
         // the reference forms the reciprocal as rsqrt(den + eps)^2 in FP32
         const float rs = __builtin_amdgcn_rsqf(den + p.eps);
         const float recip = rs * rs;
+        __syncthreads();                          // every lane holds its fragments: the tile can take the results
 #pragma unroll
         for (int rb = 0; rb < G::NB; ++rb) {
             f32x16 acc;
@@ -274,57 +380,90 @@ __global__ void __launch_bounds__(kThreads) linattn_apply_kernel(const LinDev p)
                 const u32x4 a = *reinterpret_cast<const u32x4*>(Ss + (32 * rb + lq) * G::S_STRIDE + (16 * c + 8 * lh) * 2);
                 acc = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], acc);
             }
-            if (valid) {
 #pragma unroll
-                for (int bb = 0; bb < 4; ++bb) {
-                    const int i0 = 32 * rb + 8 * bb + 4 * lh;
-                    if (i0 < D) {
-                        typedef T t4 __attribute__((ext_vector_type(4)));
-                        t4 ov;
+            for (int bb = 0; bb < 4; ++bb) {
+                const int i0 = 32 * rb + 8 * bb + 4 * lh;
+                typedef T t4 __attribute__((ext_vector_type(4)));
+                t4 ov;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(acc[4 * bb + e] * recip);
-                        *reinterpret_cast<t4*>(o_base + static_cast<long>(n) * p.o_rs + i0) = ov;
-                    }
-                }
+                for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(acc[4 * bb + e] * recip);
+                *reinterpret_cast<t4*>(Qs + trow * G::S_STRIDE + i0 * 2) = ov;
             }
         }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = tid + kThreads * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < TM * G::CPR && n0 + row <= last)
+                *reinterpret_cast<u32x4*>(o_base + static_cast<long>(n0 + row) * p.o_rs + cc * 8) =
+                    *reinterpret_cast<const u32x4*>(Qs + row * G::S_STRIDE + cc * 16);
+        }
+        if constexpr (G::DP > D) {
+            // the results overwrote the zero pad chunks of the tile (value channels D..DP-1 are zero anyway: the pad
+            // rows of S are zero), nothing to restore
+        }
+        __syncthreads();
     }
 }
 
 template <typename T, int D>
-int launch_d(LinDev p, bool accumulate, int n_cu, hipStream_t st) {
+int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st) {
     using G = LGeo<D>;
     const int BH = p.B * p.H;
-    if (!accumulate) {
-        const long n = static_cast<long>(BH) * G::WS_FLOATS;
-        const int blocks = static_cast<int>(std::min<long>((n + 255) / 256, 2048));
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, st, p.ws, n);
+    // State pass. The tokens of a head are split over enough groups to keep most CUs streaming, if the caller lent a
+    // scratch for the partial states; each group needs a few tiles to amortise its prologue and epilogue.
+    {
+        LinDev ps = p;
+        const int tiles = (ps.N + kStateTile - 1) / kStateTile;
+        int split = 1;
+        while (split * 2 <= max_split && BH * split * 2 <= n_cu && tiles / (split * 2) >= 2) split *= 2;
+#ifdef MI_EXPERIMENT_LIN_SPLIT
+        if (const char* e = getenv("MI_LIN_SPLIT")) split = std::max(1, std::min(atoi(e), max_split));
+#endif
+        ps.tokens_per_group = ((tiles + split - 1) / split) * kStateTile;
+        ps.n_chunks = (ps.N + ps.tokens_per_group - 1) / ps.tokens_per_group;
+        ps.n_blocks = BH * ps.n_chunks;
+        const bool partials = max_split > 0 && (accumulate || ps.n_chunks > 1);
+        ps.part = partials ? p.part : nullptr;
+        ps.n_part = ps.n_chunks;
+        ps.add_to_state = (!partials && accumulate) ? 1 : 0;
+        hipLaunchKernelGGL((linattn_state_kernel<T, D>), dim3(((ps.n_blocks + 7) / 8) * 8), dim3(kStateThreads),
+                           StateGeo<D>::LDS_BYTES, st, ps);
+        if (partials) {
+            const long ws4 = G::WS_FLOATS / 4, total4 = static_cast<long>(BH) * ws4;   // D is a multiple of 8: whole 16-byte pieces
+            const int blocks = static_cast<int>(std::min<long>((total4 + 255) / 256, 2048));
+            hipLaunchKernelGGL(linattn_reduce_kernel, dim3(blocks), dim3(256), 0, st, p.ws, p.part, ps.n_part, ws4, total4,
+                               accumulate ? 1 : 0);
+        }
     }
-    // enough groups to fill the chip about twice over, chunks a multiple of the 64-token tile
-    auto pick = [&](int min_tokens) {
-        int t = min_tokens;
-        while (static_cast<long>(BH) * ((p.N + t - 1) / t) > 4L * n_cu && t < p.N) t *= 2;
+    // Apply pass: chunks are multiples of the tile; two resident work groups per CU hide each other's latencies, beyond
+    // that larger chunks keep the staging of S small against the streamed tokens.
+    auto pick = [&](int tile, int min_tiles) {
+        int t = tile * min_tiles;
+        while (t < p.N && static_cast<long>(BH) * ((p.N + 2 * t - 1) / (2 * t)) >= 2L * n_cu) t *= 2;
         return t;
     };
-    p.tokens_per_group = pick(128);
-    hipLaunchKernelGGL((linattn_state_kernel<T, D>), dim3((p.N + p.tokens_per_group - 1) / p.tokens_per_group, BH),
-                       dim3(kThreads), 0, st, p);
-    p.tokens_per_group = pick(128);
-    hipLaunchKernelGGL((linattn_apply_kernel<T, D>), dim3((p.N + p.tokens_per_group - 1) / p.tokens_per_group, BH),
-                       dim3(kThreads), 0, st, p);
+    auto grid_of = [&](LinDev& q) {
+        q.n_chunks = (q.N + q.tokens_per_group - 1) / q.tokens_per_group;
+        q.n_blocks = BH * q.n_chunks;
+        return dim3(((q.n_blocks + 7) / 8) * 8);
+    };
+    p.tokens_per_group = pick(128, 1);
+    hipLaunchKernelGGL((linattn_apply_kernel<T, D>), grid_of(p), dim3(kThreads), 0, st, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("mi_linear_attn_relu_forward launch: %s", hipGetErrorString(e));
     return 0;
 }
 
 template <typename T>
-int launch_t(const LinDev& p, int d, bool acc, int n_cu, hipStream_t st) {
+int launch_t(const LinDev& p, int d, bool acc, int max_split, int n_cu, hipStream_t st) {
     switch (d) {
-        case 32: return launch_d<T, 32>(p, acc, n_cu, st);
-        case 64: return launch_d<T, 64>(p, acc, n_cu, st);
-        case 72: return launch_d<T, 72>(p, acc, n_cu, st);
-        case 112: return launch_d<T, 112>(p, acc, n_cu, st);
-        case 128: return launch_d<T, 128>(p, acc, n_cu, st);
+        case 32: return launch_d<T, 32>(p, acc, max_split, n_cu, st);
+        case 64: return launch_d<T, 64>(p, acc, max_split, n_cu, st);
+        case 72: return launch_d<T, 72>(p, acc, max_split, n_cu, st);
+        case 112: return launch_d<T, 112>(p, acc, max_split, n_cu, st);
+        case 128: return launch_d<T, 128>(p, acc, max_split, n_cu, st);
         default: return fail("mi_linear_attn_relu_forward: head_dim %d has no kernel (32, 64, 72, 112, 128)", d);
     }
 }
@@ -348,6 +487,10 @@ size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, int32_t 
     return static_cast<size_t>(batch) * num_heads * (static_cast<size_t>(head_dim) * head_dim + head_dim) * sizeof(float);
 }
 
+size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim) {
+    return mi_linear_attn_workspace_bytes(batch, num_heads, head_dim) * mi::kMaxStateSplit;
+}
+
 int mi_linear_attn_relu_forward(const mi_linear_attn_args* a) {
     using mi::fail;
     mi::clear_error();
@@ -361,6 +504,12 @@ int mi_linear_attn_relu_forward(const mi_linear_attn_args* a) {
     const size_t need = mi_linear_attn_workspace_bytes(a->batch, a->num_heads, a->head_dim);
     if (!a->workspace || a->workspace_bytes < need)
         return fail("mi_linear_attn_relu_forward: workspace needs %zu bytes (got %zu)", need, a->workspace ? a->workspace_bytes : 0);
+    // the scratch decides how far the tokens of a head may be split over work groups (one partial state per chunk)
+    int max_split = 0;
+    if (a->scratch) {
+        if (reinterpret_cast<uintptr_t>(a->scratch) & 15u) return fail("mi_linear_attn_relu_forward: scratch must be 16-byte aligned");
+        max_split = static_cast<int>(std::min<size_t>(a->scratch_bytes / need, mi::kMaxStateSplit));
+    }
     const long D = static_cast<long>(a->num_heads) * a->head_dim;
     mi::LinDev p;
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
@@ -381,10 +530,11 @@ int mi_linear_attn_relu_forward(const mi_linear_attn_args* a) {
     if (al & 15u) return fail("mi_linear_attn_relu_forward: pointers must be 16-byte aligned");
     p.eps = a->eps;
     p.ws = static_cast<float*>(a->workspace);
+    p.part = max_split > 0 ? static_cast<float*>(a->scratch) : nullptr; p.n_part = 0; p.add_to_state = 0;
     p.tokens_per_group = 0;
     hipStream_t st = mi::resolve_stream(a->stream);
     const int n_cu = mi::device_cu_count();
-    return mi::launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, n_cu, st);
+    return mi::launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, max_split, n_cu, st);
 }
 
 }  // extern "C"

@@ -99,7 +99,7 @@ void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, i
 }
 
 void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
-                                   Tensor& state, Tensor& out, bool accumulate_state) {
+                                   Tensor& state, Tensor& out, bool accumulate_state, Tensor* scratch) {
     const char* op = "linear_attention_relu_forward";
     need_gpu(op, Q); need_gpu(op, K); need_gpu(op, V);
     if (num_heads <= 0 || Q.cols % num_heads != 0) fail(std::string(op) + ": D must equal head_dim * num_heads");
@@ -123,6 +123,12 @@ void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tenso
     a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.n_tokens = Q.rows;
     a.eps = eps; a.accumulate_state = accumulate_state ? 1 : 0;
     a.workspace = state.data; a.workspace_bytes = state.bytes();
+    if (scratch) {
+        const std::size_t need = mi_linear_attn_scratch_bytes(1, num_heads, hd);
+        if (scratch->data == nullptr || scratch->bytes() < need || scratch->dtype != Dtype::FP32)
+            scratch->resize(1, static_cast<int>(need / 4), Dtype::FP32, Q.device);
+        a.scratch = scratch->data; a.scratch_bytes = scratch->bytes();
+    }
     check(op, mi_linear_attn_relu_forward(&a));
 }
 

@@ -24,9 +24,11 @@ void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_
 void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
 
 // Sana's ReLU linear-attention core on token-major (N, heads*head_dim) operands
-// (src/dit/sana.cpp:470-586). `state` receives the FP32 (S, z) blocks, heads x (d*d + d).
+// (src/dit/sana.cpp:470-586). `state` receives the FP32 (S, z) blocks, heads x (d*d + d). `scratch` (optional,
+// caller-owned like the reference's scratch tensors, sized on first use) holds partial states so that the state pass
+// can spread the tokens of a head over the whole GPU.
 void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
-                                   Tensor& state, Tensor& out, bool accumulate_state = false);
+                                   Tensor& state, Tensor& out, bool accumulate_state = false, Tensor* scratch = nullptr);
 
 }  // namespace bt
 

@@ -280,12 +280,14 @@ def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num
 
 
 def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
-                                  workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False):
+                                  workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False,
+                                  scratch: Optional[torch.Tensor] = None):
     """Sana's ReLU linear attention core (src/dit/sana.cpp:470-586) on token-major (N, heads*head_dim)
     or (batch, N, heads*head_dim) operands. `workspace` (float32, batch*heads*(d*d+d)) receives the
-    (S, z) state; pass it to capture the state or, with accumulate_state, to inject one."""
+    (S, z) state; pass it to capture the state or, with accumulate_state, to inject one. `scratch` (float32) holds
+    partial states of token chunks; None allocates one, False runs without (one work group per batch item and head)."""
     op = "linear_attention_relu_forward"
-    _dev(op, Q, K, V, out, workspace)
+    _dev(op, Q, K, V, out, workspace, scratch if scratch is not False else None)
     dt = _dtype_code(op, Q)
     if K.dtype != Q.dtype or V.dtype != Q.dtype:
         _fail(op, "Q, K, V must share one dtype")
@@ -319,6 +321,15 @@ def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.T
     a.eps = eps
     a.accumulate_state = int(accumulate_state)
     a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * 4
+    if scratch is False:
+        scratch = torch.empty(0, dtype=torch.float32, device=Q.device)      # explicitly none: one work group per (batch, head)
+    if scratch is None:
+        # partial states of the token chunks (lets the state pass use the whole GPU); comes from torch's caching allocator
+        scratch = torch.empty(capi.lib().mi_linear_attn_scratch_bytes(B, num_heads, hd) // 4, dtype=torch.float32, device=Q.device)
+    if scratch.dtype != torch.float32 or not scratch.is_contiguous():
+        _fail(op, "scratch must be contiguous float32")
+    if scratch.numel() > 0:
+        a.scratch, a.scratch_bytes = scratch.data_ptr(), scratch.numel() * 4
     a.stream = _stream()
     capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
     return out

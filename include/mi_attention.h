@@ -181,7 +181,11 @@ MI_API int mi_rope_apply(const mi_rope_args* args);
  * ((batch*heads) blocks of head_dim*head_dim + head_dim floats, S row-major with rows =
  * value channel, then z): after the call it holds the (S, z) the reference captures at
  * its identity seam (sana.cpp:489-506). accumulate_state != 0 adds this call's (S, z) to
- * what the workspace already holds instead of starting from zero (the inject form). */
+ * what the workspace already holds instead of starting from zero (the inject form).
+ * `scratch` (optional, FP32, up to mi_linear_attn_scratch_bytes) lets the state pass split the
+ * tokens of a head over several work groups, one partial state each, summed by a small
+ * reduction: several times faster at image sizes. Without it one work group streams all
+ * tokens of a (batch, head). Results are deterministic either way (no atomics). */
 typedef struct mi_linear_attn_args {
     uint32_t struct_size;
     int32_t dtype;
@@ -198,9 +202,12 @@ typedef struct mi_linear_attn_args {
     int32_t accumulate_state;
     void* workspace;
     size_t workspace_bytes;
+    void* scratch;          /* device, 16-byte aligned, or NULL */
+    size_t scratch_bytes;
     void* stream;
 } mi_linear_attn_args;
 MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
+MI_API size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API int mi_linear_attn_relu_forward(const mi_linear_attn_args* args);
 MI_API int mi_linear_attn_supported(int32_t dtype, int32_t head_dim);
 

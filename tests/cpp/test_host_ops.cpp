@@ -173,7 +173,8 @@ static void gpu_checks() {
         const std::vector<float> ql = randn_bf16(7011, static_cast<size_t>(N) * Dl), kl = randn_bf16(7012, static_cast<size_t>(N) * Dl),
                                  vl = randn_bf16(7013, static_cast<size_t>(N) * Dl);
         Tensor Ql = upload_bf16(ql, N, Dl), Kl = upload_bf16(kl, N, Dl), Vl = upload_bf16(vl, N, Dl), state, out;
-        bt::linear_attention_relu_forward(Ql, Kl, Vl, Hl, 1e-15f, state, out);
+        Tensor scratch;
+        bt::linear_attention_relu_forward(Ql, Kl, Vl, Hl, 1e-15f, state, out, false, &scratch);
         std::vector<float> ref(ql.size());
         orc_linear_attn_relu(ql.data(), kl.data(), vl.data(), N, Hl, dl, 1e-15f, ref.data(), nullptr, nullptr, 0);
         const Err e = compare(ref, download_bf16(out));

@@ -93,6 +93,7 @@ def test_argument_validation_without_launch(capi):
     l.q = l.k = l.v = l.o = 0x1000
     assert lib.mi_linear_attn_relu_forward(C.byref(l)) == -1 and "workspace needs" in capi.last_error()
     assert lib.mi_linear_attn_workspace_bytes(2, 20, 112) == 2 * 20 * (112 * 112 + 112) * 4
+    assert lib.mi_linear_attn_scratch_bytes(2, 20, 112) % lib.mi_linear_attn_workspace_bytes(2, 20, 112) == 0
 
 
 def test_python_mirror_refuses_cpu_tensors():
