@@ -26,8 +26,8 @@ sys.path.insert(0, ROOT)
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --traffic-probe`: (69290 KiB x 2.00 calibration) fetched + 27648 KiB written.
-TRAFFIC_BYTES_PER_LAUNCH = (69290 * 2 + 27648) * 1024
+# `bench.py --traffic-probe`: (69372 KiB x 2.00 calibration) fetched + 27648 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (69372 * 2 + 27648) * 1024
 
 
 def parse():
@@ -110,8 +110,9 @@ def all_configs(torch, bd):
     for name, n in (("cfg5a_sana_linear_n1024_d112_bf16", 1024), ("cfg5b_sana_linear_n4096_d112_bf16", 4096)):
         ql, kl, vl_ = (rnd(2, n, 2240) for _ in range(3))
         ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
+        sc = torch.empty(8 * ws.numel(), dtype=torch.float32, device="cuda")     # partial states (mi_linear_attn_scratch_bytes)
         o = torch.empty_like(ql)
-        mn, av = event_ms(torch, lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws), 20)
+        mn, av = event_ms(torch, lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc), 20)
         nbytes = 4 * 2 * n * 2240 * 2
         out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16 in, f32 accumulate",

@@ -12,7 +12,6 @@
 //                 global memory; the denominator is an exact FP32 dot of z with the lane's own Q
 //                 values plus one exchange between lanes l and l^32.
 #include <algorithm>
-#include <cstdlib>
 
 #include "internal.h"
 
@@ -418,9 +417,6 @@ int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st)
         const int tiles = (ps.N + kStateTile - 1) / kStateTile;
         int split = 1;
         while (split * 2 <= max_split && BH * split * 2 <= n_cu && tiles / (split * 2) >= 2) split *= 2;
-#ifdef MI_EXPERIMENT_LIN_SPLIT
-        if (const char* e = getenv("MI_LIN_SPLIT")) split = std::max(1, std::min(atoi(e), max_split));
-#endif
         ps.tokens_per_group = ((tiles + split - 1) / split) * kStateTile;
         ps.n_chunks = (ps.N + ps.tokens_per_group - 1) / ps.tokens_per_group;
         ps.n_blocks = BH * ps.n_chunks;

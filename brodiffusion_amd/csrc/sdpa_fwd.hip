@@ -440,7 +440,8 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
             }
             // Always the full stream: at t = -1 P is zero and the (zero-filled) V buffer adds nothing;
             // after the last tile the extra scores are never read. This wavefront's share of the tile
-            // movement rides along in the stream.
+            // movement rides along in the stream (measured faster than in front of the softmax: the stores
+            // and loads issue in the shadow of the matrix pipe).
             mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
                                           [&]() { advance_tiles(t + 2, t + 1); }, &neg_ref);
             if (grp == 0) {
