@@ -459,29 +459,47 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
 }
 
-// ─────────────── 8-wavefront ping-pong kernel, head_dim 128, tiles by LDS DMA ───────────────
+// ─────────────── 8-wavefront kernel with tiles by LDS DMA ───────────────
 // Same schedule as sdpa_fwd_pp_kernel, but K/V tiles go from global memory straight into LDS
 // (global_load_lds_dwordx4: lane i of a wavefront deposits its 16 bytes at base + 16*i), so tile
-// movement costs no registers and no LDS store instructions.
-// A DMA instruction writes 1024 contiguous bytes = 4 unpadded 256-byte rows, so bank conflicts are
-// avoided by an XOR swizzle instead of row padding: 16-byte chunk c of row r lives at chunk position
-// c ^ f(r), f(r) = 4*(r%4) + (r/4)%4. The swizzle is applied for free on the global side (each lane
-// fetches the chunk that belongs in its LDS slot) and undone in the LDS read addresses:
-//   K reads (one row per lane, 16 consecutive rows): f takes 16 distinct values -> 16 distinct slots
-//   V transpose reads (4 rows x 64 bytes per 32 lanes): rows r%4 = 0..3 land in distinct 64-byte windows
+// movement costs no registers and no LDS store instructions. A DMA instruction writes 1024 contiguous
+// bytes, so rows sit in LDS back to back without padding; a 64-key tile is D/8 such instructions per
+// operand, dealt out to the 8 wavefronts in turn. Bank conflicts of the unpadded rows:
+//   head_dim 128 (256-byte rows): avoided by an XOR swizzle, 16-byte chunk c of row r lives at chunk position
+//     c ^ f(r), f(r) = 4*(r%4) + (r/4)%4, applied for free on the global side (each lane fetches the chunk that
+//     belongs in its LDS slot) and undone in the LDS read addresses: K reads (one row per lane, 16 consecutive
+//     rows) hit 16 distinct slots, V transpose reads (4 rows x 64 bytes per 32 lanes) 4 distinct 64-byte windows;
+//   head_dim 72 (144-byte rows): 16 consecutive rows start on 16 distinct multiples of 4 banks, so the K reads are
+//     conflict-free as they are; the V transpose reads overlap a little.
+// Without padding, the fragment reads of the zero-padded part of the head dimension (columns D..DK-1 of K,
+// D..DV-1 of V) run into the first bytes of the next row: real key rows (rows past the end of a segment are fetched
+// from its last row), multiplied by the zero pad of Q, or producing output columns that are never stored. A little
+// zero-filled slack behind each ring keeps the reads of the last row inside the allocation.
 // Tiles are ring-buffered three deep: the loads of K_{t+3}, V_{t+2} are issued in step t, awaited at
 // the end of step t+1 and read in step t+2. The key loop is unrolled by three so that every LDS offset
 // is an instruction immediate; tile pointers advance incrementally in scalar registers.
-// Rows past the end of a segment are fetched from its last row (valid memory); their scores are masked.
 constexpr int kDmaStages = 3;
-constexpr int kRowBytes128 = 256;
-constexpr int kTileBytes128 = kBN * kRowBytes128;   // 16 KB per operand tile
-constexpr int kVbufOff128 = kDmaStages * kTileBytes128;
-constexpr int lds_bytes_dma() {
-    const int kv = 2 * kDmaStages * kTileBytes128;
-    const int o = 256 * HeadGeo<128>::O_STRIDE;
-    return kv > o ? kv : o;
-}
+template <int D> struct DmaGeo {
+    using G = HeadGeo<D>;
+    static constexpr int ROWB = D * 2;                       // bytes per row in LDS (no padding)
+    static constexpr int TILE = kBN * ROWB;                  // = (D / 8) KB
+    static constexpr int NDMA = TILE / 1024;                 // DMA instructions per operand tile
+    static constexpr int SLACK = 256;                        // zero bytes behind each ring
+    static constexpr int RING = kDmaStages * TILE + SLACK;
+    static constexpr int VOFF = RING;
+    static constexpr int MAXI = (2 * NDMA + 7) / 8;          // most DMA instructions of one wavefront per step
+    static constexpr bool SWZ = D == 128;
+    static constexpr int lds_bytes() {
+        const int kv = 2 * RING;
+        const int o = 256 * G::O_STRIDE;
+        return kv > o ? kv : o;
+    }
+    // the staged Q tile (finite values) covers the whole K ring before the first key tile arrives, so the pad reads
+    // described above never meet uninitialised LDS
+    static_assert(256 * G::O_STRIDE >= RING, "Q staging must cover the K ring");
+};
+// (head_dim 40 works the same way but measured no faster than the register-staged kernel: not instantiated)
+template <int D> constexpr bool dma_kernel_available() { return D == 72 || D == 128; }
 
 __device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2) & 3); }
 
@@ -513,10 +531,10 @@ struct TileCursor {
     }
 };
 
-template <typename T>
+template <typename T, int D>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const SdpaDev p) {
-    constexpr int D = 128;
     using G = HeadGeo<D>;
+    using DG = DmaGeo<D>;
     using V8 = typename Mma<T>::v8;
     constexpr int BM = 256;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -552,9 +570,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     __syncthreads();
     read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
     __syncthreads();
-    // the first pass through the MFMA stream multiplies a zero P with the last V buffer
-    for (int i = tid; i < kTileBytes128 / 16; i += kThreads8)
-        *reinterpret_cast<u32x4*>(smem + kVbufOff128 + (kDmaStages - 1) * kTileBytes128 + i * 16) = u32x4{0, 0, 0, 0};
+    // the first pass through the MFMA stream multiplies a zero P with the last V buffer; the slack behind both rings is zero
+    for (int i = tid; i < (DG::TILE + DG::SLACK) / 16; i += kThreads8)
+        *reinterpret_cast<u32x4*>(smem + DG::VOFF + (kDmaStages - 1) * DG::TILE + i * 16) = u32x4{0, 0, 0, 0};
+    for (int i = tid; i < DG::SLACK / 16; i += kThreads8)
+        *reinterpret_cast<u32x4*>(smem + kDmaStages * DG::TILE + i * 16) = u32x4{0, 0, 0, 0};
     __syncthreads();
     int g_lo = red[0], kv_stop = red[8];
 #pragma unroll
@@ -575,33 +595,68 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
 #pragma unroll
     for (int e = 0; e < 16; ++e) neg_ref[e] = 0.f;
 
-    // ── DMA source geometry of this lane: LDS slot (row 4*wave + lane/16 [+32], position lane%16) ──
+    // ── DMA duty of this wavefront: instructions i = wave, wave + 8, ... of the list [K 0..NDMA-1, V 0..NDMA-1];
+    //    instruction j of an operand fills LDS bytes [1024 j, 1024 j + 1024) of the tile = chunks 64 j + lane ──
     TileCursor kc, vc;
     kc.init(plan, reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D), static_cast<unsigned>(p.kp_rs) * 2u,
             reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D), static_cast<unsigned>(p.k_rs) * 2u, p.Lp);
     vc.init(plan, reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D), static_cast<unsigned>(p.vp_rs) * 2u,
             reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D), static_cast<unsigned>(p.v_rs) * 2u, p.Lp);
-    const int drow = 4 * wave + (lane >> 4);
-    const unsigned dchunk = ((lane & 15) ^ swz(drow)) * 16u;   // chunk this slot must receive (same for row + 32)
-    // One DMA instruction: rows (drow + 32*half) of the cursor's tile into LDS at lds_off + 1024*wave + 8192*half.
-    // Written as inline assembly on purpose: for the compiler's builtin every later LDS read may alias
-    // the DMA's LDS write, so it waits for the load to land (vmcnt(0)) before the next ds_read and the
-    // whole memory latency ends up inside the MFMA stream. The tiles written here are never read before
-    // the explicit wait + barrier at the end of the following VALU phase.
+    int drow[DG::MAXI];        // tile row this lane fetches in its m-th instruction
+    unsigned dcol[DG::MAXI];   // byte offset inside that row
+#pragma unroll
+    for (int m = 0; m < DG::MAXI; ++m) {
+        const int i = wave + 8 * m;
+        const int j = i < DG::NDMA ? i : i - DG::NDMA;
+        const int g = 64 * j + lane;
+        const int row = g / G::CPR;
+        int cc = g - row * G::CPR;
+        if constexpr (DG::SWZ) cc ^= swz(row);     // the chunk this slot must receive
+        drow[m] = row;
+        dcol[m] = static_cast<unsigned>(cc) * 16u;
+    }
+    // One DMA instruction. Written as inline assembly on purpose: for the compiler's builtin every later LDS read may
+    // alias the DMA's LDS write, so it waits for the load to land (vmcnt(0)) before the next ds_read. The tiles
+    // written here are never read before the explicit wait + barrier at the end of the following step.
     const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)smem));
-    auto dma = [&](const TileCursor& c, int half, int lds_off) {
-        const int row = min(drow + 32 * half, min(c.rows_left, kBN) - 1);
-        const unsigned voff = static_cast<unsigned>(row) * c.rsb + dchunk;
-        const unsigned dst = lds_base + lds_off + wave * 1024 + half * 8192;
+    auto dma = [&](const TileCursor& c, int m, int j, int lds_off) {
+        const int row = min(drow[m], min(c.rows_left, kBN) - 1);
+        const unsigned voff = static_cast<unsigned>(row) * c.rsb + dcol[m];
+        const unsigned dst = lds_base + lds_off + j * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory");
     };
+    // this wavefront's share of the loads of one K tile (if do_k) and one V tile (if do_v); returns how many it issued
+    auto dma_tiles = [&](bool do_k, int k_off, bool do_v, int v_off) -> int {
+        int n = 0;
+#pragma unroll
+        for (int m = 0; m < DG::MAXI; ++m) {
+            const int i = wave + 8 * m;
+            if constexpr (DG::NDMA % 8 == 0) {
+                // every wavefront has the same duty: its first MAXI / 2 instructions are K, the others V
+                if (m < DG::MAXI / 2) { if (do_k) { dma(kc, m, i, k_off); ++n; } }
+                else { if (do_v) { dma(vc, m, i - DG::NDMA, v_off); ++n; } }
+            } else {
+                if (i < DG::NDMA) { if (do_k) { dma(kc, m, i, k_off); ++n; } }
+                else if (i < 2 * DG::NDMA) { if (do_v) { dma(vc, m, i - DG::NDMA, v_off); ++n; } }
+            }
+        }
+        return n;
+    };
+    auto wait_all_but = [&](int n) {     // loads complete in order: everything older than the last n has landed
+        if (n >= 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else if (n == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+        else if (n == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        else if (n == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    static_assert(DG::MAXI <= 4, "wait_all_but covers at most 4 loads per step");
 
-    // ── LDS read addresses in the swizzled layout (stage and block offsets are immediates) ──
-    // K fragment (kb, c): row 32kb + lq, chunk 2c + lh  ->  position (2c + lh) ^ f(lq)
+    // ── LDS read addresses (stage and block offsets are immediates) ──
+    // K fragment (kb, c): row 32kb + lq, chunk 2c + lh (at position (2c + lh) ^ f(lq) in the swizzled layout)
     const int fk = swz(lq);
     unsigned kaddr[G::KC];
 #pragma unroll
-    for (int c = 0; c < G::KC; ++c) kaddr[c] = lq * kRowBytes128 + (((2 * c + lh) ^ fk) << 4);
+    for (int c = 0; c < G::KC; ++c) kaddr[c] = lq * DG::ROWB + ((DG::SWZ ? ((2 * c + lh) ^ fk) : (2 * c + lh)) << 4);
     // V fragment (c4, vb), halves hh = 0, 1: key row 16c4 + 4lh + 8hh + trow, 8 bytes at head-dim 32vb + tcol
     const int trow = (lane & 15) >> 2;
     const int j4 = lane & 3;
@@ -613,7 +668,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         for (int hh = 0; hh < 2; ++hh) {
             const int row = 4 * lh + 8 * hh + trow;
             const int chunk = 4 * vb + 2 * g1 + (j4 >> 1);
-            vaddr[vb][hh] = kVbufOff128 + row * kRowBytes128 + ((chunk ^ swz(row)) << 4) + 8 * (j4 & 1);
+            vaddr[vb][hh] = DG::VOFF + row * DG::ROWB + ((DG::SWZ ? (chunk ^ swz(row)) : chunk) << 4) + 8 * (j4 & 1);
         }
 
     f32x16 sacc[2];
@@ -632,9 +687,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     //   loads K_{t+3} into K stage (S + 2) % 3 and V_{t+2} into V stage (S + 1) % 3.
     auto step = [&](auto stage_tag, int t) {
         constexpr int S = decltype(stage_tag)::value;
-        constexpr int KS = S * kTileBytes128, VS = ((S + 2) % 3) * kTileBytes128;
-        constexpr int KD = ((S + 2) % 3) * kTileBytes128, VD = kVbufOff128 + ((S + 1) % 3) * kTileBytes128;
+        constexpr int KS = S * DG::TILE, VS = ((S + 2) % 3) * DG::TILE;
+        constexpr int KD = ((S + 2) % 3) * DG::TILE, VD = DG::VOFF + ((S + 1) % 3) * DG::TILE;
         const bool load_k = t + 3 < n_tiles, load_v = t + 2 < n_tiles;
+        int issued = 0;
         auto softmax_of = [&](int tt) {
             if (tile_active(tt)) {
                 const int j0 = plan.j0(tt);
@@ -648,11 +704,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             }
         };
         // An LDS read issued behind an LDS-DMA load does not return before that load has landed (measured: the
-        // read takes the full memory latency), so the four DMA instructions of a step go where the wavefront
-        // has no LDS access ahead of it for a long time: right before its softmax.
+        // read takes the full memory latency), so the DMA instructions of a step go where the wavefront has no
+        // LDS access ahead of it for a long time: right before its softmax.
         auto issue_dma = [&]() {
-            if (load_k) { dma(kc, 0, KD); dma(kc, 1, KD); }
-            if (load_v) { dma(vc, 0, VD); dma(vc, 1, VD); }
+            issued = dma_tiles(load_k, KD, load_v, VD);
             if (load_k) kc.next();
             if (load_v) vc.next();
         };
@@ -669,15 +724,15 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 if (i < NPV) {
                     const int c4 = i / G::VB, vb = i % G::VB;
                     const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * kRowBytes128 + vaddr[vb][0]));
+                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * DG::ROWB + vaddr[vb][0]));
                     const s16x4 v_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * kRowBytes128 + vaddr[vb][1]));
+                        (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * DG::ROWB + vaddr[vb][1]));
                     const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
                     return __builtin_bit_cast(V8, a);
                 } else {
                     const int k = i - NPV;
                     const int kb = k / G::KC, c = k % G::KC;
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * kRowBytes128 + kaddr[c]);
+                    const u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * DG::ROWB + kaddr[c]);
                     return __builtin_bit_cast(V8, a);
                 }
             };
@@ -710,19 +765,24 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             softmax_of(t + 1);
         }
         // The tiles loaded in the PREVIOUS step are read in the next one: wait for those only (this step's
-        // loads stay in flight; loads complete in order), then meet the other wavefronts.
-        if (load_k) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else if (load_v) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // loads stay in flight), then meet the other wavefronts.
+        if constexpr (DG::NDMA % 8 == 0) {
+            // every wavefront issues NDMA / 8 loads per operand tile: the count follows from the flags alone
+            if (load_k) wait_all_but(DG::NDMA / 4);
+            else if (load_v) wait_all_but(DG::NDMA / 8);
+            else wait_all_but(0);
+        } else {
+            wait_all_but(issued);
+        }
         __syncthreads();
     };
 
     if (n_tiles > 0) {
         // prologue: K_0, K_1, V_0 (the loop loads K_{t+3}, V_{t+2} from t = -1 on); cursors end at K_2, V_1
-        dma(kc, 0, 0); dma(kc, 1, 0);
-        if (n_tiles > 1) { kc.next(); dma(kc, 0, kTileBytes128); dma(kc, 1, kTileBytes128); }
+        dma_tiles(true, 0, false, 0);
+        if (n_tiles > 1) { kc.next(); dma_tiles(true, DG::TILE, false, 0); }
         if (n_tiles > 2) kc.next();
-        dma(vc, 0, kVbufOff128); dma(vc, 1, kVbufOff128);
+        dma_tiles(false, 0, true, DG::VOFF);
         if (n_tiles > 1) vc.next();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -757,7 +817,10 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
         const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads8);
         if constexpr (D <= 128) {
             if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
-            else if (D == 128 && sdpa_kernel_choice() != 3) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T>), grid, block, lds_bytes_dma(), stream, p);
+            else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
+                if constexpr (dma_kernel_available<D>())
+                    hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
+            }
             else hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false>), grid, block, lds_bytes_8<D>(), stream, p);
         }
     } else {
