@@ -7,20 +7,23 @@ tests and the benchmark; PyTorch only provides device memory and streams.
 from .ops import (  # noqa: F401
     SdpaMask,
     build_axial_rope_tables,
+    build_qwen_rope_tables,
     device_info,
     flash_attention_forward,
     flash_attention_windowed_forward,
     gqa_attention_masked,
     joint_attention,
     linear_attention_relu_forward,
+    qwen_rope_positions,
     rope_apply,
     rope_apply_perhead,
+    rope_tables_from_positions,
     sdpa_forward,
     set_sdpa_kernel_choice,
 )
 
 __all__ = [
-    "SdpaMask", "build_axial_rope_tables", "device_info", "flash_attention_forward",
+    "SdpaMask", "build_axial_rope_tables", "build_qwen_rope_tables", "qwen_rope_positions", "rope_tables_from_positions", "device_info", "flash_attention_forward",
     "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
     "linear_attention_relu_forward", "rope_apply", "rope_apply_perhead", "sdpa_forward", "set_sdpa_kernel_choice",
 ]

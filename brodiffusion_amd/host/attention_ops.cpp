@@ -1,5 +1,6 @@
 #include "attention_ops.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 
@@ -164,6 +165,48 @@ RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, co
                 const double ang = (ax == 0 ? 0.0 : ax == 1 ? static_cast<double>(i) : static_cast<double>(j)) * omega[p];
                 cs[row * half + p] = static_cast<float>(std::cos(ang));
                 sn[row * half + p] = static_cast<float>(std::sin(ang));
+            }
+        }
+    RopeTables t;
+    t.cos = Tensor::from_host(cs.data(), static_cast<int>(L), half, Dtype::FP32);
+    t.sin = Tensor::from_host(sn.data(), static_cast<int>(L), half, Dtype::FP32);
+    return t;
+}
+
+RopeTables build_qwen_rope_tables(const std::vector<QwenSegment>& prefix, int hp, int wp, int head_dim,
+                                  const std::vector<int>& axes, float theta) {
+    if (head_dim % 2 != 0) fail("build_qwen_rope_tables: head_dim must be even");
+    if (axes.size() != 3 || axes[0] + axes[1] + axes[2] != head_dim) fail("build_qwen_rope_tables: three axes_dims_rope summing to head_dim");
+    // positions (frame, height, width) of every token, in sequence order
+    struct Pos { int f, h, w; };
+    std::vector<Pos> at;
+    int cursor = 0;
+    auto image = [&](int h, int w) {
+        const int top = -(h - h / 2), left = -(w - w / 2);
+        for (int i = 0; i < h; ++i)
+            for (int j = 0; j < w; ++j) at.push_back({cursor, top + i, left + j});
+        cursor += std::max(h, w);
+    };
+    for (const QwenSegment& s : prefix) {
+        if (s.kind == QwenSegment::Kind::Text) {
+            for (int i = 0; i < s.n_tokens; ++i, ++cursor) at.push_back({cursor, cursor, cursor});
+        } else {
+            image(s.h, s.w);
+        }
+    }
+    image(hp, wp);
+    const int half = head_dim / 2;
+    const std::size_t L = at.size();
+    std::vector<float> cs(L * half), sn(L * half);
+    int col = 0;
+    for (int a = 0; a < 3; ++a)
+        for (int p = 0; p < axes[a] / 2; ++p, ++col) {
+            const double omega = std::pow(static_cast<double>(theta), -2.0 * p / static_cast<double>(axes[a]));
+            for (std::size_t r = 0; r < L; ++r) {
+                const int x = a == 0 ? at[r].f : a == 1 ? at[r].h : at[r].w;
+                const double ang = static_cast<double>(x) * omega;
+                cs[r * half + col] = static_cast<float>(std::cos(ang));
+                sn[r * half + col] = static_cast<float>(std::sin(ang));
             }
         }
     RopeTables t;

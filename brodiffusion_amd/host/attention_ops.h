@@ -41,6 +41,20 @@ struct RopeTables {
 RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const std::vector<int>& axes_dims_rope,
                                    float theta = 10000.0f);
 
+// One segment of a Qwen-Image prefix as the table builder sees it (include/brodiffusion/dit/qwenimage21.h: QwenImage21Segment).
+struct QwenSegment {
+    enum class Kind { Text, Image } kind;
+    int n_tokens;   // Text
+    int h, w;       // Image
+};
+// 3-axis RoPE tables of the joint sequence [prefix segments ; target image hp x wp]
+// (QwenImage21Transformer2DModel::build_rope_tables_, src/dit/qwenimage21_forward.cpp:124-200): a shared running
+// position walks the sequence; a text token sits at (p, p, p) and advances it by one; an image block freezes the frame
+// axis, lays its tokens on a grid centred on zero and advances the position by max(h, w). A cached step uses the rows
+// of its target tokens (row_view).
+RopeTables build_qwen_rope_tables(const std::vector<QwenSegment>& prefix, int hp, int wp, int head_dim,
+                                  const std::vector<int>& axes_dims_rope, float theta = 10000.0f);
+
 // RoPE on Q and K, then full-bidirectional attention. Q is rotated while it is loaded; K is rotated
 // into Kr (resized to K's shape, holds RoPE(K) afterwards as in the reference) and read from there.
 // Qr is accepted and left untouched.

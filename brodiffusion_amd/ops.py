@@ -359,3 +359,48 @@ def build_axial_rope_tables(txt_len: int, hp: int, wp: int, head_dim: int, axes_
     cos = torch.from_numpy(np.cos(ang).astype(np.float32)).to(device)
     sin = torch.from_numpy(np.sin(ang).astype(np.float32)).to(device)
     return cos, sin
+
+
+def qwen_rope_positions(prefix_segments, hp: int, wp: int) -> np.ndarray:
+    """(3, L) integer positions (frame, height, width) of the Qwen-Image joint sequence [prefix segments ; target
+    image hp x wp] (src/dit/qwenimage21_forward.cpp:130-161). `prefix_segments` holds ("text", n) and
+    ("image", h, w) entries. A shared running position walks the sequence: a text token sits at (p, p, p) and
+    advances it by one; an image block freezes the frame axis at the current position, lays its tokens on a grid
+    centred on zero (first row at -(h - h//2)), then advances the position by max(h, w)."""
+    cols = []
+    pos = 0
+    for seg in list(prefix_segments) + [("image", hp, wp)]:
+        if seg[0] == "text":
+            n = int(seg[1])
+            run = np.arange(pos, pos + n, dtype=np.int64)
+            cols.append(np.stack([run, run, run]))
+            pos += n
+        elif seg[0] == "image":
+            h, w = int(seg[1]), int(seg[2])
+            ii, jj = np.meshgrid(np.arange(h) - (h - h // 2), np.arange(w) - (w - w // 2), indexing="ij")
+            cols.append(np.stack([np.full(h * w, pos, dtype=np.int64), ii.reshape(-1), jj.reshape(-1)]))
+            pos += max(h, w)
+        else:
+            _fail("qwen_rope_positions", f"unknown segment kind {seg[0]!r}")
+    return np.concatenate(cols, axis=1) if cols else np.zeros((3, 0), dtype=np.int64)
+
+
+def rope_tables_from_positions(positions: np.ndarray, head_dim: int, axes_dims_rope: Sequence[int], theta: float = 10000.0):
+    """FP32 (L, head_dim/2) cos / sin from per-axis integer positions (n_axes, L): pair p of axis a turns by
+    position * theta^(-2p / axes[a]); the axes' pairs are concatenated in order. Angles are formed in double."""
+    if head_dim % 2 != 0 or sum(axes_dims_rope) != head_dim or len(axes_dims_rope) != positions.shape[0]:
+        _fail("rope_tables_from_positions", "axes_dims_rope must sum to head_dim, one entry per position axis")
+    blocks = []
+    for a, dim in enumerate(axes_dims_rope):
+        omega = np.power(float(theta), -2.0 * np.arange(dim // 2, dtype=np.float64) / float(dim))
+        blocks.append(positions[a].astype(np.float64)[:, None] * omega[None, :])
+    ang = np.concatenate(blocks, axis=1)
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+def build_qwen_rope_tables(prefix_segments, hp: int, wp: int, head_dim: int, axes_dims_rope: Sequence[int] = (16, 56, 56),
+                           theta: float = 10000.0, device="cuda"):
+    """3-axis RoPE tables of the Qwen-Image joint sequence (QwenImage21Transformer2DModel::build_rope_tables_,
+    src/dit/qwenimage21_forward.cpp:124-200). A cached step slices the rows of its target tokens."""
+    cos, sin = rope_tables_from_positions(qwen_rope_positions(prefix_segments, hp, wp), head_dim, axes_dims_rope, theta)
+    return torch.from_numpy(cos).to(device), torch.from_numpy(sin).to(device)

@@ -146,8 +146,8 @@ typedef struct mi_sdpa_args {
 MI_API int mi_sdpa_forward(const mi_sdpa_args* args);
 /* Tuning / testing knob for the calling thread: 0 = choose the kernel by problem size (default),
  * 1 = always the 4-wavefront kernel (128 query rows per work group), 2 = always the 8-wavefront
- * ping-pong kernel (256 rows; head_dim <= 128), 3 = as 2 but with register-staged tiles where the
- * default would use LDS DMA (head_dim 128). Results agree to rounding; no reference counterpart. */
+ * kernel (256 rows; head_dim <= 128), 3 = as 2 but with register-staged tiles where the default
+ * would move tiles by LDS DMA (head_dim 72 and 128). Results agree to rounding; no reference counterpart. */
 MI_API int mi_sdpa_set_kernel_choice(int32_t choice);
 /* 1 if (dtype, head_dim) has a compiled kernel, else 0. */
 MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);

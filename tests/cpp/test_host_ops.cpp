@@ -17,6 +17,8 @@ void orc_f32_to_bf16_bits(const float* x, size_t n, uint16_t* out);
 void orc_bf16_bits_to_f32(const uint16_t* x, size_t n, float* out);
 int orc_build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const int* axes, int n_axes, float theta,
                                 float* cos_out, float* sin_out);
+int orc_build_qwen_rope_tables(const int* seg_kind, const int* seg_a, const int* seg_b, int n_seg, int hp, int wp, int head_dim,
+                               const int* axes, double theta, float* cos_out, float* sin_out);
 void orc_rope_apply(const float* x, const float* cs, const float* sn, int L, int H, int d, int split_half, int round_mode, float* out);
 void orc_sdpa(const float* q, const float* k, const float* v, int Lq, int Lk, int H, int d, double scale, const float* key_mask,
               const int* row_lo, const int* row_hi, const uint8_t* dense_mask, const float* bias, int bias_q0, int bias_cols,
@@ -87,6 +89,7 @@ static void cpu_checks() {
     CHECK(throws_with([&] { bt::flash_attention_windowed_forward(g, g, g, nullptr, 2, -1, out); }, "window must be >= 0"));
     CHECK(throws_with([&] { dit::build_axial_rope_tables(4, 2, 2, 32, {8, 8, 8}); }, "must sum to head_dim"));
     CHECK(throws_with([&] { dit::build_axial_rope_tables(4, 2, 2, 31, {15, 8, 8}); }, "head_dim must be even"));
+    CHECK(throws_with([&] { dit::build_qwen_rope_tables({}, 2, 2, 32, {8, 8, 8}); }, "summing to head_dim"));
     Tensor Qr, Kr;
     CHECK(throws_with([&] { dit::joint_attention(g, k, g, f, f, 128, 2, out, Qr, Kr); }, "Q/K/V must share shape"));
     CHECK(throws_with([&] { g.row_view(4, 8); }, "rows out of range"));
@@ -127,6 +130,18 @@ static void gpu_checks() {
         bt::rope_apply(K, tabs.cos, tabs.sin, d, H, Krot);
         bt::flash_attention_forward(Qrot, Krot, V, nullptr, H, false, out3);
         CHECK(out.to_host_bytes() == out3.to_host_bytes());
+    }
+    {   // Qwen-Image 3-axis tables: host builder == checker's restatement of build_rope_tables_
+        const std::vector<dit::QwenSegment> pre = {{dit::QwenSegment::Kind::Text, 5, 0, 0}, {dit::QwenSegment::Kind::Image, 0, 3, 4},
+                                                   {dit::QwenSegment::Kind::Text, 2, 0, 0}};
+        dit::RopeTables t = dit::build_qwen_rope_tables(pre, 2, 3, 16, {4, 6, 6});
+        const int kind[3] = {0, 1, 0}, sa[3] = {5, 3, 2}, sb[3] = {0, 4, 0}, ax[3] = {4, 6, 6};
+        const int Lq = orc_build_qwen_rope_tables(kind, sa, sb, 3, 2, 3, 16, ax, 10000.0, nullptr, nullptr);
+        CHECK(Lq == 5 + 12 + 2 + 6 && t.cos.rows == Lq && t.cos.cols == 8);
+        std::vector<float> oc(static_cast<size_t>(Lq) * 8), os(oc.size());
+        orc_build_qwen_rope_tables(kind, sa, sb, 3, 2, 3, 16, ax, 10000.0, oc.data(), os.data());
+        const std::vector<uint8_t> tc = t.cos.to_host_bytes(), ts = t.sin.to_host_bytes();
+        CHECK(std::memcmp(tc.data(), oc.data(), tc.size()) == 0 && std::memcmp(ts.data(), os.data(), ts.size()) == 0);
     }
     {   // windowed causal vs checker
         Tensor Qs = Q.row_view(10, 30), out;

@@ -112,6 +112,29 @@ def test_python_mirror_refuses_cpu_tensors():
     assert abs(cos.numpy() - oc).max() < 1e-7 and abs(sin.numpy() - os_).max() < 1e-7
 
 
+def test_qwen_rope_tables_host_builder():
+    """The host-side 3-axis table builder (src/dit/qwenimage21_forward.cpp:124-200) against the checker's
+    restatement and against positions worked out by hand."""
+    import numpy as np
+    import brodiffusion_amd as bd
+    import oracle
+    segs = [("text", 5), ("image", 3, 4), ("text", 2)]
+    pos = bd.qwen_rope_positions(segs, 2, 3)
+    # text 0..4 at (p,p,p); image 3x4 at frame 5, rows -2..0 (h0 = -(3 - 1)), cols -2..1; position then 5 + max(3,4) = 9;
+    # text at 9, 10; target 2x3 at frame 11, rows -1..0, cols -2..0
+    assert pos.shape == (3, 5 + 12 + 2 + 6)
+    assert pos[:, 4].tolist() == [4, 4, 4] and pos[:, 5].tolist() == [5, -2, -2] and pos[:, 16].tolist() == [5, 0, 1]
+    assert pos[:, 17].tolist() == [9, 9, 9] and pos[:, 19].tolist() == [11, -1, -2] and pos[:, 24].tolist() == [11, 0, 0]
+    cos, sin = bd.build_qwen_rope_tables(segs, 2, 3, 16, (4, 6, 6), device="cpu")
+    oc, os_ = oracle.build_qwen_rope_tables(segs, 2, 3, 16, axes=(4, 6, 6))
+    assert cos.shape == oc.shape and abs(cos.numpy() - oc).max() < 1e-7 and abs(sin.numpy() - os_).max() < 1e-7
+    # pair 1 of the height axis (dim 6) at height position -2: angle -2 * theta^(-2/6)
+    ang = -2.0 * 10000.0 ** (-2.0 / 6.0)
+    assert abs(cos[5, 2 + 1].item() - np.cos(ang)) < 1e-6 and abs(sin[5, 2 + 1].item() - np.sin(ang)) < 1e-6
+    with pytest.raises(RuntimeError, match="axes_dims_rope"):
+        bd.build_qwen_rope_tables(segs, 2, 3, 16, (4, 4, 4), device="cpu")
+
+
 def test_host_cpp_layer_error_paths():
     from brodiffusion_amd import build
     if not os.path.exists(build.HOST_TEST):

@@ -238,6 +238,8 @@ def test_rope_on_fresh_keys_only_with_prefix(oracle):
     dtype, H, d, prefix, hp, wp = "bf16", 2, 128, 50, 8, 8
     img = hp * wp
     cos, sin = oracle.build_qwen_rope_tables([("text", prefix)], hp, wp, d)
+    pcos, psin = bd.build_qwen_rope_tables([("text", prefix)], hp, wp, d)      # the product's host builder
+    assert np.max(np.abs(to_np(pcos) - cos)) < 1e-6 and np.max(np.abs(to_np(psin) - sin)) < 1e-6
     k_all = randn(111, (prefix + img, H * d), dtype); v_all = randn(112, (prefix + img, H * d), dtype)
     q = randn(113, (img, H * d), dtype)
     kr_all = oracle.rope_apply(k_all, cos, sin, H, d, round_to_dtype=dtype)
