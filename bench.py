@@ -85,6 +85,25 @@ def all_configs(torch, bd):
 
     q, k, v = (rnd(2, 4096, 320, dt=torch.float16) for _ in range(3))
     sdpa_entry("cfg1_sd15_selfattn_d40_fp16", 4 * 2 * 8 * 4096 * 4096 * 40, lambda: bd.flash_attention_forward(q, k, v, None, 8, False), "fp16")
+    # the same attention inside the U-Net block: Q/K/V projections (one launch), attention, output projection
+    x, ctx = rnd(2, 4096, 320, dt=torch.float16), rnd(2, 77, 768, dt=torch.float16)
+    wq, wk, wv, wo = (rnd(320, 320, dt=torch.float16) / 320 ** 0.5 for _ in range(4))
+    wk2, wv2 = (rnd(320, 768, dt=torch.float16) / 768 ** 0.5 for _ in range(2))
+    bo = rnd(320, dt=torch.float16)
+    blk_out = torch.empty_like(x)
+    blk_scratch = torch.empty(bd.flash_attention_scratch_bytes(2, 4096, 4096, 320, True), dtype=torch.uint8, device="cuda")
+    sdpa_entry("sd15_unet_block_selfattn_qkvo_c320_fp16", 4 * 2 * 8 * 4096 * 4096 * 40 + 4 * 2 * 8192 * 320 * 320,
+               lambda: bd.flash_attention_qkvo_forward(x, None, wq, None, wk, None, wv, None, wo, bo, None, 8, False, out=blk_out, scratch=blk_scratch), "fp16")
+    kc1, vc1 = bd.flash_attention_project_kv(ctx, wk2, None, wv2, None)
+    sdpa_entry("sd15_unet_block_crossattn_kvcached_c320_fp16", 4 * 2 * 8 * 4096 * 77 * 40 + 2 * 2 * 8192 * 320 * 320,
+               lambda: bd.flash_attention_q_with_kv_cached_forward(x, kc1, vc1, wq, None, wo, bo, None, 8, False, out=blk_out, scratch=blk_scratch), "fp16")
+    x2 = x.view(8192, 320)
+    y2 = torch.empty(8192, 320, dtype=torch.float16, device="cuda")
+    sdpa_entry("linear_8192x320x320_fp16", 2 * 8192 * 320 * 320, lambda: bd.linear_batched(wo, bo, x2, y2), "fp16")
+    xl, wl = rnd(4608, 3072), rnd(3072, 3072) / 3072 ** 0.5
+    yl = torch.empty(4608, 3072, dtype=torch.bfloat16, device="cuda")
+    sdpa_entry("linear_4608x3072x3072_bf16", 2 * 4608 * 3072 * 3072, lambda: bd.linear_batched(wl, None, xl, yl), "bf16")
+    del xl, wl, yl
     q, k, v = (rnd(2, 4096, 1152) for _ in range(3))
     sdpa_entry("cfg2a_pixart_selfattn_d72_bf16", 4 * 2 * 16 * 4096 * 4096 * 72, lambda: bd.flash_attention_forward(q, k, v, None, 16, False), "bf16")
     kc, vc = rnd(2, 300, 1152), rnd(2, 300, 1152)

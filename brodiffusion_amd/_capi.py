@@ -23,6 +23,8 @@ EXPORTS = [
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
     "mi_sdpa_forward", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
+    "mi_linear_forward", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
+    "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv",
 ]
 
 
@@ -81,6 +83,31 @@ class MiLinearAttnArgs(C.Structure):
     ]
 
 
+class MiLinearArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("x", C.c_void_p), ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p),
+        ("rows", C.c_int32), ("in_features", C.c_int32), ("out_features", C.c_int32),
+        ("x_row_stride", C.c_int64), ("w_row_stride", C.c_int64), ("y_row_stride", C.c_int64),
+        ("stream", C.c_void_p),
+    ]
+
+
+class MiAttnBlockArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("x", C.c_void_p), ("ctx", C.c_void_p),
+        ("wq", C.c_void_p), ("bq", C.c_void_p), ("wk", C.c_void_p), ("bk", C.c_void_p),
+        ("wv", C.c_void_p), ("bv", C.c_void_p), ("wo", C.c_void_p), ("bo", C.c_void_p),
+        ("k", C.c_void_p), ("v", C.c_void_p), ("out", C.c_void_p),
+        ("batch", C.c_int32), ("q_len", C.c_int32), ("kv_len", C.c_int32),
+        ("channels", C.c_int32), ("ctx_channels", C.c_int32), ("inner", C.c_int32), ("out_channels", C.c_int32),
+        ("num_heads", C.c_int32), ("causal", C.c_int32),
+        ("key_mask", C.c_void_p), ("key_mask_batch_stride", C.c_int64),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("stream", C.c_void_p),
+    ]
+
+
 _lib = None
 
 
@@ -116,6 +143,11 @@ def lib() -> C.CDLL:
         L.mi_linear_attn_scratch_bytes.restype = C.c_size_t
         L.mi_linear_attn_relu_forward.argtypes = [C.POINTER(MiLinearAttnArgs)]
         L.mi_linear_attn_supported.argtypes = [C.c_int32, C.c_int32]
+        L.mi_linear_forward.argtypes = [C.POINTER(MiLinearArgs)]
+        L.mi_flash_attention_scratch_bytes.argtypes = [C.c_int32] * 5
+        L.mi_flash_attention_scratch_bytes.restype = C.c_size_t
+        for name in ("mi_flash_attention_qkvo_forward", "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv"):
+            getattr(L, name).argtypes = [C.POINTER(MiAttnBlockArgs)]
         _lib = L
     return _lib
 

@@ -204,8 +204,9 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
         p.k = a->rope_k_scratch; p.k_rs = Dkv; p.k_bs = Dkv * a->kv_len;
         p.cos_k = nullptr; p.sin_k = nullptr;
     }
-    const long nb = static_cast<long>(a->batch) * a->num_heads * ((a->q_len + 127) / 128);
-    if (nb > 0x3fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
+    // the grid pads batch*heads to a multiple of 8 for masked calls
+    const long nb = ((static_cast<long>(a->batch) * a->num_heads + 7) & ~7L) * ((a->q_len + 127) / 128);
+    if (nb > 0x7fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
     return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
 }
 

@@ -53,4 +53,15 @@ int sdpa_kernel_choice();
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 bool sdpa_supported(int dtype, int head_dim);
 
+// One Y = X W^T + bias problem: X (M, K), W (N, K), Y (M, N), bias (N) or null; strides in elements.
+struct LinearProblem {
+    const void* x; const void* w; const void* bias; void* y;
+    int M, N, K;
+    long ldx, ldw, ldy;
+};
+constexpr int kMaxLinearProblems = 3;
+struct LinearBatch { LinearProblem p[kMaxLinearProblems]; };
+// Validates and launches up to kMaxLinearProblems problems as one grid.
+int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t stream);
+
 }  // namespace mi

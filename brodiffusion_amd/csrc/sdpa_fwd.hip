@@ -32,6 +32,32 @@ __device__ __forceinline__ int logical_block(int n_blocks) {
     return logical < n_blocks ? logical : -1;
 }
 
+// Work-group id -> (query tile, batch*head). False for the padding groups of the grid.
+// Unmasked calls: every tile costs the same, so the order only serves locality (logical_block).
+// Masked calls (causal, windowed, block-causal): later query tiles see more keys, and work groups start in id
+// order, so ids run over the query tiles from the last to the first with the heads innermost — the longest tiles
+// start first and the short ones fill the gaps at the end (longest-processing-time order). The head count is
+// padded to a multiple of 8 in id space so that id % 8, the XCD, still depends on the head alone and an XCD
+// keeps meeting the same K/V.
+__device__ __forceinline__ bool block_to_tile(const SdpaDev& p, int& qt, int& bh) {
+    if (p.mask_mode == MI_MASK_NONE) {
+        const int logical = logical_block(p.n_blocks);
+        if (logical < 0) return false;
+        qt = logical % p.n_q_tiles;
+        bh = logical / p.n_q_tiles;
+        return true;
+    }
+    const int bh8 = (p.B * p.H + 7) & ~7;
+    qt = p.n_q_tiles - 1 - static_cast<int>(blockIdx.x) / bh8;
+    bh = static_cast<int>(blockIdx.x) % bh8;
+    return qt >= 0 && bh < p.B * p.H;
+}
+// Grid size that block_to_tile expects for n_q_tiles query tiles.
+inline unsigned grid_blocks(const SdpaDev& p) {
+    if (p.mask_mode == MI_MASK_NONE) return static_cast<unsigned>(((p.n_blocks + 7) / 8) * 8);
+    return static_cast<unsigned>(((p.B * p.H + 7) & ~7) * p.n_q_tiles);
+}
+
 // The key axis is cut into 64-row tiles that never straddle the prefix / fresh boundary: prefix
 // tiles start at a multiple of 64 below prefix_len (the last one may be partial), fresh tiles start at
 // prefix_len + a multiple of 64. Rows of a tile at or beyond its segment's limit are zero in LDS and
@@ -201,13 +227,10 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     __shared__ int red[8];
     constexpr int STAGE = G::K_BYTES + G::V_BYTES + kBN * 4;   // K tile, V tile, 64 key-mask floats
 
-    const int logical = logical_block(p.n_blocks);
-    if (logical < 0) return;
-    int qt = logical % p.n_q_tiles;
-    const int bh = logical / p.n_q_tiles;
+    int qt, bh;
+    if (!block_to_tile(p, qt, bh)) return;
     const int h = bh % p.H;
     const int b = bh / p.H;
-    if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;  // longest key ranges first
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
@@ -336,13 +359,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     unsigned char* const Kbuf = smem;                    // 2 x K tile
     unsigned char* const Vbuf = smem + 2 * G::K_BYTES;   // 2 x V tile
 
-    const int logical = logical_block(p.n_blocks);
-    if (logical < 0) return;
-    int qt = logical % p.n_q_tiles;
-    const int bh = logical / p.n_q_tiles;
+    int qt, bh;
+    if (!block_to_tile(p, qt, bh)) return;
     const int h = bh % p.H;
     const int b = bh / p.H;
-    if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;  // longest key ranges first
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
@@ -540,13 +560,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int red[16];
 
-    const int logical = logical_block(p.n_blocks);
-    if (logical < 0) return;
-    int qt = logical % p.n_q_tiles;
-    const int bh = logical / p.n_q_tiles;
+    int qt, bh;
+    if (!block_to_tile(p, qt, bh)) return;
     const int h = bh % p.H;
     const int b = bh / p.H;
-    if (p.mask_mode != MI_MASK_NONE) qt = p.n_q_tiles - 1 - qt;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -814,7 +831,7 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     if (pingpong) {
         p.n_q_tiles = (p.Lq + 255) / 256;
         p.n_blocks = static_cast<int>(tiles256);
-        const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads8);
+        const dim3 grid(grid_blocks(p)), block(kThreads8);
         if constexpr (D <= 128) {
             if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
             else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
@@ -826,7 +843,7 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     } else {
         p.n_q_tiles = (p.Lq + 127) / 128;
         p.n_blocks = p.B * p.H * p.n_q_tiles;
-        const dim3 grid(((p.n_blocks + 7) / 8) * 8), block(kThreads4);
+        const dim3 grid(grid_blocks(p)), block(kThreads4);
         if (rope_k) hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, true>), grid, block, lds_bytes_4<D>(), stream, p);
         else hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false>), grid, block, lds_bytes_4<D>(), stream, p);
     }

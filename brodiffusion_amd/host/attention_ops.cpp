@@ -133,6 +133,117 @@ void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tenso
     check(op, mi_linear_attn_relu_forward(&a));
 }
 
+namespace {
+const void* bias_ptr(const char* op, const Tensor* b, const char* name, Dtype dt, int n) {
+    if (!b) return nullptr;
+    need_gpu(op, *b);
+    if (b->dtype != dt || b->size() != static_cast<std::size_t>(n)) fail(std::string(op) + ": " + name + " must hold " + std::to_string(n) + " values of X's dtype");
+    return b->data;
+}
+void need_weight(const char* op, const Tensor& W, const char* name, Dtype dt, int rows, int cols) {
+    need_gpu(op, W);
+    if (W.dtype != dt) fail(std::string(op) + ": " + name + " must have X's dtype");
+    if ((rows >= 0 && W.rows != rows) || W.cols != cols)
+        fail(std::string(op) + ": " + name + " is (" + std::to_string(W.rows) + ", " + std::to_string(W.cols) + "), expected (" +
+             (rows >= 0 ? std::to_string(rows) : std::string("out")) + ", " + std::to_string(cols) + ")");
+}
+Tensor& thread_scratch() {
+    // never destroyed: a destructor running at thread or process exit could call into a GPU runtime that is already gone
+    static thread_local Tensor* t = new Tensor;
+    return *t;
+}
+void lend_scratch(mi_attn_block_args& a, Tensor* scratch, bool with_kv) {
+    Tensor& s = scratch ? *scratch : thread_scratch();
+    const std::size_t need = mi_flash_attention_scratch_bytes(a.batch, a.q_len, a.kv_len, a.inner, with_kv ? 1 : 0);
+    if (s.data == nullptr || s.bytes() < need) s.resize(1, static_cast<int>((need + 3) / 4), Dtype::FP32, Device::GPU);
+    a.scratch = s.data; a.scratch_bytes = s.bytes();
+}
+void init_block(mi_attn_block_args& a, const char* op, const Tensor& X, const Tensor& Wq, const Tensor* bq, const Tensor& Wo,
+                const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out) {
+    need_gpu(op, X);
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    need_weight(op, Wq, "Wq", X.dtype, -1, X.cols);
+    need_weight(op, Wo, "Wo", X.dtype, -1, Wq.rows);
+    if (out.data == nullptr || out.rows != X.rows || out.cols != Wo.rows || out.dtype != X.dtype) out.resize(X.rows, Wo.rows, X.dtype, X.device);
+    a.x = X.data; a.wq = Wq.data; a.wo = Wo.data; a.out = out.data;
+    a.bq = bias_ptr(op, bq, "bq", X.dtype, Wq.rows);
+    a.bo = bias_ptr(op, bo, "bo", X.dtype, Wo.rows);
+    a.batch = 1; a.q_len = X.rows; a.channels = X.cols; a.inner = Wq.rows; a.out_channels = Wo.rows;
+    a.num_heads = num_heads; a.causal = causal ? 1 : 0;
+    a.key_mask = d_mask;
+}
+}  // namespace
+
+void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor& Y) {
+    const char* op = "linear_batched";
+    need_gpu(op, X);
+    need_weight(op, W, "W", X.dtype, -1, X.cols);
+    if (Y.data == nullptr || Y.rows != X.rows || Y.cols != W.rows || Y.dtype != X.dtype) Y.resize(X.rows, W.rows, X.dtype, X.device);
+    mi_linear_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    a.x = X.data; a.w = W.data; a.y = Y.data;
+    a.bias = bias_ptr(op, bias, "bias", X.dtype, W.rows);
+    a.rows = X.rows; a.in_features = X.cols; a.out_features = W.rows;
+    check(op, mi_linear_forward(&a));
+}
+
+void flash_attention_qkvo_forward(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor* bq, const Tensor& Wk,
+                                  const Tensor* bk, const Tensor& Wv, const Tensor* bv, const Tensor& Wo, const Tensor* bo,
+                                  const float* d_mask, int num_heads, bool causal, Tensor& out, Tensor* scratch) {
+    const char* op = "flash_attention_qkvo_forward";
+    mi_attn_block_args a;
+    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out);
+    const Tensor& S = Ctx ? *Ctx : X;
+    if (Ctx) { need_gpu(op, S); if (S.dtype != X.dtype) fail(std::string(op) + ": Ctx must have X's dtype"); }
+    need_weight(op, Wk, "Wk", X.dtype, Wq.rows, S.cols);
+    need_weight(op, Wv, "Wv", X.dtype, Wq.rows, S.cols);
+    a.ctx = Ctx ? S.data : nullptr;
+    a.wk = Wk.data; a.wv = Wv.data;
+    a.bk = bias_ptr(op, bk, "bk", X.dtype, Wq.rows);
+    a.bv = bias_ptr(op, bv, "bv", X.dtype, Wq.rows);
+    a.kv_len = S.rows; a.ctx_channels = S.cols;
+    lend_scratch(a, scratch, true);
+    check(op, mi_flash_attention_qkvo_forward(&a));
+}
+
+void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq, const Tensor* bq,
+                                              const Tensor& Wo, const Tensor* bo, const float* d_mask, int num_heads, bool causal,
+                                              Tensor& out, Tensor* scratch) {
+    const char* op = "flash_attention_q_with_kv_cached_forward";
+    mi_attn_block_args a;
+    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out);
+    need_gpu(op, K); need_gpu(op, V);
+    if (K.dtype != X.dtype || V.dtype != X.dtype || K.cols != Wq.rows || V.cols != K.cols || V.rows != K.rows)
+        fail(std::string(op) + ": K and V must be (Lk, " + std::to_string(Wq.rows) + ") of X's dtype");
+    a.k = K.data; a.v = V.data; a.kv_len = K.rows;
+    lend_scratch(a, scratch, false);
+    check(op, mi_flash_attention_q_with_kv_cached_forward(&a));
+}
+
+void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
+                                Tensor& K_out, Tensor& V_out) {
+    const char* op = "flash_attention_project_kv";
+    need_gpu(op, ctx);
+    need_weight(op, Wk, "Wk", ctx.dtype, -1, ctx.cols);
+    need_weight(op, Wv, "Wv", ctx.dtype, Wk.rows, ctx.cols);
+    for (Tensor* t : {&K_out, &V_out})
+        if (t->data == nullptr || t->rows != ctx.rows || t->cols != Wk.rows || t->dtype != ctx.dtype) t->resize(ctx.rows, Wk.rows, ctx.dtype, ctx.device);
+    mi_attn_block_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, ctx.dtype);
+    a.ctx = ctx.data; a.wk = Wk.data; a.wv = Wv.data;
+    a.bk = bias_ptr(op, bk, "bk", ctx.dtype, Wk.rows);
+    a.bv = bias_ptr(op, bv, "bv", ctx.dtype, Wk.rows);
+    a.k = K_out.data; a.v = V_out.data;
+    a.batch = 1; a.kv_len = ctx.rows; a.ctx_channels = ctx.cols; a.inner = Wk.rows;
+    check(op, mi_flash_attention_project_kv(&a));
+}
+
 }  // namespace bt
 
 namespace dit {

@@ -7,6 +7,10 @@
 //   dit::joint_attention                   include/brodiffusion/dit/common.h:80-88
 //   dit::gqa_attention_masked              include/brodiffusion/dit/common.h:144-153
 //   dit::build_axial_rope_tables           include/brodiffusion/dit/common.h:70-72
+//   bt::flash_attention_qkvo_forward       src/unet_blocks.cpp:264-272
+//   bt::flash_attention_q_with_kv_cached_forward  src/unet_blocks.cpp:311-317
+//   bt::flash_attention_project_kv         src/unet.cpp:476-480
+//   detail::linear_batched                 include/brodiffusion/detail/compute.h:52-62
 // Precondition failures throw std::runtime_error("<op>: <message>"); a CPU tensor is refused.
 #pragma once
 #include <vector>
@@ -29,6 +33,23 @@ void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, i
 // can spread the tokens of a head over the whole GPU.
 void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
                                    Tensor& state, Tensor& out, bool accumulate_state = false, Tensor* scratch = nullptr);
+
+// Y = X W^T + bias, W (out_features, in_features); bias may be null.
+void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor& Y);
+
+// Attention with its projections (the U-Net spatial transformer's operators). Weights are (out_features, in_features),
+// biases may be null, Ctx == nullptr is self-attention. The projections and the attention output live in a scratch
+// tensor owned by the calling thread, grown on demand and kept (no allocation after warm-up, as the reference's
+// persistent scratch slots, src/unet_blocks.cpp:244-249); pass `scratch` to own it instead.
+void flash_attention_qkvo_forward(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor* bq,
+                                  const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
+                                  const Tensor& Wo, const Tensor* bo, const float* d_mask, int num_heads, bool causal,
+                                  Tensor& out, Tensor* scratch = nullptr);
+void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq,
+                                              const Tensor* bq, const Tensor& Wo, const Tensor* bo, const float* d_mask,
+                                              int num_heads, bool causal, Tensor& out, Tensor* scratch = nullptr);
+void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
+                                Tensor& K_out, Tensor& V_out);
 
 }  // namespace bt
 

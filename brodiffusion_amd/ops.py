@@ -10,6 +10,12 @@ Names, argument order and error behaviour follow the brotensor operators the ref
     joint_attention(Q, K, V, cos, sin, head_dim, num_heads, out, Qr, Kr)     include/brodiffusion/dit/common.h:80-88
     gqa_attention_masked(...)                                                include/brodiffusion/dit/common.h:144-153
     build_axial_rope_tables(txt_len, hp, wp, head_dim, axes, theta)          src/dit/common.cpp:116-184
+    flash_attention_qkvo_forward(X, Ctx, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out)
+                                                                             src/unet_blocks.cpp:264-272
+    flash_attention_q_with_kv_cached_forward(X, K, V, Wq, bq, Wo, bo, d_mask, num_heads, causal, out)
+                                                                             src/unet_blocks.cpp:311-317
+    flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out, V_out)            src/unet.cpp:476-480
+    linear_batched(W, bias, X, Y)                                            include/brodiffusion/detail/compute.h:52
 
 Tensors are torch CUDA tensors (rows = tokens, cols = heads*head_dim), used for device memory
 and the current stream only; every computation is a call through the C ABI. Shape and dtype
@@ -210,6 +216,168 @@ def flash_attention_windowed_forward(Q, K, V, d_mask, num_heads: int, window: in
         _fail(op, "window must be >= 0")
     Lq, Lk = Q.shape[-2], K.shape[-2]
     return sdpa_forward(Q, K, V, num_heads, out=out, key_mask=d_mask, mask=SdpaMask.causal(Lk - Lq, window), op=op)
+
+
+def _mat(op: str, t, name: str, dtype, rows=None, cols=None):
+    """A dense 2-D (or, for activations, 3-D batch-major) operand of the projection ops."""
+    if t is None:
+        return
+    _dev(op, t)
+    if t.dtype != dtype:
+        _fail(op, f"{name} has dtype {t.dtype}, expected {dtype}")
+    if not t.is_contiguous():
+        _fail(op, f"{name} must be contiguous")
+    if rows is not None and t.shape[-2] != rows:
+        _fail(op, f"{name} has {t.shape[-2]} rows, expected {rows}")
+    if cols is not None and t.shape[-1] != cols:
+        _fail(op, f"{name} has {t.shape[-1]} columns, expected {cols}")
+
+
+def _bias(op: str, b, name: str, dtype, n: int):
+    if b is None:
+        return 0
+    _dev(op, b)
+    if b.dtype != dtype or b.numel() != n or not b.is_contiguous():
+        _fail(op, f"{name} must be a contiguous {dtype} vector of {n} values")
+    return b.data_ptr()
+
+
+def linear_batched(W, bias, X, Y: Optional[torch.Tensor] = None):
+    """Y = X W^T + bias; W (out_features, in_features), X (..., in_features)."""
+    op = "linear_batched"
+    _dev(op, W, X)
+    if W.dim() != 2 or X.shape[-1] != W.shape[1]:
+        _fail(op, f"X has {X.shape[-1]} columns, W is {tuple(W.shape)}")
+    _mat(op, W, "W", X.dtype)
+    _mat(op, X, "X", X.dtype)
+    rows = X.numel() // X.shape[-1]
+    if Y is None:
+        Y = torch.empty(*X.shape[:-1], W.shape[0], dtype=X.dtype, device=X.device)
+    _mat(op, Y, "Y", X.dtype, cols=W.shape[0])
+    if Y.numel() != rows * W.shape[0]:
+        _fail(op, "Y has the wrong number of rows")
+    a = capi.MiLinearArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, X)
+    a.x, a.w, a.y = X.data_ptr(), W.data_ptr(), Y.data_ptr()
+    a.bias = _bias(op, bias, "bias", X.dtype, W.shape[0])
+    a.rows, a.in_features, a.out_features = rows, W.shape[1], W.shape[0]
+    a.stream = _stream()
+    capi.check(capi.lib().mi_linear_forward(C.byref(a)), op)
+    return Y
+
+
+def flash_attention_scratch_bytes(batch: int, q_len: int, kv_len: int, inner: int, with_kv: bool) -> int:
+    return int(capi.lib().mi_flash_attention_scratch_bytes(batch, q_len, kv_len, inner, int(with_kv)))
+
+
+def _attn_block(op: str, fn_name: str, X, Ctx, K, V, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch):
+    _dev(op, X, Ctx, K, V, Wq, Wk, Wv, Wo, d_mask, out, scratch)
+    dt = X.dtype
+    B, Lq, Cx, _, _ = _as3(op, X, "X")
+    if not X.is_contiguous():
+        _fail(op, "X must be contiguous")
+    if Wq.dim() != 2 or Wo.dim() != 2:
+        _fail(op, "Wq and Wo must be 2-D (out_features, in_features)")
+    inner, Cout = Wq.shape[0], Wo.shape[0]
+    _mat(op, Wq, "Wq", dt, cols=Cx)
+    _mat(op, Wo, "Wo", dt, cols=inner)
+    a = capi.MiAttnBlockArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, X)
+    a.x, a.wq, a.wo = X.data_ptr(), Wq.data_ptr(), Wo.data_ptr()
+    a.bq, a.bo = _bias(op, bq, "bq", dt, inner), _bias(op, bo, "bo", dt, Cout)
+    Lk = Lq
+    if K is not None:
+        Bk, Lk, Ck, _, _ = _as3(op, K, "K")
+        if Bk != B or Ck != inner or tuple(V.shape) != tuple(K.shape):
+            _fail(op, f"K / V must be ({B} x) (Lk, {inner}) and alike")
+        _mat(op, K, "K", dt)
+        _mat(op, V, "V", dt)
+        a.k, a.v = K.data_ptr(), V.data_ptr()
+    else:
+        Cc = Cx
+        if Ctx is not None:
+            Bc, Lk, Cc, _, _ = _as3(op, Ctx, "Ctx")
+            if Bc != B:
+                _fail(op, f"Ctx has batch {Bc}, X has {B}")
+            _mat(op, Ctx, "Ctx", dt)
+            a.ctx = Ctx.data_ptr()
+        for W, nm in ((Wk, "Wk"), (Wv, "Wv")):
+            _mat(op, W, nm, dt, rows=inner, cols=Cc)
+        a.wk, a.wv = Wk.data_ptr(), Wv.data_ptr()
+        a.bk, a.bv = _bias(op, bk, "bk", dt, inner), _bias(op, bv, "bv", dt, inner)
+        a.ctx_channels = Cc
+    a.batch, a.q_len, a.kv_len = B, Lq, Lk
+    a.channels, a.inner, a.out_channels = Cx, inner, Cout
+    a.num_heads, a.causal = num_heads, int(bool(causal))
+    if d_mask is not None:
+        if d_mask.dtype != torch.float32 or not d_mask.is_contiguous() or d_mask.numel() not in (Lk, B * Lk):
+            _fail(op, "d_mask must be contiguous float32 with Lk (or batch*Lk) values")
+        a.key_mask = d_mask.data_ptr()
+        a.key_mask_batch_stride = Lk if (d_mask.numel() == B * Lk and B > 1) else 0
+    if out is None:
+        out = torch.empty(*X.shape[:-1], Cout, dtype=dt, device=X.device)
+    _mat(op, out, "out", dt, cols=Cout)
+    if out.numel() != B * Lq * Cout:
+        _fail(op, "out has the wrong number of rows")
+    a.out = out.data_ptr()
+    need = flash_attention_scratch_bytes(B, Lq, Lk, inner, K is None)
+    if scratch is None:
+        scratch = torch.empty(need, dtype=torch.uint8, device=X.device)
+    if not scratch.is_contiguous():
+        _fail(op, "scratch must be contiguous")
+    a.scratch, a.scratch_bytes = scratch.data_ptr(), scratch.numel() * scratch.element_size()
+    a.stream = _stream()
+    capi.check(getattr(capi.lib(), fn_name)(C.byref(a)), op)
+    return out
+
+
+def flash_attention_qkvo_forward(X, Ctx, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads: int, causal: bool,
+                                 out: Optional[torch.Tensor] = None, scratch: Optional[torch.Tensor] = None):
+    """out = attention(X Wq^T + bq, S Wk^T + bk, S Wv^T + bv) Wo^T + bo with S = Ctx, or X when Ctx is None.
+    `scratch` (flash_attention_scratch_bytes(..., with_kv=True) bytes) holds the projections; None allocates it."""
+    return _attn_block("flash_attention_qkvo_forward", "mi_flash_attention_qkvo_forward", X, Ctx, None, None,
+                       Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch)
+
+
+def flash_attention_q_with_kv_cached_forward(X, K, V, Wq, bq, Wo, bo, d_mask, num_heads: int, causal: bool,
+                                             out: Optional[torch.Tensor] = None, scratch: Optional[torch.Tensor] = None):
+    """As flash_attention_qkvo_forward with K and V already projected (the cross-attention K/V cache)."""
+    return _attn_block("flash_attention_q_with_kv_cached_forward", "mi_flash_attention_q_with_kv_cached_forward", X, None, K, V,
+                       Wq, bq, None, None, None, None, Wo, bo, d_mask, num_heads, causal, out, scratch)
+
+
+def flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out: Optional[torch.Tensor] = None, V_out: Optional[torch.Tensor] = None):
+    """K_out = ctx Wk^T + bk, V_out = ctx Wv^T + bv in one launch (fills the cross-attention K/V cache)."""
+    op = "flash_attention_project_kv"
+    _dev(op, ctx, Wk, Wv, K_out, V_out)
+    dt = ctx.dtype
+    B, Lk, Cc, _, _ = _as3(op, ctx, "ctx")
+    _mat(op, ctx, "ctx", dt)
+    if Wk.dim() != 2 or tuple(Wv.shape) != tuple(Wk.shape):
+        _fail(op, "Wk and Wv must be 2-D and alike")
+    inner = Wk.shape[0]
+    _mat(op, Wk, "Wk", dt, cols=Cc)
+    _mat(op, Wv, "Wv", dt, cols=Cc)
+    if K_out is None:
+        K_out = torch.empty(*ctx.shape[:-1], inner, dtype=dt, device=ctx.device)
+    if V_out is None:
+        V_out = torch.empty(*ctx.shape[:-1], inner, dtype=dt, device=ctx.device)
+    for t, nm in ((K_out, "K_out"), (V_out, "V_out")):
+        _mat(op, t, nm, dt, cols=inner)
+        if t.numel() != B * Lk * inner:
+            _fail(op, f"{nm} has the wrong number of rows")
+    a = capi.MiAttnBlockArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, ctx)
+    a.ctx, a.wk, a.wv = ctx.data_ptr(), Wk.data_ptr(), Wv.data_ptr()
+    a.bk, a.bv = _bias(op, bk, "bk", dt, inner), _bias(op, bv, "bv", dt, inner)
+    a.k, a.v = K_out.data_ptr(), V_out.data_ptr()
+    a.batch, a.kv_len, a.ctx_channels, a.inner = B, Lk, Cc, inner
+    a.stream = _stream()
+    capi.check(capi.lib().mi_flash_attention_project_kv(C.byref(a)), op)
+    return K_out, V_out
 
 
 def _rope(op: str, X, cos, sin, head_dim, num_heads, out, per_head: bool, split_half: bool):

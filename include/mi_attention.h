@@ -12,6 +12,9 @@
  *                                          src/dit/qwenimage21_forward.cpp:584-585;
  *                                          src/triposplat/flow_model.cpp:374
  *   ReLU linear-attention core             src/dit/sana.cpp:470-586
+ *   bt::flash_attention_qkvo_forward,      src/unet_blocks.cpp:255-327; src/unet.cpp:470-480
+ *   ..._q_with_kv_cached_forward, ..._project_kv
+ *   bt::linear_forward_batched_fp16        include/brodiffusion/detail/compute.h:52-62
  *
  * Conventions (the reference's own C-API conventions, include/brodiffusion/krea2_capi.h:12-18):
  *   - functions return 0 on success, -1 on failure; mi_last_error() holds the message
@@ -210,6 +213,77 @@ MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, i
 MI_API size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API int mi_linear_attn_relu_forward(const mi_linear_attn_args* args);
 MI_API int mi_linear_attn_supported(int32_t dtype, int32_t head_dim);
+
+/* ── linear layer ──────────────────────────────────────────────────────────
+ * Y = X W^T + bias: X (rows, in_features), W (out_features, in_features) — the layout of a
+ * torch / diffusers Linear weight, which is what the reference loads (tests/test_unet.cpp:144-162) —
+ * bias (out_features) of the same dtype or NULL, Y (rows, out_features). FP32 accumulation, bias added
+ * in FP32, one rounding. Replaces brotensor::linear_forward_batched_fp16 as reached through
+ * detail::linear_batched (include/brodiffusion/detail/compute.h:52-62). in_features and out_features
+ * must be multiples of 8; strides in elements (0 = dense), multiples of 8. */
+typedef struct mi_linear_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* x;
+    const void* w;
+    const void* bias;
+    void* y;
+    int32_t rows, in_features, out_features;
+    int64_t x_row_stride, w_row_stride, y_row_stride;
+    void* stream;
+} mi_linear_args;
+MI_API int mi_linear_forward(const mi_linear_args* args);
+
+/* ── attention with its projections ────────────────────────────────────────
+ * The three operators the U-Net spatial transformer calls (src/unet_blocks.cpp:255-327,
+ * src/unet.cpp:470-480; also the VAE mid blocks, src/vae.cpp:268):
+ *
+ *   mi_flash_attention_qkvo_forward               bt::flash_attention_qkvo_forward(X, Ctx*, Wq,bq*, Wk,bk*,
+ *       Q = X Wq^T + bq;  S = ctx ? ctx : X;         Wv,bv*, Wo,bo*, d_mask, num_heads, causal, out)
+ *       K = S Wk^T + bk;  V = S Wv^T + bv;
+ *       out = attention(Q, K, V) Wo^T + bo
+ *   mi_flash_attention_q_with_kv_cached_forward   bt::flash_attention_q_with_kv_cached_forward(X, K, V, Wq,bq*,
+ *       as above with K, V given (k, v)              Wo,bo*, d_mask, num_heads, causal, out)
+ *   mi_flash_attention_project_kv                 bt::flash_attention_project_kv(ctx, Wk,bk*, Wv,bv*, K_out, V_out)
+ *       k = ctx Wk^T + bk;  v = ctx Wv^T + bv
+ *
+ * Weights are (out_features, in_features) row-major, biases may be NULL. Q, K, V and the attention
+ * output are rounded to `dtype` between the stages (they are tensors of that dtype in the reference too) and
+ * live in `scratch`, which the caller lends: mi_flash_attention_scratch_bytes() bytes, 16-byte aligned.
+ * The three projections of the qkvo form run as ONE launch, attention as one, the output projection as
+ * one. Rows are batch-major: item b of x is rows [b*q_len, (b+1)*q_len); with ctx == NULL kv_len is
+ * taken as q_len. head_dim = inner / num_heads must be one mi_sdpa_supported() accepts. */
+typedef struct mi_attn_block_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* x;     /* (batch*q_len, channels) */
+    const void* ctx;   /* (batch*kv_len, ctx_channels) or NULL (self-attention) */
+    const void* wq;    /* (inner, channels) */
+    const void* bq;    /* (inner) or NULL */
+    const void* wk;    /* (inner, ctx_channels) — (inner, channels) when ctx == NULL */
+    const void* bk;
+    const void* wv;
+    const void* bv;
+    const void* wo;    /* (out_channels, inner) */
+    const void* bo;    /* (out_channels) or NULL */
+    void* k;           /* (batch*kv_len, inner): input of the kv_cached form, output of project_kv, unused by qkvo */
+    void* v;
+    void* out;         /* (batch*q_len, out_channels) */
+    int32_t batch, q_len, kv_len;
+    int32_t channels, ctx_channels, inner, out_channels;
+    int32_t num_heads;
+    int32_t causal;    /* != 0: key j visible to query r iff j <= r + (kv_len - q_len) */
+    const float* key_mask;           /* device FP32 [batch or 1][kv_len], 1 valid / 0 not, or NULL */
+    int64_t key_mask_batch_stride;   /* 0 = shared */
+    void* scratch;
+    size_t scratch_bytes;
+    void* stream;
+} mi_attn_block_args;
+/* Scratch bytes of the qkvo form (with_kv != 0) or the kv_cached form (with_kv == 0); project_kv needs none. */
+MI_API size_t mi_flash_attention_scratch_bytes(int32_t batch, int32_t q_len, int32_t kv_len, int32_t inner, int32_t with_kv);
+MI_API int mi_flash_attention_qkvo_forward(const mi_attn_block_args* args);
+MI_API int mi_flash_attention_q_with_kv_cached_forward(const mi_attn_block_args* args);
+MI_API int mi_flash_attention_project_kv(const mi_attn_block_args* args);
 
 #ifdef __cplusplus
 }

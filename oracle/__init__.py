@@ -71,6 +71,8 @@ _lib.orc_dense_block_causal.restype = None
 _lib.orc_linear_attn_relu.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, _f32p,
                                       C.c_void_p, C.c_void_p, C.c_int]
 _lib.orc_linear_attn_relu.restype = None
+_lib.orc_linear.argtypes = [_f32p, _f32p, C.c_void_p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int]
+_lib.orc_linear.restype = None
 _lib.orc_max_threads.restype = C.c_int
 
 
@@ -230,6 +232,36 @@ def linear_attn_relu(q, k, v, num_heads, eps=1e-15, return_state=False, n_thread
     z = np.empty((num_heads, d), dtype=np.float32) if return_state else None
     _lib.orc_linear_attn_relu(q, k, v, N, num_heads, d, eps, out, _ptr(S), _ptr(z), n_threads)
     return (out, S, z) if return_state else out
+
+
+def linear(x, w, bias=None, n_threads=0):
+    """y = x w^T + bias; x (M, K), w (N, K), bias (N) or None."""
+    x, w = _f32(x), _f32(w)
+    M, K = x.shape
+    N = w.shape[0]
+    assert w.shape == (N, K)
+    b = None if bias is None else _f32(bias).reshape(N)
+    y = np.empty((M, N), dtype=np.float32)
+    _lib.orc_linear(x, w, _ptr(b), M, N, K, y, n_threads)
+    return y
+
+
+def attention_qkvo(x, ctx, wq, bq, wk, bk, wv, bv, wo, bo, num_heads, dtype, key_mask=None, causal=False,
+                   k=None, v=None, n_threads=0):
+    """bt::flash_attention_qkvo_forward (src/unet_blocks.cpp:264-272) as linear -> attention -> linear for one
+    batch item; with k / v given, the kv_cached form (src/unet_blocks.cpp:311-317). Q, K, V and the attention
+    output are rounded to `dtype` between the stages ("fp32" keeps them exact)."""
+    q = round_to(linear(x, wq, bq, n_threads), dtype)
+    if k is None:
+        src = x if ctx is None else ctx
+        k = round_to(linear(src, wk, bk, n_threads), dtype)
+        v = round_to(linear(src, wv, bv, n_threads), dtype)
+    Lq, Lk = q.shape[0], k.shape[0]
+    lo = hi = None
+    if causal:
+        lo, hi = rows_causal(Lq, Lk)
+    a = round_to(sdpa(q, k, v, num_heads, key_mask=key_mask, row_lo=lo, row_hi=hi, n_threads=n_threads), dtype)
+    return linear(a, wo, bo, n_threads)
 
 
 def compare(ref: np.ndarray, x: np.ndarray) -> dict:

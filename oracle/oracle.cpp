@@ -22,6 +22,10 @@
 //                              Fully masked row -> zeros follows src/dit/common.cpp:293; what
 //                              brotensor's flash kernel does there is "parity unpinned".
 //   orc_linear_attn_relu       pinned: quadratic-form brute force, (S,z) additivity over token chunks
+//   orc_linear                 pinned: numpy float64 matmul, identity weight, one-hot rows.
+//                              WHERE the fused projection operators round their intermediates
+//                              (Q, K, V, attention output to the tensor dtype) is "parity unpinned":
+//                              brotensor's source is not in the reference tree
 //
 // Build: see oracle/Makefile (g++ -O3 -fopenmp, no dependencies).
 
@@ -474,6 +478,31 @@ ORC_API void orc_linear_attn_relu(const float* q, const float* k, const float* v
                 for (int j = 0; j < d; ++j) num += static_cast<double>(Si[j]) * static_cast<double>(qr[j]);
                 orow[i] = static_cast<float>(num) * recip;
             }
+        }
+    }
+}
+
+// ─── linear layer ───────────────────────────────────────────────────────────
+// Y = X W^T + bias with X (M, K), W (N, K) row-major — the torch Linear weight layout the
+// reference's loaders and tests use (tests/test_unet.cpp:144-162: to_k.weight is {C, ctx_dim})
+// — as computed by brotensor::linear_forward_batched_fp16 behind detail::linear_batched
+// (include/brodiffusion/detail/compute.h:52-62). Sums run in double and are stored as float;
+// bias may be null. The projections around attention (bt::flash_attention_qkvo_forward,
+// src/unet_blocks.cpp:264-272) are this function applied four times.
+ORC_API void orc_linear(const float* x, const float* w, const float* bias, int M, int N, int K, float* y, int n_threads) {
+#ifdef _OPENMP
+    if (n_threads > 0) omp_set_num_threads(n_threads);
+#else
+    (void)n_threads;
+#endif
+#pragma omp parallel for schedule(static)
+    for (int m = 0; m < M; ++m) {
+        const float* xr = x + static_cast<size_t>(m) * K;
+        for (int n = 0; n < N; ++n) {
+            const float* wr = w + static_cast<size_t>(n) * K;
+            double acc = bias ? static_cast<double>(bias[n]) : 0.0;
+            for (int k = 0; k < K; ++k) acc += static_cast<double>(xr[k]) * static_cast<double>(wr[k]);
+            y[static_cast<size_t>(m) * N + n] = static_cast<float>(acc);
         }
     }
 }

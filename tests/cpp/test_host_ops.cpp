@@ -28,6 +28,7 @@ void orc_rows_block_causal(int Lq, int Lk, int q_offset, const int* seg_q_end, c
                            int n_seg, int* row_lo, int* row_hi);
 void orc_linear_attn_relu(const float* q, const float* k, const float* v, int N, int H, int d, float eps, float* out,
                           float* S_out, float* z_out, int n_threads);
+void orc_linear(const float* x, const float* w, const float* bias, int M, int N, int K, float* y, int n_threads);
 }
 
 using namespace bdamd;
@@ -196,6 +197,50 @@ static void gpu_checks() {
         std::printf("linear attention      rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
         CHECK(state.rows == Hl && state.cols == dl * dl + dl);
+    }
+    {   // attention with its projections (SD1.5 level-0 widths: C 320, 8 heads of 40, text context 77 x 768)
+        const int Lx = 100, C = 320, Hh = 8, Lc = 77, Cc = 768;
+        auto scaled = [](std::vector<float> w, int fan_in) {
+            for (float& x : w) x /= std::sqrt(static_cast<float>(fan_in));
+            orc_round_bf16(w.data(), w.size());
+            return w;
+        };
+        const std::vector<float> x = randn_bf16(7101, static_cast<size_t>(Lx) * C), ctx = randn_bf16(7102, static_cast<size_t>(Lc) * Cc);
+        const std::vector<float> wq = scaled(randn_bf16(7103, static_cast<size_t>(C) * C), C), wk = scaled(randn_bf16(7104, static_cast<size_t>(C) * Cc), Cc),
+                                 wv = scaled(randn_bf16(7105, static_cast<size_t>(C) * Cc), Cc), wo = scaled(randn_bf16(7106, static_cast<size_t>(C) * C), C),
+                                 bo = randn_bf16(7107, C);
+        Tensor X = upload_bf16(x, Lx, C), Ctx = upload_bf16(ctx, Lc, Cc), Wq = upload_bf16(wq, C, C), Wk = upload_bf16(wk, C, Cc),
+               Wv = upload_bf16(wv, C, Cc), Wo = upload_bf16(wo, C, C), Bo = upload_bf16(bo, C, 1), out;
+        bt::flash_attention_qkvo_forward(X, &Ctx, Wq, nullptr, Wk, nullptr, Wv, nullptr, Wo, &Bo, nullptr, Hh, false, out);
+        auto lin = [](const std::vector<float>& a, const std::vector<float>& w, const float* b, int M, int N, int K, bool round) {
+            std::vector<float> y(static_cast<size_t>(M) * N);
+            orc_linear(a.data(), w.data(), b, M, N, K, y.data(), 0);
+            if (round) orc_round_bf16(y.data(), y.size());
+            return y;
+        };
+        const std::vector<float> rq = lin(x, wq, nullptr, Lx, C, C, true), rk = lin(ctx, wk, nullptr, Lc, C, Cc, true),
+                                 rv = lin(ctx, wv, nullptr, Lc, C, Cc, true);
+        std::vector<float> ra(rq.size());
+        orc_sdpa(rq.data(), rk.data(), rv.data(), Lx, Lc, Hh, C / Hh, -1.0, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr, 0, ra.data(), nullptr, 0);
+        orc_round_bf16(ra.data(), ra.size());
+        const std::vector<float> ref = lin(ra, wo, bo.data(), Lx, C, C, false);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("qkvo cross attention  rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        // K/V cache filled once, then the cached form: same kernels, same bits
+        Tensor Kc, Vc, out2, own_scratch;
+        bt::flash_attention_project_kv(Ctx, Wk, nullptr, Wv, nullptr, Kc, Vc);
+        CHECK(Kc.rows == Lc && Kc.cols == C);
+        CHECK(within_bf16(compare(rk, download_bf16(Kc))));
+        bt::flash_attention_q_with_kv_cached_forward(X, Kc, Vc, Wq, nullptr, Wo, &Bo, nullptr, Hh, false, out2, &own_scratch);
+        CHECK(out.to_host_bytes() == out2.to_host_bytes());
+        CHECK(own_scratch.bytes() >= mi_flash_attention_scratch_bytes(1, Lx, Lc, C, 0));
+        // the linear layer alone
+        Tensor Y;
+        bt::linear_batched(Wo, &Bo, X, Y);
+        CHECK(within_bf16(compare(lin(x, wo, bo.data(), Lx, C, C, false), download_bf16(Y))));
+        CHECK(throws_with([&] { bt::flash_attention_qkvo_forward(X, &Ctx, Wq, nullptr, Wq, nullptr, Wv, nullptr, Wo, &Bo, nullptr, Hh, false, out); }, "Wk is (320, 320)"));
+        CHECK(throws_with([&] { bt::flash_attention_qkvo_forward(X, nullptr, Wq, nullptr, Wq, nullptr, Wq, nullptr, Wo, &Bo, nullptr, 7, false, out); }, "does not divide"));
     }
     {   // GPU-side error path: unsupported head_dim surfaces the C ABI's message
         Tensor out;

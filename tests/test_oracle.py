@@ -369,3 +369,49 @@ def test_compare_metrics(oracle):
     a = np.array([1.0, 2.0, 2.0]); b = np.array([1.0, 2.0, 2.5])
     m = oracle.compare(a, b)
     assert abs(m["rel_l2"] - 0.5 / 3.0) < 1e-12 and abs(m["max_abs"] - 0.5) < 1e-12
+
+
+# ── linear layer and the projection composition ─────────────────────────────
+@pytest.mark.parametrize("M,N,K", [(7, 5, 3), (33, 320, 768), (1, 8, 1000)])
+def test_linear_vs_numpy_float64(oracle, M, N, K):
+    rng = np.random.default_rng(M * 1000 + N)
+    x = rng.standard_normal((M, K)).astype(np.float32)
+    w = rng.standard_normal((N, K)).astype(np.float32)
+    b = rng.standard_normal(N).astype(np.float32)
+    ref = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.allclose(oracle.linear(x, w), ref, rtol=1e-6, atol=1e-6)
+    assert np.allclose(oracle.linear(x, w, b), ref + b, rtol=1e-6, atol=1e-6)
+
+
+def test_linear_weight_layout_is_out_by_in(oracle):
+    """Row n of W produces output feature n: a one-hot weight row copies one input column, a transposed
+    reading would copy a different one (the matrix is not square and not symmetric)."""
+    M, N, K = 4, 3, 5
+    x = np.arange(M * K, dtype=np.float32).reshape(M, K)
+    w = np.zeros((N, K), np.float32)
+    w[0, 4] = 1; w[1, 0] = 2; w[2, 2] = -1
+    y = oracle.linear(x, w, np.array([10, 20, 30], np.float32))
+    assert np.array_equal(y, np.stack([x[:, 4] + 10, 2 * x[:, 0] + 20, -x[:, 2] + 30], axis=1))
+
+
+def test_attention_qkvo_composition(oracle):
+    """Identity projections reduce the block to plain attention; the kv_cached form with K, V taken from
+    the projections equals the full form; fp32 vs rounded intermediates differ only by rounding."""
+    rng = np.random.default_rng(5)
+    L, Lc, C, H = 19, 7, 16, 2
+    x = rng.standard_normal((L, C)).astype(np.float32)
+    ctx = rng.standard_normal((Lc, 24)).astype(np.float32)
+    eye = np.eye(C, dtype=np.float32)
+    got = oracle.attention_qkvo(x, None, eye, None, eye, None, eye, None, eye, None, H, "fp32")
+    assert np.allclose(got, oracle.sdpa(x, x, x, H), atol=1e-6)
+    wq, wo = (rng.standard_normal((C, C)).astype(np.float32) / 4 for _ in range(2))
+    wk, wv = (rng.standard_normal((C, 24)).astype(np.float32) / 5 for _ in range(2))
+    bq, bk, bv, bo = (rng.standard_normal(C).astype(np.float32) for _ in range(4))
+    full = oracle.attention_qkvo(x, ctx, wq, bq, wk, bk, wv, bv, wo, bo, H, "fp32")
+    k, v = oracle.linear(ctx, wk, bk), oracle.linear(ctx, wv, bv)
+    cached = oracle.attention_qkvo(x, None, wq, bq, None, None, None, None, wo, bo, H, "fp32", k=k, v=v)
+    assert np.array_equal(full, cached)
+    by_hand = oracle.linear(oracle.sdpa(oracle.linear(x, wq, bq), k, v, H), wo, bo)
+    assert np.array_equal(full, by_hand)
+    rounded = oracle.attention_qkvo(x, ctx, wq, bq, wk, bk, wv, bv, wo, bo, H, "bf16")
+    assert 0 < np.abs(rounded - full).max() < 0.05
