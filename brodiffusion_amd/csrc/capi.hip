@@ -106,8 +106,12 @@ int mi_sdpa_set_kernel_choice(int32_t choice) {
 
 int mi_sdpa_supported(int32_t dtype, int32_t head_dim) { return mi::sdpa_supported(dtype, head_dim) ? 1 : 0; }
 
-int mi_sdpa_forward(const mi_sdpa_args* a) {
-    mi::clear_error();
+}  // extern "C"
+
+namespace mi {
+namespace {
+// Validates the arguments and fills the device-side view. Returns 0, -1 (error recorded) or 1 (nothing to do).
+int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
     if (!a) return fail("mi_sdpa_forward: null args");
     if (a->struct_size != sizeof(mi_sdpa_args))
         return fail("mi_sdpa_forward: struct_size %u != %zu (header mismatch)", a->struct_size, sizeof(mi_sdpa_args));
@@ -115,7 +119,7 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
         return fail("mi_sdpa_forward: no kernel for dtype %d head_dim %d", a->dtype, a->head_dim);
     if (a->batch <= 0 || a->num_heads <= 0) return fail("mi_sdpa_forward: batch and num_heads must be positive");
     if (a->q_len < 0 || a->kv_len < 0 || a->prefix_len < 0) return fail("mi_sdpa_forward: negative length");
-    if (a->q_len == 0) return 0;
+    if (a->q_len == 0) return 1;
     if (!a->q || !a->o) return fail("mi_sdpa_forward: q and o must not be null");
     if (a->kv_len > 0 && (!a->k || !a->v)) return fail("mi_sdpa_forward: k and v must not be null");
     if (a->prefix_len > 0 && (!a->k_prefix || !a->v_prefix))
@@ -127,8 +131,8 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
     const long Lk = static_cast<long>(a->prefix_len) + a->kv_len;
     if (Lk > 0x7fffff00L) return fail("mi_sdpa_forward: too many keys");
 
-    mi::SdpaDev p;
     std::memset(&p, 0, sizeof(p));
+    Dkv_out = Dkv;
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
     p.kp = a->prefix_len > 0 ? a->k_prefix : nullptr;
     p.vp = a->prefix_len > 0 ? a->v_prefix : nullptr;
@@ -183,10 +187,42 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
     for (const void* t : tabs)
         if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
     p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
+    if (a->rope_k_scratch && !mi::aligned16(a->rope_k_scratch)) return fail("mi_sdpa_forward: rope_k_scratch must be 16-byte aligned");
+    if (a->split_scratch && !mi::aligned16(a->split_scratch)) return fail("mi_sdpa_forward: split_scratch must be 16-byte aligned");
+    // the grid pads batch*heads to a multiple of 8 for masked calls
+    const long nb = ((static_cast<long>(a->batch) * a->num_heads + 7) & ~7L) * ((a->q_len + 127) / 128);
+    if (nb > 0x7fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
+    return 0;
+}
+// K rotated into the caller's scratch is what the attention kernel reads.
+void use_rotated_k(const mi_sdpa_args* a, SdpaDev& p, long Dkv) {
+    p.k = a->rope_k_scratch; p.k_rs = Dkv; p.k_bs = Dkv * a->kv_len;
+    p.cos_k = nullptr; p.sin_k = nullptr;
+}
+}  // namespace
+}  // namespace mi
+
+extern "C" {
+
+size_t mi_sdpa_split_scratch_bytes(const mi_sdpa_args* a) {
+    mi::clear_error();
+    mi::SdpaDev p;
+    long Dkv = 0;
+    if (mi::prepare_sdpa(a, p, Dkv) != 0) return 0;
+    if (p.cos_k && a->rope_k_scratch && a->kv_len > 0) mi::use_rotated_k(a, p, Dkv);
+    return mi::sdpa_split_scratch_bytes(p, a->dtype, a->head_dim);
+}
+
+int mi_sdpa_forward(const mi_sdpa_args* a) {
+    mi::clear_error();
+    mi::SdpaDev p;
+    long Dkv = 0;
+    const int rc = mi::prepare_sdpa(a, p, Dkv);
+    if (rc != 0) return rc < 0 ? -1 : 0;
+    const int Hkv = a->num_kv_heads > 0 ? a->num_kv_heads : a->num_heads;
     if (p.cos_k && a->rope_k_scratch && a->kv_len > 0) {
         // K is rotated once into the caller's scratch (a pure HBM pass) and the attention kernel reads the
         // rotated copy: the LDS-DMA tile path stays usable and no work group repeats the rotation.
-        if (!mi::aligned16(a->rope_k_scratch)) return fail("mi_sdpa_forward: rope_k_scratch must be 16-byte aligned");
         const size_t esz = 2;
         for (int b = 0; b < a->batch; ++b) {
             mi_rope_args r;
@@ -201,12 +237,10 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
             r.stream = mi::resolve_stream(a->stream);
             if (mi_rope_apply(&r) != 0) return -1;
         }
-        p.k = a->rope_k_scratch; p.k_rs = Dkv; p.k_bs = Dkv * a->kv_len;
-        p.cos_k = nullptr; p.sin_k = nullptr;
+        mi::use_rotated_k(a, p, Dkv);
     }
-    // the grid pads batch*heads to a multiple of 8 for masked calls
-    const long nb = ((static_cast<long>(a->batch) * a->num_heads + 7) & ~7L) * ((a->q_len + 127) / 128);
-    if (nb > 0x7fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
+    p.split_scratch = static_cast<unsigned char*>(a->split_scratch);
+    p.split_scratch_bytes = a->split_scratch ? a->split_scratch_bytes : 0;
     return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
 }
 

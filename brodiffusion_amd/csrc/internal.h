@@ -22,6 +22,39 @@ int device_cu_count();
         if (_e != hipSuccess) return ::mi::fail("%s: %s", #expr, hipGetErrorString(_e)); \
     } while (0)
 
+// Split of the last, partly filled round of an unmasked attention launch.
+//
+// A launch of n_blocks equal query tiles on a GPU that runs n_cu work groups at a time takes ceil(n_blocks / n_cu)
+// rounds even when the last round fills only part of the GPU (432 tiles on 256 compute units: 2 rounds for 1.69
+// rounds of work). With the split, the tiles of the full rounds are processed whole and the tiles of the last round
+// are cut along the KEY axis into as many equal pieces as there are work-group slots; a piece covers the end of one
+// tile and the start of the next, each part leaves a normalised partial output plus its softmax statistics in a
+// scratch slot, and a small second kernel merges the parts of every tile. Everything is done per XCD group (work
+// groups whose id is g mod 8 share an L2): group g owns the logical tiles [g*chunk, (g+1)*chunk) and cu_g work-group
+// slots. All quantities are counted in key tiles of 64 keys ("steps"); T is the number of steps of one query tile.
+struct SplitGeo {
+    int enabled;
+    int T, chunk, n_blocks, cu_g;
+    int max_tail;   // most tail tiles of any group
+    int max_parts;  // partial slots per tail tile
+    static constexpr int kMinPiece = 8;   // shortest piece worth a work group of its own, in steps
+    __host__ __device__ int tiles_of(int g) const { const int n = n_blocks - g * chunk; return n < 0 ? 0 : (n > chunk ? chunk : n); }
+    __host__ __device__ int full_of(int g) const { return tiles_of(g) / cu_g * cu_g; }
+    __host__ __device__ int tail_of(int g) const { return tiles_of(g) - full_of(g); }
+    // pieces the tail steps S of a group are cut into
+    __host__ __device__ int pieces_for(int S) const {
+        if (S <= 0) return 0;
+        const int np = S / kMinPiece;
+        return np < 1 ? 1 : (np > cu_g ? cu_g : np);
+    }
+    // piece c of np covers tail steps [piece_begin(c), piece_begin(c + 1))
+    __host__ __device__ static int piece_begin(int c, int S, int np) { return static_cast<int>(static_cast<long>(c) * S / np); }
+    // the piece that holds tail step x
+    __host__ __device__ static int piece_of(int x, int S, int np) { return static_cast<int>((static_cast<long>(x + 1) * np + S - 1) / S) - 1; }
+    // bytes of one partial slot: 256 rows of head_dim 16-bit values, then 256 references and 256 denominators (FP32)
+    __host__ __device__ static long slot_bytes(int head_dim) { return 256L * head_dim * 2 + 256L * 8; }
+};
+
 // Device-side view of one softmax-attention launch. Strides in elements.
 struct SdpaDev {
     const void* q; const void* k; const void* v; void* o;
@@ -40,6 +73,9 @@ struct SdpaDev {
     const float* cos_q; const float* sin_q;
     const float* cos_k; const float* sin_k;
     int n_q_tiles; int n_blocks;  // logical work items = B*H*n_q_tiles
+    SplitGeo split;               // enabled != 0: split the last round along the key axis
+    unsigned char* split_scratch; // partial slots, [8 groups][max_tail][max_parts] of SplitGeo::slot_bytes
+    size_t split_scratch_bytes;   // what the caller lent
 };
 
 // One rotation, written with explicit fused multiply-adds so that every kernel that rotates
@@ -51,6 +87,8 @@ __device__ __forceinline__ float rope_im(float a, float b, float c, float s) { r
 int sdpa_kernel_choice();
 
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
+// Scratch bytes with which launch_sdpa would split the last round of this launch (0: it would not split).
+size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim);
 bool sdpa_supported(int dtype, int head_dim);
 
 // One Y = X W^T + bias problem: X (M, K), W (N, K), Y (M, N), bias (N) or null; strides in elements.

@@ -551,7 +551,10 @@ struct TileCursor {
     }
 };
 
-template <typename T, int D>
+// SPLIT: the launch follows p.split — a work group either processes one whole query tile or one piece of the last
+// round, i.e. one or more (tile, key range) parts in sequence, each leaving a partial result in its scratch slot
+// (merged by sdpa_combine_kernel). Only for unmasked calls without prefix.
+template <typename T, int D, bool SPLIT>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const SdpaDev p) {
     using G = HeadGeo<D>;
     using DG = DmaGeo<D>;
@@ -560,17 +563,64 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int red[16];
 
+    // ── what this work group does ──
     int qt, bh;
-    if (!block_to_tile(p, qt, bh)) return;
-    const int h = bh % p.H;
-    const int b = bh / p.H;
-
-    const int tid = threadIdx.x;
+    int kv_begin = 0, kv_end = 0x7fffffff;   // key range of the current part
+    unsigned char* part = nullptr;            // scratch slot of the current part; null: the output itself
+    // SPLIT bookkeeping (all wave-uniform): tail steps [seg_s, seg_end) of group xg still to do
+    int xg = 0, n_full = 0, seg_s = 0, seg_end = 0, piece = 0, tail_steps = 0, n_pieces = 0;
+    bool whole = true;
+    if constexpr (!SPLIT) {
+        if (!block_to_tile(p, qt, bh)) return;
+    } else {
+        xg = static_cast<int>(blockIdx.x) & 7;
+        const int i = static_cast<int>(blockIdx.x) >> 3;
+        n_full = p.split.full_of(xg);
+        whole = i < n_full;
+        if (whole) {
+            const int logical = xg * p.split.chunk + i;
+            qt = logical % p.n_q_tiles;
+            bh = logical / p.n_q_tiles;
+        } else {
+            tail_steps = p.split.tail_of(xg) * p.split.T;
+            n_pieces = p.split.pieces_for(tail_steps);
+            piece = i - n_full;
+            if (piece >= n_pieces) return;
+            seg_s = SplitGeo::piece_begin(piece, tail_steps, n_pieces);
+            seg_end = SplitGeo::piece_begin(piece + 1, tail_steps, n_pieces);
+            qt = bh = 0;
+        }
+    }
+  for (;;) {   // one pass per part (a single pass unless SPLIT)
+    // The thread id is made opaque per pass: otherwise every address computation of the prologue and the epilogue,
+    // being the same for all parts, is hoisted out of this loop and stays in registers through the key loop.
+    int tid = threadIdx.x;
+    if constexpr (SPLIT) asm volatile("" : "+v"(tid));
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2;
     const int lane = tid & 63;
     const int lq = lane & 31;
     const int lh = lane >> 5;
+    if constexpr (SPLIT) {
+        if (!whole) {
+            const int tt = seg_s / p.split.T;                  // tail tile of this group
+            const int s0 = seg_s - tt * p.split.T;
+            const int s1 = min(seg_end - tt * p.split.T, p.split.T);
+            const int logical = xg * p.split.chunk + n_full + tt;
+            qt = logical % p.n_q_tiles;
+            bh = logical / p.n_q_tiles;
+            kv_begin = s0 * kBN;
+            kv_end = s1 * kBN;
+            part = nullptr;
+            if (s0 != 0 || s1 != p.split.T) {
+                const int k = piece - SplitGeo::piece_of(tt * p.split.T, tail_steps, n_pieces);
+                part = p.split_scratch + (static_cast<long>(xg * p.split.max_tail + tt) * p.split.max_parts + k) * SplitGeo::slot_bytes(D);
+            }
+            seg_s = tt * p.split.T + s1;
+        }
+    }
+    const int h = bh % p.H;
+    const int b = bh / p.H;
     const int q0 = qt * BM;
     const int qrow = q0 + wave * 32 + lq;
     const bool qvalid = qrow < p.Lq;
@@ -580,6 +630,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
 
     int lo, hi;
     row_interval(p, b, qrow, qvalid, lo, hi);
+    if constexpr (SPLIT) {
+        lo = max(lo, kv_begin);
+        hi = min(hi, kv_end);
+        if (hi <= lo) { lo = 0; hi = 0; }
+    }
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
     V8 qf[G::KC];
@@ -816,12 +871,138 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
     __syncthreads();
-    write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+    if constexpr (!SPLIT) {
+        write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+        break;
+    } else {
+        if (part == nullptr) {
+            write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+        } else {
+            // normalised partial output of the part, then per row the softmax reference (log2 domain) and the
+            // denominator relative to it: the part's weight in the merge is l * 2^ref
+            write_output<T, D, kThreads8>(smem, reinterpret_cast<T*>(part), D, 0, min(BM, p.Lq - q0), BM, tid);
+            if (lh == 0) {
+                float* stat = reinterpret_cast<float*>(part + static_cast<long>(BM) * D * 2);
+                stat[wave * 32 + lq] = -neg_ref[0];
+                stat[BM + wave * 32 + lq] = l_tot;
+            }
+        }
+        if (whole || seg_s >= seg_end) break;
+        __syncthreads();   // the staged output is read by all threads before the next part stages its Q tile
+    }
+  }
+}
+
+// Merge of the parts of one split query tile: out = sum_k w_k O_k / sum_k w_k with w_k = l_k 2^(ref_k - max ref).
+// blockIdx.x = (XCD group, tail tile); tiles that were written whole are skipped.
+template <typename T, int D>
+__global__ void __launch_bounds__(256) sdpa_combine_kernel(const SdpaDev p) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    constexpr int BM = 256, CPR = D / 8;
+    const SplitGeo& sg = p.split;
+    const int xg = static_cast<int>(blockIdx.x) & 7, tt = static_cast<int>(blockIdx.x) >> 3;
+    if (tt >= sg.tail_of(xg)) return;
+    const int S = sg.tail_of(xg) * sg.T, np = sg.pieces_for(S);
+    const int first = SplitGeo::piece_of(tt * sg.T, S, np);
+    const int n_parts = SplitGeo::piece_of((tt + 1) * sg.T - 1, S, np) - first + 1;
+    if (n_parts == 1) return;
+    const int logical = xg * sg.chunk + sg.full_of(xg) + tt;
+    const int qt = logical % p.n_q_tiles, bh = logical / p.n_q_tiles;
+    const int h = bh % p.H, b = bh / p.H;
+    const int q0 = qt * BM;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+    const unsigned char* slots = p.split_scratch + static_cast<long>(xg * sg.max_tail + tt) * sg.max_parts * SplitGeo::slot_bytes(D);
+    // one 16-byte piece of one row per thread; blockIdx.y walks the tile (many short work groups: the merge is a
+    // chain of two dependent loads per part, hidden by occupancy rather than by unrolling)
+    {
+        const int idx = static_cast<int>(blockIdx.y) * 256 + static_cast<int>(threadIdx.x);
+        if (idx >= BM * CPR) return;
+        const int row = idx / CPR, cc = idx - row * CPR;
+        if (q0 + row >= p.Lq) return;
+        float ref = kNegInf;
+        for (int k = 0; k < n_parts; ++k) {
+            const float* stat = reinterpret_cast<const float*>(slots + k * SplitGeo::slot_bytes(D) + static_cast<long>(BM) * D * 2);
+            if (stat[BM + row] > 0.f) ref = fmaxf(ref, stat[row]);
+        }
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        float wsum = 0.f;
+        for (int k = 0; k < n_parts; ++k) {
+            const unsigned char* slot = slots + k * SplitGeo::slot_bytes(D);
+            const float* stat = reinterpret_cast<const float*>(slot + static_cast<long>(BM) * D * 2);
+            const float l = stat[BM + row];
+            if (!(l > 0.f)) continue;
+            const float w = l * __builtin_amdgcn_exp2f(stat[row] - ref);
+            wsum += w;
+            const t8 o = *reinterpret_cast<const t8*>(slot + (static_cast<long>(row) * D + cc * 8) * 2);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, static_cast<float>(o[e]), acc[e]);
+        }
+        const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+        t8 out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = static_cast<T>(acc[e] * inv);
+        *reinterpret_cast<t8*>(o_base + static_cast<long>(q0 + row) * p.o_rs + cc * 8) = out;
+    }
+}
+
+// Decides whether the launch splits its last round (see SplitGeo) and fills p.split. The split costs every tail work
+// group a second prologue and the launch a merge pass (together about ten key steps), so it is taken only when it
+// shortens the last round by more than that — and only when the last round would fill at most half of the GPU:
+// under sustained MFMA load the GPU runs at its power limit, a partly idle last round runs at a higher clock, and
+// measured time follows the total work rather than the number of rounds (432 tiles on 256 compute units take 1.70
+// times one full round, not 2). Measured on head_dim 128, 24 heads: last round 7/32 full: 12 % faster with the
+// split, 10/32: 10 %, 16/32: 6 %, 22/32: 5 % slower.
+template <int D>
+bool plan_split(SdpaDev& p, int n_cu) {
+    p.split = SplitGeo{};
+    if constexpr (!dma_kernel_available<D>()) return false;
+    if (p.mask_mode != MI_MASK_NONE || p.kv_valid_len || p.key_mask || p.Lp > 0 || p.cos_k) return false;
+    if (n_cu < 8 || n_cu % 8 != 0 || sdpa_kernel_choice() == 1 || sdpa_kernel_choice() == 3) return false;
+    const long tiles = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
+    const int T = (p.Lk + kBN - 1) / kBN;
+    if (tiles < n_cu || tiles > (1 << 24) || T < 16 || T > (1 << 20)) return false;
+    SplitGeo g{};
+    g.T = T; g.n_blocks = static_cast<int>(tiles); g.chunk = static_cast<int>((tiles + 7) / 8); g.cu_g = n_cu / 8;
+    const int tail0 = g.tail_of(0);
+    if (tail0 == 0 || 2 * tail0 > g.cu_g) return false;
+    const int np0 = g.pieces_for(tail0 * T);
+    const int piece_len = (tail0 * T + np0 - 1) / np0;
+    if (T - piece_len < 12) return false;
+    for (int xg = 0; xg < 8; ++xg) {
+        const int tail = g.tail_of(xg), S = tail * T, np = g.pieces_for(S);
+        g.max_tail = max(g.max_tail, tail);
+        for (int tt = 0; tt < tail; ++tt)
+            g.max_parts = max(g.max_parts, SplitGeo::piece_of((tt + 1) * T - 1, S, np) - SplitGeo::piece_of(tt * T, S, np) + 1);
+    }
+    g.enabled = 1;
+    p.split = g;
+    return true;
+}
+template <int D>
+size_t split_scratch_bytes_d(SdpaDev p, int n_cu) {
+    if (!plan_split<D>(p, n_cu)) return 0;
+    return static_cast<size_t>(8) * p.split.max_tail * p.split.max_parts * SplitGeo::slot_bytes(D);
 }
 
 template <typename T, int D>
 int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     const bool rope_k = p.cos_k != nullptr;
+    if constexpr (dma_kernel_available<D>()) {
+        if (p.split_scratch != nullptr && plan_split<D>(p, n_cu) &&
+            p.split_scratch_bytes >= static_cast<size_t>(8) * p.split.max_tail * p.split.max_parts * SplitGeo::slot_bytes(D)) {
+            p.n_q_tiles = (p.Lq + 255) / 256;
+            p.n_blocks = p.split.n_blocks;
+            int per_group = 0;
+            for (int xg = 0; xg < 8; ++xg)
+                per_group = max(per_group, p.split.full_of(xg) + p.split.pieces_for(p.split.tail_of(xg) * p.split.T));
+            hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, true>), dim3(8 * per_group), dim3(kThreads8), DmaGeo<D>::lds_bytes(), stream, p);
+            hipLaunchKernelGGL((sdpa_combine_kernel<T, D>), dim3(8 * p.split.max_tail, (256 * (D / 8) + 255) / 256), dim3(256), 0, stream, p);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail("sdpa_fwd launch: %s", hipGetErrorString(e));
+            return 0;
+        }
+        p.split = SplitGeo{};
+    }
     // 256-row tiles when they give every CU at least one work group; head_dim above 128 does not fit
     // two wavefronts per SIMD and stays on the 128-row kernel.
     const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
@@ -836,7 +1017,7 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
             if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
             else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
                 if constexpr (dma_kernel_available<D>())
-                    hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
+                    hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
             }
             else hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false>), grid, block, lds_bytes_8<D>(), stream, p);
         }
@@ -875,6 +1056,14 @@ bool sdpa_supported(int dtype, int head_dim) {
         case 40: case 64: case 72: case 80: case 96: case 112: case 128: case 160: return true;
         default: return false;
     }
+}
+
+size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim) {
+    if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_F16) return 0;
+    const int n_cu = device_cu_count();
+    if (head_dim == 72) return split_scratch_bytes_d<72>(p, n_cu);
+    if (head_dim == 128) return split_scratch_bytes_d<128>(p, n_cu);
+    return 0;
 }
 
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream) {

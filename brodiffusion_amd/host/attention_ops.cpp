@@ -37,6 +37,18 @@ void init_args(mi_sdpa_args& a, const char* op, const Tensor& Q, const Tensor& K
     a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.num_kv_heads = num_kv_heads;
     a.q_len = Q.rows; a.kv_len = K.rows;
 }
+// Launch with this thread's split scratch lent when the call can use one (grown on demand, then kept: no allocation
+// after warm-up; never destroyed, see thread_scratch below for why).
+void run_sdpa(const char* op, mi_sdpa_args& a) {
+    static thread_local Tensor* scratch = new Tensor;
+    const std::size_t need = mi_sdpa_split_scratch_bytes(&a);
+    if (need > 0) {
+        if (scratch->data == nullptr || scratch->bytes() < need) scratch->resize(1, static_cast<int>((need + 3) / 4), Dtype::FP32, Device::GPU);
+        a.split_scratch = scratch->data;
+        a.split_scratch_bytes = scratch->bytes();
+    }
+    check(op, mi_sdpa_forward(&a));
+}
 void set_rope(mi_sdpa_args& a, const char* op, const Tensor* cos, const Tensor* sin, int rows, bool for_q) {
     if (!cos && !sin) return;
     if (!cos || !sin) fail(std::string(op) + ": cos and sin must be given together");
@@ -59,7 +71,7 @@ void flash_attention_forward(const Tensor& Q, const Tensor& K, const Tensor& V, 
     init_args(a, op, Q, K, V, num_heads, num_heads, out);
     a.key_mask = d_mask;
     if (causal) { a.mask_mode = MI_MASK_CAUSAL; a.q_offset = K.rows - Q.rows; }
-    check(op, mi_sdpa_forward(&a));
+    run_sdpa(op, a);
 }
 
 void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask,
@@ -70,7 +82,7 @@ void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Te
     init_args(a, op, Q, K, V, num_heads, num_heads, out);
     a.key_mask = d_mask;
     a.mask_mode = MI_MASK_CAUSAL; a.q_offset = K.rows - Q.rows; a.window = window;
-    check(op, mi_sdpa_forward(&a));
+    run_sdpa(op, a);
 }
 
 static void rope_impl(const char* op, const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads,
@@ -337,7 +349,7 @@ void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Te
     set_rope(a, op, &cos, &sin, K.rows, false);
     Kr.resize(K.rows, K.cols, K.dtype, K.device);  // receives RoPE(K), as in the reference
     a.rope_k_scratch = Kr.data;
-    check(op, mi_sdpa_forward(&a));
+    run_sdpa(op, a);
 }
 
 void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin, int head_dim,
@@ -356,7 +368,7 @@ void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, con
         Kr.resize(K.rows, K.cols, K.dtype, K.device);
         a.rope_k_scratch = Kr.data;
     }
-    check(op, mi_sdpa_forward(&a));
+    run_sdpa(op, a);
 }
 
 void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix, const Tensor* v_prefix,
@@ -390,7 +402,7 @@ void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, c
     set_rope(a, op, cos_q, sin_q, Q.rows, true);
     if (cos_q && K.rows == Q.rows) set_rope(a, op, cos_q, sin_q, K.rows, false);
     else if (cos_q) fail(std::string(op) + ": fused RoPE needs K and Q to cover the same positions");
-    check(op, mi_sdpa_forward(&a));
+    run_sdpa(op, a);
 }
 
 }  // namespace dit

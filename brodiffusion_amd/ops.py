@@ -108,8 +108,11 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
                  kv_valid_len: Optional[torch.Tensor] = None, key_mask: Optional[torch.Tensor] = None,
                  rope_q: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                 rope_k_scratch: Optional[torch.Tensor] = None, op: str = "sdpa_forward") -> torch.Tensor:
-    """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None)."""
+                 rope_k_scratch: Optional[torch.Tensor] = None, split_scratch=None,
+                 op: str = "sdpa_forward") -> torch.Tensor:
+    """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None).
+    split_scratch: None = lend the module's own scratch (grown on demand, one per device, shared by all calls of the
+    process: use one stream at a time) when the launch can use one, False = never split, a uint8 tensor = lend that."""
     _dev(op, q, k, v, out, k_prefix, v_prefix, kv_valid_len, key_mask, rope_k_scratch)
     dt = _dtype_code(op, q)
     if k.dtype != q.dtype or v.dtype != q.dtype:
@@ -195,8 +198,29 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
             _fail(op, "rope_k_scratch must be contiguous, of Q's dtype and at least as large as K")
         a.rope_k_scratch = rope_k_scratch.data_ptr()
     a.stream = _stream()
+    if split_scratch is not False:
+        need = int(capi.lib().mi_sdpa_split_scratch_bytes(C.byref(a)))
+        if need > 0:
+            if split_scratch is None:
+                split_scratch = _own_split_scratch(q.device, need)
+            _dev(op, split_scratch)
+            if not split_scratch.is_contiguous():
+                _fail(op, "split_scratch must be contiguous")
+            a.split_scratch = split_scratch.data_ptr()
+            a.split_scratch_bytes = split_scratch.numel() * split_scratch.element_size()
     capi.check(capi.lib().mi_sdpa_forward(C.byref(a)), op)
     return out
+
+
+_split_scratch_cache = {}
+
+
+def _own_split_scratch(device, nbytes: int) -> torch.Tensor:
+    t = _split_scratch_cache.get(device)
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _split_scratch_cache[device] = t
+    return t
 
 
 def flash_attention_forward(Q, K, V, d_mask, num_heads: int, causal: bool, out: Optional[torch.Tensor] = None):

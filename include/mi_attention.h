@@ -143,10 +143,20 @@ typedef struct mi_sdpa_args {
                                     K is rotated into it by one bandwidth-bound pass and attention reads the rotated copy
                                     (fastest form); afterwards it holds RoPE(K) like the Kr scratch of dit::joint_attention
                                     (src/dit/common.cpp:193). NULL: K is rotated tile by tile as it is loaded */
+    void* split_scratch;         /* device, 16-byte aligned, or NULL: lets a launch whose last round of work groups would fill
+                                    only part of the GPU cut the query tiles of that round along the key axis into equal
+                                    pieces for all compute units (partial results in the scratch, merged by a second small
+                                    kernel). Used when at least mi_sdpa_split_scratch_bytes(args) bytes are lent and that
+                                    value is not 0; results agree with the unsplit launch to rounding */
+    size_t split_scratch_bytes;
     void* stream;                /* hipStream_t; NULL = library current stream */
 } mi_sdpa_args;
 
 MI_API int mi_sdpa_forward(const mi_sdpa_args* args);
+/* Bytes of split_scratch with which this call (same args, split_scratch fields ignored) would split its last round;
+ * 0 when it would not (masked calls, short key sequences, a last round that is nearly full, kernels without the
+ * split). No reference counterpart. */
+MI_API size_t mi_sdpa_split_scratch_bytes(const mi_sdpa_args* args);
 /* Tuning / testing knob for the calling thread: 0 = choose the kernel by problem size (default),
  * 1 = always the 4-wavefront kernel (128 query rows per work group), 2 = always the 8-wavefront
  * kernel (256 rows; head_dim <= 128), 3 = as 2 but with register-staged tiles where the default
