@@ -126,6 +126,13 @@ def all_configs(torch, bd):
     sdpa_entry("cfg4_qwen_blockcausal_prefixkv_d128_bf16", 4 * 24 * sum(1024 * e for e in sk) * 128,
                lambda: bd.sdpa_forward(qb, kb, vb, 24, k_prefix=kp, v_prefix=vp, mask=mask), "bf16")
     out["cfg4_qwen_blockcausal_prefixkv_d128_bf16"]["dense_equivalent_gflop"] = round(4 * 24 * 4096 * 4608 * 128 / 1e9, 2)
+    xh, gh = rnd(4608, 3072), rnd(128)
+    oh = torch.empty_like(xh)
+    mn, av = event_ms(torch, lambda: bd.headnorm_rope(xh, gh, 1e-6, cos, sin, 128, 24, out=oh), 20)
+    nbytes = 2 * xh.numel() * 2
+    out["headnorm_rope_4608x24x128_bf16"] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
+                                             "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16",
+                                             "mbytes": round(nbytes / 1e6, 2)}
     for name, n in (("cfg5a_sana_linear_n1024_d112_bf16", 1024), ("cfg5b_sana_linear_n4096_d112_bf16", 4096)):
         ql, kl, vl_ = (rnd(2, n, 2240) for _ in range(3))
         ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")

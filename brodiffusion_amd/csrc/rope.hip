@@ -61,6 +61,81 @@ __global__ void __launch_bounds__(256) rope_split_kernel(const T* __restrict__ x
     }
 }
 
+// Per-head RMS normalisation fused with the rotation (adjacent pairs) and an optional second destination for the
+// leading rows: y = RoPE(x * rsqrt(mean_d(x^2) + eps) * gain), one read of x, one rounding. One thread per 16-byte
+// chunk; the CPR = d/8 threads of a head row are neighbouring lanes of one wavefront (CPR is a power of two <= 16),
+// so the sum of squares is CPR-lane butterfly. Everything is FP32 between the load and the single rounding.
+template <typename T, int CPR>
+__global__ void __launch_bounds__(256) headnorm_rope_kernel(const T* x, T* out, T* out2,
+                                                            const T* __restrict__ gain, const float* __restrict__ cs,
+                                                            const float* __restrict__ sn, int rows, int H, float eps,
+                                                            long x_rs, long o_rs, long o2_rs, int out2_rows) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    constexpr int d = CPR * 8;
+    const int cpr = H * CPR;
+    const long total = static_cast<long>(rows) * cpr;
+    for (long idx = blockIdx.x * 256L + threadIdx.x; idx < total; idx += gridDim.x * 256L) {
+        const int r = static_cast<int>(idx / cpr);
+        const int c = static_cast<int>(idx - static_cast<long>(r) * cpr);
+        const int col = c * 8;
+        const int dc = (c % CPR) * 8;
+        const t8 v = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(x + r * x_rs + col));
+        const t8 g = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(gain + dc));
+        float f[8];
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { f[e] = static_cast<float>(v[e]); ss = __builtin_fmaf(f[e], f[e], ss); }
+#pragma unroll
+        for (int off = 1; off < CPR; off <<= 1) ss += __shfl_xor(ss, off);
+        const float inv = __builtin_amdgcn_rsqf(ss * (1.0f / d) + eps);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) f[e] = f[e] * inv * static_cast<float>(g[e]);
+        t8 o;
+        if (cs != nullptr) {
+            const f32x4 cv = *reinterpret_cast<const f32x4*>(cs + static_cast<long>(r) * (d / 2) + dc / 2);
+            const f32x4 sv = *reinterpret_cast<const f32x4*>(sn + static_cast<long>(r) * (d / 2) + dc / 2);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                o[2 * p] = static_cast<T>(rope_re(f[2 * p], f[2 * p + 1], cv[p], sv[p]));
+                o[2 * p + 1] = static_cast<T>(rope_im(f[2 * p], f[2 * p + 1], cv[p], sv[p]));
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(f[e]);
+        }
+        const u32x4 bits = __builtin_bit_cast(u32x4, o);
+        *reinterpret_cast<u32x4*>(out + r * o_rs + col) = bits;
+        if (r < out2_rows) *reinterpret_cast<u32x4*>(out2 + r * o2_rs + col) = bits;
+    }
+}
+
+template <typename T>
+int launch_headnorm(const mi_headnorm_rope_args* a, long x_rs, long o_rs, long o2_rs, hipStream_t st) {
+    const long work = static_cast<long>(a->rows) * a->num_heads * a->head_dim / 8;
+    long blocks = (work + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    const T* x = static_cast<const T*>(a->x);
+    T* o = static_cast<T*>(a->out);
+    T* o2 = static_cast<T*>(a->out2);
+    const T* g = static_cast<const T*>(a->gain);
+    const int r2 = a->out2 ? a->out2_rows : 0;
+#define MI_HEADNORM_CASE(CPR)                                                                                          \
+    case CPR * 8:                                                                                                      \
+        hipLaunchKernelGGL((headnorm_rope_kernel<T, CPR>), dim3(blocks), dim3(256), 0, st, x, o, o2, g, a->cos, a->sin, \
+                           a->rows, a->num_heads, a->eps, x_rs, o_rs, o2_rs, r2);                                      \
+        break;
+    switch (a->head_dim) {
+        MI_HEADNORM_CASE(4)
+        MI_HEADNORM_CASE(8)
+        MI_HEADNORM_CASE(16)
+        default: return fail("mi_headnorm_rope: head_dim %d not supported (32, 64, 128)", a->head_dim);
+    }
+#undef MI_HEADNORM_CASE
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("mi_headnorm_rope launch: %s", hipGetErrorString(e));
+    return 0;
+}
+
 template <typename T>
 int launch(const mi_rope_args* a, long x_rs, long o_rs, hipStream_t st) {
     const long work = a->split_half ? static_cast<long>(a->rows) * a->num_heads * (a->head_dim / 2)
@@ -109,4 +184,32 @@ extern "C" int mi_rope_apply(const mi_rope_args* a) {
     if (a->dtype == MI_DTYPE_BF16) return mi::launch<__bf16>(a, x_rs, o_rs, st);
     if (a->dtype == MI_DTYPE_F16) return mi::launch<_Float16>(a, x_rs, o_rs, st);
     return fail("mi_rope_apply: dtype %d not supported", a->dtype);
+}
+
+extern "C" int mi_headnorm_rope(const mi_headnorm_rope_args* a) {
+    using mi::fail;
+    mi::clear_error();
+    if (!a) return fail("mi_headnorm_rope: null args");
+    if (a->struct_size != sizeof(mi_headnorm_rope_args)) return fail("mi_headnorm_rope: struct_size mismatch");
+    if (a->rows < 0 || a->num_heads <= 0) return fail("mi_headnorm_rope: bad shape");
+    if (a->head_dim != 32 && a->head_dim != 64 && a->head_dim != 128)
+        return fail("mi_headnorm_rope: head_dim %d not supported (32, 64, 128)", a->head_dim);
+    if (a->rows == 0) return 0;
+    if (!a->x || !a->out || !a->gain) return fail("mi_headnorm_rope: x, out and gain must not be null");
+    if ((a->cos == nullptr) != (a->sin == nullptr)) return fail("mi_headnorm_rope: cos and sin must be given together");
+    if (!(a->eps >= 0.f)) return fail("mi_headnorm_rope: eps must be >= 0");
+    if (a->out2_rows < 0 || a->out2_rows > a->rows) return fail("mi_headnorm_rope: out2_rows %d outside 0..rows", a->out2_rows);
+    const long D = static_cast<long>(a->num_heads) * a->head_dim;
+    const long x_rs = a->x_row_stride ? a->x_row_stride : D;
+    const long o_rs = a->out_row_stride ? a->out_row_stride : D;
+    const long o2_rs = a->out2_row_stride ? a->out2_row_stride : D;
+    if (x_rs < D || o_rs < D || o2_rs < D) return fail("mi_headnorm_rope: row stride smaller than heads*head_dim");
+    if (x_rs % 8 != 0 || o_rs % 8 != 0 || o2_rs % 8 != 0) return fail("mi_headnorm_rope: row strides must be multiples of 8 elements");
+    const uintptr_t al = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->out) | reinterpret_cast<uintptr_t>(a->out2) |
+                         reinterpret_cast<uintptr_t>(a->gain) | reinterpret_cast<uintptr_t>(a->cos) | reinterpret_cast<uintptr_t>(a->sin);
+    if (al & 15u) return fail("mi_headnorm_rope: pointers must be 16-byte aligned");
+    hipStream_t st = mi::resolve_stream(a->stream);
+    if (a->dtype == MI_DTYPE_BF16) return mi::launch_headnorm<__bf16>(a, x_rs, o_rs, o2_rs, st);
+    if (a->dtype == MI_DTYPE_F16) return mi::launch_headnorm<_Float16>(a, x_rs, o_rs, o2_rs, st);
+    return fail("mi_headnorm_rope: dtype %d not supported", a->dtype);
 }

@@ -338,6 +338,38 @@ RopeTables build_qwen_rope_tables(const std::vector<QwenSegment>& prefix, int hp
     return t;
 }
 
+void headnorm_rope(const Tensor& X, const Tensor& gain, float eps, const Tensor* cos, const Tensor* sin, int head_dim,
+                   int num_heads, Tensor& out, Tensor* cache_out, int cache_rows) {
+    const char* op = "headnorm_rope";
+    need_gpu(op, X); need_gpu(op, gain);
+    if (head_dim <= 0 || num_heads <= 0 || X.cols != head_dim * num_heads) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if (gain.dtype != X.dtype || gain.size() != static_cast<std::size_t>(head_dim)) fail(std::string(op) + ": gain must hold head_dim values of X's dtype");
+    if ((cos == nullptr) != (sin == nullptr)) fail(std::string(op) + ": cos and sin must be given together");
+    if (cos) {
+        need_gpu(op, *cos); need_gpu(op, *sin);
+        if (cos->dtype != Dtype::FP32 || sin->dtype != Dtype::FP32 || cos->rows != X.rows || sin->rows != X.rows ||
+            cos->cols != head_dim / 2 || sin->cols != head_dim / 2)
+            fail(std::string(op) + ": cos/sin must be FP32 (L, head_dim/2)");
+    }
+    if (cache_out && (cache_rows < 0 || cache_rows > X.rows)) fail(std::string(op) + ": cache_rows outside 0..L");
+    if (out.data == nullptr || out.rows != X.rows || out.cols != X.cols || out.dtype != X.dtype) out.resize(X.rows, X.cols, X.dtype, X.device);
+    mi_headnorm_rope_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    a.x = X.data; a.out = out.data; a.gain = gain.data;
+    a.cos = cos ? static_cast<const float*>(cos->data) : nullptr;
+    a.sin = sin ? static_cast<const float*>(sin->data) : nullptr;
+    a.eps = eps;
+    a.rows = X.rows; a.num_heads = num_heads; a.head_dim = head_dim;
+    if (cache_out && cache_rows > 0) {
+        if (cache_out->data == nullptr || cache_out->rows != cache_rows || cache_out->cols != X.cols || cache_out->dtype != X.dtype)
+            cache_out->resize(cache_rows, X.cols, X.dtype, X.device);
+        a.out2 = cache_out->data; a.out2_rows = cache_rows;
+    }
+    check(op, mi_headnorm_rope(&a));
+}
+
 void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin, int head_dim,
                      int num_heads, Tensor& out, Tensor& /*Qr*/, Tensor& Kr) {
     const char* op = "joint_attention";

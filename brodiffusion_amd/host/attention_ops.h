@@ -11,6 +11,7 @@
 //   bt::flash_attention_q_with_kv_cached_forward  src/unet_blocks.cpp:311-317
 //   bt::flash_attention_project_kv         src/unet.cpp:476-480
 //   detail::linear_batched                 include/brodiffusion/detail/compute.h:52-62
+//   headnorm + bt::rope_apply              src/dit/qwenimage21_forward.cpp:53-63, :582-585
 // Precondition failures throw std::runtime_error("<op>: <message>"); a CPU tensor is refused.
 #pragma once
 #include <vector>
@@ -75,6 +76,13 @@ struct QwenSegment {
 // of its target tokens (row_view).
 RopeTables build_qwen_rope_tables(const std::vector<QwenSegment>& prefix, int hp, int wp, int head_dim,
                                   const std::vector<int>& axes_dims_rope, float theta = 10000.0f);
+
+// headnorm + rope_apply of the DiT blocks in one pass (src/dit/qwenimage21_forward.cpp:53-63, :582-585;
+// src/dit/flux.cpp:462-469): per (row, head) RMS normalisation with `gain` (1 x head_dim or head_dim x 1), then the
+// rotation (cos == sin == nullptr: normalisation only). cache_out, if given, is resized to (cache_rows, D) and receives
+// the first cache_rows rows as well: the prefix rows of K on their way into the prefix cache (:587-597).
+void headnorm_rope(const Tensor& X, const Tensor& gain, float eps, const Tensor* cos, const Tensor* sin, int head_dim,
+                   int num_heads, Tensor& out, Tensor* cache_out = nullptr, int cache_rows = 0);
 
 // RoPE on Q and K, then full-bidirectional attention. Q is rotated while it is loaded; K is rotated
 // into Kr (resized to K's shape, holds RoPE(K) afterwards as in the reference) and read from there.

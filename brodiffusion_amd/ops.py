@@ -441,6 +441,46 @@ def rope_apply_perhead(X, cos, sin, head_dim: int, num_heads: int, out: Optional
     return _rope("rope_apply_perhead", X, cos, sin, head_dim, num_heads, out, True, split_half)
 
 
+def headnorm_rope(X, gain, eps: float, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
+                  cache_out: Optional[torch.Tensor] = None):
+    """headnorm + rope_apply of the DiT blocks (src/dit/qwenimage21_forward.cpp:582-585, src/dit/flux.cpp:462-469) in
+    one pass: per (row, head) RMS normalisation with `gain` (head_dim), then the rotation (cos = sin = None: the
+    normalisation alone). cache_out (rows <= X's rows): its rows also receive the result — the prefix rows of K going
+    into the prefix cache (qwenimage21_forward.cpp:587-597)."""
+    op = "headnorm_rope"
+    _dev(op, X, gain, cos, sin, out, cache_out)
+    if X.dim() != 2 or X.stride(1) != 1 or X.shape[1] != head_dim * num_heads:
+        _fail(op, "X must be (L, head_dim * num_heads), contiguous along columns")
+    if gain.dtype != X.dtype or gain.numel() != head_dim or not gain.is_contiguous():
+        _fail(op, "gain must hold head_dim values of X's dtype")
+    if out is None:
+        out = torch.empty_like(X)
+    if out.shape != X.shape or out.dtype != X.dtype or out.stride(1) != 1:
+        _fail(op, "out must have X's shape and dtype")
+    a = capi.MiHeadnormRopeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, X)
+    a.x, a.out, a.gain = X.data_ptr(), out.data_ptr(), gain.data_ptr()
+    if (cos is None) != (sin is None):
+        _fail(op, "cos and sin must be given together")
+    if cos is not None:
+        for t in (cos, sin):
+            if t.dtype != torch.float32 or tuple(t.shape) != (X.shape[0], head_dim // 2) or not t.is_contiguous():
+                _fail(op, "cos/sin must be contiguous float32 (L, head_dim/2)")
+        a.cos, a.sin = cos.data_ptr(), sin.data_ptr()
+    a.eps = eps
+    a.rows, a.num_heads, a.head_dim = X.shape[0], num_heads, head_dim
+    a.x_row_stride, a.out_row_stride = X.stride(0), out.stride(0)
+    if cache_out is not None:
+        if cache_out.dim() != 2 or cache_out.dtype != X.dtype or cache_out.shape[1] != X.shape[1] or cache_out.stride(1) != 1 \
+                or cache_out.shape[0] > X.shape[0]:
+            _fail(op, "cache_out must be (rows <= L, head_dim * num_heads) of X's dtype")
+        a.out2, a.out2_rows, a.out2_row_stride = cache_out.data_ptr(), cache_out.shape[0], cache_out.stride(0)
+    a.stream = _stream()
+    capi.check(capi.lib().mi_headnorm_rope(C.byref(a)), op)
+    return out
+
+
 def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
                     Qr: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
     """Full-bidirectional joint attention with RoPE on Q and K (include/brodiffusion/dit/common.h:74-88).

@@ -186,6 +186,32 @@ typedef struct mi_rope_args {
 } mi_rope_args;
 MI_API int mi_rope_apply(const mi_rope_args* args);
 
+/* ── per-head RMSNorm + RoPE in one pass ───────────────────────────────────
+ * out = RoPE(x * rsqrt(mean over head_dim of x^2 + eps) * gain) per (row, head): what the DiT blocks do between the
+ * Q/K projections and attention as two passes, bt::rms_norm_forward on the (L*heads, head_dim) view followed by
+ * bt::rope_apply (headnorm, src/dit/qwenimage21_forward.cpp:53-63 and :582-585; src/dit/flux.cpp:462-469). One read
+ * of x, FP32 in between, a single rounding. gain: (head_dim) of `dtype`. cos / sin: FP32 (rows, head_dim/2), adjacent
+ * pairs, or both NULL for the normalisation alone. out2 (optional): rows [0, out2_rows) are written there as well —
+ * the prefix rows of K going into the prefix cache while the full K goes to attention
+ * (qwenimage21_forward.cpp:587-597). In-place (out == x) is allowed. head_dim 32, 64 or 128. */
+typedef struct mi_headnorm_rope_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* x;
+    void* out;
+    const void* gain;
+    const float* cos;
+    const float* sin;
+    float eps;
+    int32_t rows, num_heads, head_dim;
+    int64_t x_row_stride, out_row_stride;
+    void* out2;
+    int32_t out2_rows;
+    int64_t out2_row_stride;
+    void* stream;
+} mi_headnorm_rope_args;
+MI_API int mi_headnorm_rope(const mi_headnorm_rope_args* args);
+
 /* ── ReLU linear attention ─────────────────────────────────────────────────
  * Per (batch, head): Kr = relu(K), Qr = relu(Q); S = V^T Kr (d x d), z = sum_n Kr (d);
  * O[n] = (S Qr[n]) / (z . Qr[n] + eps). Replaces the core of

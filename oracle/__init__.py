@@ -71,6 +71,8 @@ _lib.orc_dense_block_causal.restype = None
 _lib.orc_linear_attn_relu.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, _f32p,
                                       C.c_void_p, C.c_void_p, C.c_int]
 _lib.orc_linear_attn_relu.restype = None
+_lib.orc_rms_norm.argtypes = [_f32p, _f32p, C.c_double, C.c_int, C.c_int, _f32p]
+_lib.orc_rms_norm.restype = None
 _lib.orc_linear.argtypes = [_f32p, _f32p, C.c_void_p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int]
 _lib.orc_linear.restype = None
 _lib.orc_max_threads.restype = C.c_int
@@ -232,6 +234,29 @@ def linear_attn_relu(q, k, v, num_heads, eps=1e-15, return_state=False, n_thread
     z = np.empty((num_heads, d), dtype=np.float32) if return_state else None
     _lib.orc_linear_attn_relu(q, k, v, N, num_heads, d, eps, out, _ptr(S), _ptr(z), n_threads)
     return (out, S, z) if return_state else out
+
+
+def rms_norm(x, gain, eps):
+    """Row-wise RMS normalisation of a (rows, cols) array with a (cols) gain."""
+    x = _f32(x)
+    rows, cols = x.shape
+    out = np.empty_like(x)
+    _lib.orc_rms_norm(x, _f32(gain).reshape(cols), float(eps), rows, cols, out)
+    return out
+
+
+def headnorm_rope(x, gain, eps, cos, sin, num_heads, head_dim, round_to_dtype="fp32", round_between=None):
+    """headnorm then rope_apply (src/dit/qwenimage21_forward.cpp:582-585) on x (L, heads*head_dim). round_between
+    names the dtype the normalised tensor is rounded to before the rotation, as the reference's two passes do;
+    None keeps FP32 in between (what the fused kernel computes)."""
+    x = _f32(x)
+    L = x.shape[0]
+    y = rms_norm(x.reshape(L * num_heads, head_dim), gain, eps).reshape(L, num_heads * head_dim)
+    if round_between is not None:
+        y = round_to(y, round_between)
+    if cos is None:
+        return round_to(y, round_to_dtype)
+    return rope_apply(y, cos, sin, num_heads, head_dim, round_to_dtype=round_to_dtype)
 
 
 def linear(x, w, bias=None, n_threads=0):

@@ -22,6 +22,9 @@
 //                              Fully masked row -> zeros follows src/dit/common.cpp:293; what
 //                              brotensor's flash kernel does there is "parity unpinned".
 //   orc_linear_attn_relu       pinned: quadratic-form brute force, (S,z) additivity over token chunks
+//   orc_rms_norm               pinned: torch.nn.functional.rms_norm in float64, unit-RMS invariant, scale
+//                              invariance; eps placement (inside the square root) follows diffusers'
+//                              RMSNorm — brotensor's own is "parity unpinned"
 //   orc_linear                 pinned: numpy float64 matmul, identity weight, one-hot rows.
 //                              WHERE the fused projection operators round their intermediates
 //                              (Q, K, V, attention output to the tensor dtype) is "parity unpinned":
@@ -479,6 +482,24 @@ ORC_API void orc_linear_attn_relu(const float* q, const float* k, const float* v
                 orow[i] = static_cast<float>(num) * recip;
             }
         }
+    }
+}
+
+// ─── per-head RMS normalisation ─────────────────────────────────────────────
+// bt::rms_norm_forward(X viewed as (L*heads, head_dim), gain, eps, out) as the DiT blocks use it
+// (headnorm, src/dit/qwenimage21_forward.cpp:53-63; src/dit/flux.cpp:462-469):
+//   y[r][j] = x[r][j] * gain[j] / sqrt(mean_j(x[r][j]^2) + eps)
+// (the RMSNorm of diffusers' Flux / Qwen-Image attention processors, which the reference ports). Sums in
+// double, result stored as float; x is (rows, cols), gain (cols).
+ORC_API void orc_rms_norm(const float* x, const float* gain, double eps, int rows, int cols, float* out) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; ++r) {
+        const float* xr = x + static_cast<size_t>(r) * cols;
+        double ss = 0.0;
+        for (int j = 0; j < cols; ++j) ss += static_cast<double>(xr[j]) * static_cast<double>(xr[j]);
+        const double inv = 1.0 / std::sqrt(ss / cols + eps);
+        for (int j = 0; j < cols; ++j)
+            out[static_cast<size_t>(r) * cols + j] = static_cast<float>(static_cast<double>(xr[j]) * inv * static_cast<double>(gain[j]));
     }
 }
 

@@ -28,6 +28,7 @@ void orc_rows_block_causal(int Lq, int Lk, int q_offset, const int* seg_q_end, c
                            int n_seg, int* row_lo, int* row_hi);
 void orc_linear_attn_relu(const float* q, const float* k, const float* v, int N, int H, int d, float eps, float* out,
                           float* S_out, float* z_out, int n_threads);
+void orc_rms_norm(const float* x, const float* gain, double eps, int rows, int cols, float* out);
 void orc_linear(const float* x, const float* w, const float* bias, int M, int N, int K, float* y, int n_threads);
 }
 
@@ -197,6 +198,25 @@ static void gpu_checks() {
         std::printf("linear attention      rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
         CHECK(state.rows == Hl && state.cols == dl * dl + dl);
+    }
+    {   // headnorm + RoPE in one pass, with the prefix rows also written to a cache tensor
+        const std::vector<int> axes = {16, 56, 56};
+        dit::RopeTables tabs = dit::build_axial_rope_tables(txt, hp, wp, d, axes);
+        std::vector<float> oc(static_cast<size_t>(L) * d / 2), os(oc.size());
+        orc_build_axial_rope_tables(txt, hp, wp, d, axes.data(), 3, 10000.0f, oc.data(), os.data());
+        std::vector<float> gain = randn_bf16(7201, d);
+        Tensor G = upload_bf16(gain, 1, d), out, cache;
+        dit::headnorm_rope(K, G, 1e-6f, &tabs.cos, &tabs.sin, d, H, out, &cache, txt);
+        std::vector<float> normed(k.size()), ref(k.size());
+        orc_rms_norm(k.data(), gain.data(), 1e-6, L * H, d, normed.data());
+        orc_rope_apply(normed.data(), oc.data(), os.data(), L, H, d, 0, 1, ref.data());
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("headnorm + rope       rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(e.rel_l2 <= 5e-3);
+        CHECK(cache.rows == txt && cache.cols == D);
+        const std::vector<uint8_t> ob = out.to_host_bytes(), cb = cache.to_host_bytes();
+        CHECK(std::memcmp(ob.data(), cb.data(), cb.size()) == 0);
+        CHECK(throws_with([&] { Tensor o2; dit::headnorm_rope(K, Q, 1e-6f, nullptr, nullptr, d, H, o2); }, "gain must hold"));
     }
     {   // attention with its projections (SD1.5 level-0 widths: C 320, 8 heads of 40, text context 77 x 768)
         const int Lx = 100, C = 320, Hh = 8, Lc = 77, Cc = 768;

@@ -415,3 +415,42 @@ def test_attention_qkvo_composition(oracle):
     assert np.array_equal(full, by_hand)
     rounded = oracle.attention_qkvo(x, ctx, wq, bq, wk, bk, wv, bv, wo, bo, H, "bf16")
     assert 0 < np.abs(rounded - full).max() < 0.05
+
+
+# ── per-head RMS normalisation ───────────────────────────────────────────────
+def test_rms_norm_vs_torch_float64_and_invariants(oracle):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((37, 128)).astype(np.float32) * 3
+    g = rng.standard_normal(128).astype(np.float32)
+    eps = 1e-6
+    ref = torch.nn.functional.rms_norm(torch.from_numpy(x).double(), (128,), torch.from_numpy(g).double(), eps).numpy()
+    got = oracle.rms_norm(x, g, eps)
+    assert np.allclose(got, ref, rtol=1e-6, atol=1e-7)
+    # unit gain: every row leaves with RMS 1 (eps is negligible against these rows)
+    unit = oracle.rms_norm(x, np.ones(128, np.float32), eps)
+    assert np.allclose(np.sqrt((unit.astype(np.float64) ** 2).mean(axis=1)), 1.0, atol=1e-5)
+    # scale invariance: normalising 5x gives what normalising x gives
+    assert np.allclose(oracle.rms_norm(5 * x, g, 0.0), oracle.rms_norm(x, g, 0.0), rtol=1e-6, atol=1e-7)
+    # eps sits inside the square root: a zero row stays zero, a tiny row is damped by sqrt(eps)
+    tiny = np.full((1, 128), 1e-4, np.float32)
+    assert np.allclose(oracle.rms_norm(tiny, np.ones(128, np.float32), 1e-6), 1e-4 / np.sqrt(1e-8 + 1e-6), rtol=1e-5)
+    assert np.array_equal(oracle.rms_norm(np.zeros((2, 128), np.float32), g, eps), np.zeros((2, 128), np.float32))
+
+
+def test_headnorm_rope_is_norm_then_rotation(oracle):
+    rng = np.random.default_rng(12)
+    L, H, d = 9, 3, 32
+    x = rng.standard_normal((L, H * d)).astype(np.float32)
+    g = rng.standard_normal(d).astype(np.float32)
+    ang = rng.uniform(0, 6.28, (L, d // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    got = oracle.headnorm_rope(x, g, 1e-6, cos, sin, H, d)
+    by_hand = np.empty_like(x)
+    for l in range(L):
+        for h in range(H):
+            row = x[l, h * d:(h + 1) * d].astype(np.float64)
+            y = row / np.sqrt((row ** 2).mean() + 1e-6) * g
+            by_hand[l, h * d:(h + 1) * d:2] = y[0::2] * cos[l] - y[1::2] * sin[l]
+            by_hand[l, h * d + 1:(h + 1) * d:2] = y[0::2] * sin[l] + y[1::2] * cos[l]
+    assert np.allclose(got, by_hand, rtol=1e-5, atol=1e-6)
+    assert np.allclose(oracle.headnorm_rope(x, g, 1e-6, None, None, H, d), oracle.rms_norm(x.reshape(L * H, d), g, 1e-6).reshape(L, H * d))
