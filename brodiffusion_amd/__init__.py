@@ -24,6 +24,7 @@ from .ops import (  # noqa: F401
     rope_apply,
     rope_apply_perhead,
     rope_tables_from_positions,
+    scale_rows,
     sdpa_forward,
     set_sdpa_kernel_choice,
 )
@@ -32,5 +33,5 @@ __all__ = [
     "SdpaMask", "build_axial_rope_tables", "build_qwen_rope_tables", "qwen_rope_positions", "rope_tables_from_positions", "device_info", "flash_attention_forward",
     "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
     "linear_attention_relu_forward", "rope_apply", "flash_attention_qkvo_forward", "flash_attention_q_with_kv_cached_forward",
-    "flash_attention_project_kv", "flash_attention_scratch_bytes", "linear_batched", "headnorm_rope", "rope_apply_perhead", "sdpa_forward", "set_sdpa_kernel_choice",
+    "flash_attention_project_kv", "flash_attention_scratch_bytes", "linear_batched", "headnorm_rope", "scale_rows", "rope_apply_perhead", "sdpa_forward", "set_sdpa_kernel_choice",
 ]

@@ -21,7 +21,7 @@ MI_MAX_SEGMENTS = 32
 EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
-    "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply", "mi_headnorm_rope",
+    "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
     "mi_linear_forward", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
     "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv",
@@ -76,6 +76,15 @@ class MiHeadnormRopeArgs(C.Structure):
         ("eps", C.c_float), ("rows", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32),
         ("x_row_stride", C.c_int64), ("out_row_stride", C.c_int64),
         ("out2", C.c_void_p), ("out2_rows", C.c_int32), ("out2_row_stride", C.c_int64), ("stream", C.c_void_p),
+    ]
+
+
+class MiScaleRowsArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("x", C.c_void_p), ("out", C.c_void_p), ("row_scale", C.c_void_p), ("scale", C.c_float),
+        ("rows", C.c_int32), ("cols", C.c_int32), ("x_row_stride", C.c_int64), ("out_row_stride", C.c_int64),
+        ("stream", C.c_void_p),
     ]
 
 
@@ -151,6 +160,7 @@ def lib() -> C.CDLL:
         L.mi_sdpa_set_kernel_choice.argtypes = [C.c_int32]
         L.mi_rope_apply.argtypes = [C.POINTER(MiRopeArgs)]
         L.mi_headnorm_rope.argtypes = [C.POINTER(MiHeadnormRopeArgs)]
+        L.mi_scale_rows.argtypes = [C.POINTER(MiScaleRowsArgs)]
         L.mi_linear_attn_workspace_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         L.mi_linear_attn_workspace_bytes.restype = C.c_size_t
         L.mi_linear_attn_scratch_bytes.argtypes = [C.c_int32, C.c_int32, C.c_int32]

@@ -109,6 +109,24 @@ __global__ void __launch_bounds__(256) headnorm_rope_kernel(const T* x, T* out, 
     }
 }
 
+// out[r][c] = x[r][c] * scale * (row_scale ? row_scale[r] : 1): one thread per 16-byte chunk.
+template <typename T>
+__global__ void __launch_bounds__(256) scale_rows_kernel(const T* x, T* out, const float* __restrict__ row_scale, float scale,
+                                                         int rows, int cols, long x_rs, long o_rs) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    const int cpr = cols / 8;
+    const long total = static_cast<long>(rows) * cpr;
+    for (long idx = blockIdx.x * 256L + threadIdx.x; idx < total; idx += gridDim.x * 256L) {
+        const int r = static_cast<int>(idx / cpr);
+        const int col = static_cast<int>(idx - static_cast<long>(r) * cpr) * 8;
+        const float f = row_scale ? scale * row_scale[r] : scale;
+        t8 v = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(x + r * x_rs + col));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = static_cast<T>(static_cast<float>(v[e]) * f);
+        *reinterpret_cast<u32x4*>(out + r * o_rs + col) = __builtin_bit_cast(u32x4, v);
+    }
+}
+
 template <typename T>
 int launch_headnorm(const mi_headnorm_rope_args* a, long x_rs, long o_rs, long o2_rs, hipStream_t st) {
     const long work = static_cast<long>(a->rows) * a->num_heads * a->head_dim / 8;
@@ -212,4 +230,35 @@ extern "C" int mi_headnorm_rope(const mi_headnorm_rope_args* a) {
     if (a->dtype == MI_DTYPE_BF16) return mi::launch_headnorm<__bf16>(a, x_rs, o_rs, o2_rs, st);
     if (a->dtype == MI_DTYPE_F16) return mi::launch_headnorm<_Float16>(a, x_rs, o_rs, o2_rs, st);
     return fail("mi_headnorm_rope: dtype %d not supported", a->dtype);
+}
+
+extern "C" int mi_scale_rows(const mi_scale_rows_args* a) {
+    using mi::fail;
+    mi::clear_error();
+    if (!a) return fail("mi_scale_rows: null args");
+    if (a->struct_size != sizeof(mi_scale_rows_args)) return fail("mi_scale_rows: struct_size mismatch");
+    if (a->rows < 0 || a->cols <= 0 || a->cols % 8 != 0) return fail("mi_scale_rows: cols must be a positive multiple of 8, rows >= 0");
+    if (a->rows == 0) return 0;
+    if (!a->x || !a->out) return fail("mi_scale_rows: x and out must not be null");
+    const long x_rs = a->x_row_stride ? a->x_row_stride : a->cols;
+    const long o_rs = a->out_row_stride ? a->out_row_stride : a->cols;
+    if (x_rs < a->cols || o_rs < a->cols || x_rs % 8 != 0 || o_rs % 8 != 0)
+        return fail("mi_scale_rows: row strides must be multiples of 8 elements and at least cols");
+    if ((reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->out)) & 15u) return fail("mi_scale_rows: pointers must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(a->row_scale) & 3u) return fail("mi_scale_rows: row_scale must be 4-byte aligned");
+    const long work = static_cast<long>(a->rows) * (a->cols / 8);
+    long blocks = (work + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    hipStream_t st = mi::resolve_stream(a->stream);
+    if (a->dtype == MI_DTYPE_BF16)
+        hipLaunchKernelGGL(mi::scale_rows_kernel<__bf16>, dim3(blocks), dim3(256), 0, st, static_cast<const __bf16*>(a->x),
+                           static_cast<__bf16*>(a->out), a->row_scale, a->scale, a->rows, a->cols, x_rs, o_rs);
+    else if (a->dtype == MI_DTYPE_F16)
+        hipLaunchKernelGGL(mi::scale_rows_kernel<_Float16>, dim3(blocks), dim3(256), 0, st, static_cast<const _Float16*>(a->x),
+                           static_cast<_Float16*>(a->out), a->row_scale, a->scale, a->rows, a->cols, x_rs, o_rs);
+    else
+        return fail("mi_scale_rows: dtype %d not supported", a->dtype);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("mi_scale_rows launch: %s", hipGetErrorString(e));
+    return 0;
 }

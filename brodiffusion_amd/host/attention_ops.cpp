@@ -403,6 +403,27 @@ void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, con
     run_sdpa(op, a);
 }
 
+void scale_rows(const Tensor& X, float scale, const Tensor* row_scale, Tensor& out) {
+    const char* op = "scale_rows";
+    need_gpu(op, X);
+    if (row_scale) {
+        need_gpu(op, *row_scale);
+        if (row_scale->dtype != Dtype::FP32 || row_scale->size() != static_cast<std::size_t>(X.rows))
+            fail(std::string(op) + ": the row scale holds " + std::to_string(row_scale->size()) + " values but the tensor has " +
+                 std::to_string(X.rows) + " rows");
+    }
+    if (out.data == nullptr || out.rows != X.rows || out.cols != X.cols || out.dtype != X.dtype) out.resize(X.rows, X.cols, X.dtype, X.device);
+    mi_scale_rows_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    a.x = X.data; a.out = out.data;
+    a.row_scale = row_scale ? static_cast<const float*>(row_scale->data) : nullptr;
+    a.scale = scale;
+    a.rows = X.rows; a.cols = X.cols;
+    check(op, mi_scale_rows(&a));
+}
+
 void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix, const Tensor* v_prefix,
                             const std::vector<Segment>& segments, int q_offset, int num_heads, const Tensor* cos_q,
                             const Tensor* sin_q, Tensor& out) {

@@ -94,6 +94,12 @@ void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, con
                           int head_dim, int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out,
                           Tensor& Qr, Tensor& Kr, Tensor& Krep, Tensor& Vrep);
 
+// out = X * scale * row_scale (per row; row_scale: FP32 (rows, 1) / (1, rows) or null). The prefix-KV dial of the
+// Qwen-Image cached step (set_prefix_kv_scale, src/dit/qwenimage21_forward.cpp:612-645): scale a copy of the cached
+// prefix rows and hand the copy to block_causal_attention as k_prefix / v_prefix; the cache itself stays pristine,
+// which is what makes the dial idempotent (tests/test_qwenimage21_slots.cpp:361-412).
+void scale_rows(const Tensor& X, float scale, const Tensor* row_scale, Tensor& out);
+
 // One segment of the Qwen-Image joint sequence (src/dit/qwenimage21_forward.cpp:650-676).
 struct Segment {
     enum class Kind { Text, Image } kind;

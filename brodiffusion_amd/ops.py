@@ -441,6 +441,32 @@ def rope_apply_perhead(X, cos, sin, head_dim: int, num_heads: int, out: Optional
     return _rope("rope_apply_perhead", X, cos, sin, head_dim, num_heads, out, True, split_half)
 
 
+def scale_rows(X, scale: float = 1.0, row_scale: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """out = X * scale * row_scale[:, None]: the prefix-KV dial of the Qwen-Image cached step
+    (src/dit/qwenimage21_forward.cpp:612-645) applied to a copy of the prefix rows, the cache itself untouched."""
+    op = "scale_rows"
+    _dev(op, X, row_scale, out)
+    if X.dim() != 2 or X.stride(1) != 1:
+        _fail(op, "X must be 2-D, contiguous along columns")
+    if out is None:
+        out = torch.empty_like(X)
+    if out.shape != X.shape or out.dtype != X.dtype or out.stride(1) != 1:
+        _fail(op, "out must have X's shape and dtype")
+    a = capi.MiScaleRowsArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, X)
+    a.x, a.out, a.scale = X.data_ptr(), out.data_ptr(), float(scale)
+    if row_scale is not None:
+        if row_scale.dtype != torch.float32 or row_scale.numel() != X.shape[0] or not row_scale.is_contiguous():
+            _fail(op, f"row_scale must hold {X.shape[0]} float32 values (one per row)")
+        a.row_scale = row_scale.data_ptr()
+    a.rows, a.cols = X.shape
+    a.x_row_stride, a.out_row_stride = X.stride(0), out.stride(0)
+    a.stream = _stream()
+    capi.check(capi.lib().mi_scale_rows(C.byref(a)), op)
+    return out
+
+
 def headnorm_rope(X, gain, eps: float, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
                   cache_out: Optional[torch.Tensor] = None):
     """headnorm + rope_apply of the DiT blocks (src/dit/qwenimage21_forward.cpp:582-585, src/dit/flux.cpp:462-469) in

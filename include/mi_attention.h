@@ -212,6 +212,25 @@ typedef struct mi_headnorm_rope_args {
 } mi_headnorm_rope_args;
 MI_API int mi_headnorm_rope(const mi_headnorm_rope_args* args);
 
+/* ── row scaling ───────────────────────────────────────────────────────────
+ * out[r][c] = x[r][c] * scale * (row_scale ? row_scale[r] : 1), one rounding. The prefix-KV dial of the Qwen-Image
+ * cached step (set_prefix_kv_scale: a per-layer scalar, or per-token weights with the scalars folded in,
+ * src/dit/qwenimage21_forward.cpp:612-645): the reference scales the prefix rows of its assembled [cache ; fresh]
+ * copy and leaves the cache pristine; here the scaled prefix (prefix_len rows only) goes to a scratch that is then
+ * passed as k_prefix / v_prefix. row_scale: device FP32 [rows] or NULL. In place (out == x) is allowed. */
+typedef struct mi_scale_rows_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* x;
+    void* out;
+    const float* row_scale;
+    float scale;
+    int32_t rows, cols;
+    int64_t x_row_stride, out_row_stride;
+    void* stream;
+} mi_scale_rows_args;
+MI_API int mi_scale_rows(const mi_scale_rows_args* args);
+
 /* ── ReLU linear attention ─────────────────────────────────────────────────
  * Per (batch, head): Kr = relu(K), Qr = relu(Q); S = V^T Kr (d x d), z = sum_n Kr (d);
  * O[n] = (S Qr[n]) / (z . Qr[n] + eps). Replaces the core of

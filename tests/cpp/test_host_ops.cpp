@@ -185,6 +185,54 @@ static void gpu_checks() {
         std::printf("block-causal          rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
     }
+    {   // the prefix-KV dial, as tests/test_qwenimage21_slots.cpp:361-412 exercises it: armed it changes the cached
+        // step, set twice it is the same picture (the cache stays pristine), two halvings equal one quarter,
+        // identity scales are the unscaled step bit for bit
+        const int prefix = 21;
+        Tensor kp = K.row_view(0, prefix), vp = V.row_view(0, prefix);
+        Tensor Qt = Q.row_view(prefix, L - prefix), Kt = K.row_view(prefix, L - prefix), Vt = V.row_view(prefix, L - prefix);
+        const std::vector<dit::Segment> seg = {{dit::Segment::Kind::Image, L - prefix}};
+        auto step = [&](float ks, float vs) {
+            Tensor ksc, vsc, o;
+            dit::scale_rows(kp, ks, nullptr, ksc);
+            dit::scale_rows(vp, vs, nullptr, vsc);
+            dit::block_causal_attention(Qt, Kt, Vt, &ksc, &vsc, seg, prefix, H, nullptr, nullptr, o);
+            return o.to_host_bytes();
+        };
+        Tensor o_plain;
+        dit::block_causal_attention(Qt, Kt, Vt, &kp, &vp, seg, prefix, H, nullptr, nullptr, o_plain);
+        const std::vector<uint8_t> cache_before = kp.to_host_bytes();
+        const std::vector<uint8_t> plain = o_plain.to_host_bytes(), halved = step(1.0f, 0.5f), again = step(1.0f, 0.5f);
+        CHECK(plain != halved);
+        CHECK(halved == again);
+        CHECK(step(1.0f, 1.0f) == plain);
+        CHECK(kp.to_host_bytes() == cache_before);
+        // composition: scaling the already halved copy by 0.5 is the quarter dial (powers of two are exact)
+        Tensor vh, vq, o_q;
+        dit::scale_rows(vp, 0.5f, nullptr, vh);
+        dit::scale_rows(vh, 0.5f, nullptr, vq);
+        dit::block_causal_attention(Qt, Kt, Vt, &kp, &vq, seg, prefix, H, nullptr, nullptr, o_q);
+        CHECK(o_q.to_host_bytes() == step(1.0f, 0.25f));
+        // per-token weights against the checker: keys scaled before the scores, values before the sum
+        std::vector<float> wk(prefix), wv(prefix);
+        for (int i = 0; i < prefix; ++i) { wk[i] = 0.5f + 0.05f * i; wv[i] = 1.5f - 0.04f * i; }
+        Tensor Wk = Tensor::from_host(wk.data(), prefix, 1, Dtype::FP32), Wv = Tensor::from_host(wv.data(), prefix, 1, Dtype::FP32), ksc, vsc, o_w;
+        dit::scale_rows(kp, 0.8f, &Wk, ksc);
+        dit::scale_rows(vp, 1.0f, &Wv, vsc);
+        dit::block_causal_attention(Qt, Kt, Vt, &ksc, &vsc, seg, prefix, H, nullptr, nullptr, o_w);
+        std::vector<float> k2 = k, v2 = v;
+        for (int i = 0; i < prefix; ++i)
+            for (int c = 0; c < D; ++c) { k2[static_cast<size_t>(i) * D + c] *= 0.8f * wk[i]; v2[static_cast<size_t>(i) * D + c] *= wv[i]; }
+        orc_round_bf16(k2.data(), static_cast<size_t>(prefix) * D);   // the scaled copy is a bf16 tensor, in the reference too
+        orc_round_bf16(v2.data(), static_cast<size_t>(prefix) * D);
+        std::vector<float> ref(static_cast<size_t>(L - prefix) * D);
+        orc_sdpa(q.data() + static_cast<size_t>(prefix) * D, k2.data(), v2.data(), L - prefix, L, H, d, -1.0, nullptr, nullptr, nullptr, nullptr,
+                 nullptr, 0, 0, nullptr, 0, ref.data(), nullptr, 0);
+        const Err e = compare(ref, download_bf16(o_w));
+        std::printf("prefix-KV dial        rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        CHECK(throws_with([&] { Tensor o2; dit::scale_rows(kp, 1.0f, &Wk, o2); dit::scale_rows(K, 1.0f, &Wk, o2); }, "the row scale holds 21 values"));
+    }
     {   // ReLU linear attention, 70 x 32 (the reference's own head split) on a short sequence
         const int Hl = 70, dl = 32, N = 96, Dl = Hl * dl;
         const std::vector<float> ql = randn_bf16(7011, static_cast<size_t>(N) * Dl), kl = randn_bf16(7012, static_cast<size_t>(N) * Dl),

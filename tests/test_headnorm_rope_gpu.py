@@ -75,3 +75,39 @@ def test_headnorm_rope_errors():
     with pytest.raises(RuntimeError, match="not on the GPU"):
         bd.headnorm_rope(z(4, 256).cpu(), z(128), 1e-6, None, None, 128, 2)
     assert bd.headnorm_rope(z(0, 256), z(128), 1e-6, None, None, 128, 2).shape == (0, 256)
+
+
+# ── row scaling: the prefix-KV dial ──────────────────────────────────────────
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_scale_rows(oracle, dtype):
+    rows, cols = 77, 3072
+    x = randn(9200, (rows, cols), dtype)
+    w = (0.25 + np.arange(rows, dtype=np.float32) / 64).astype(np.float32)
+    dx = to_dev(x, dtype)
+    dw = torch.from_numpy(w).cuda()
+    got = bd.scale_rows(dx, 0.75, dw)
+    ref = oracle.round_to(x * (np.float32(0.75) * w)[:, None], dtype)          # one FP32 product, one rounding
+    assert np.array_equal(to_np(got), ref)
+    assert torch.equal(bd.scale_rows(dx, 1.0), dx)
+    assert torch.equal(bd.scale_rows(bd.scale_rows(dx, 0.5), 0.5), bd.scale_rows(dx, 0.25))
+    # in place on a row slice of a larger buffer
+    buf = torch.zeros(rows + 3, cols, device="cuda", dtype=dx.dtype)
+    buf[1:rows + 1] = dx
+    bd.scale_rows(buf[1:rows + 1], 0.75, dw, out=buf[1:rows + 1])
+    assert torch.equal(buf[1:rows + 1], got) and (buf[0] == 0).all() and (buf[rows + 1:] == 0).all()
+    with pytest.raises(RuntimeError, match="row_scale must hold 77"):
+        bd.scale_rows(dx, 1.0, dw[:5])
+
+
+def test_prefix_dial_equals_scaled_keys_and_values(oracle):
+    """Attention over [scaled prefix ; fresh] against the checker fed the same scaled rows."""
+    dtype, H, d, prefix, Lq = "bf16", 4, 128, 96, 200
+    q, kf, vf = (randn(9300 + i, (Lq, H * d), dtype) for i in range(3))
+    kp, vp = randn(9304, (prefix, H * d), dtype), randn(9305, (prefix, H * d), dtype)
+    dq, dkf, dvf, dkp, dvp = (to_dev(t, dtype) for t in (q, kf, vf, kp, vp))
+    ks, vs = bd.scale_rows(dkp, 0.5), bd.scale_rows(dvp, 1.25)
+    out = bd.sdpa_forward(dq, dkf, dvf, H, k_prefix=ks, v_prefix=vs)
+    k = np.concatenate([oracle.round_to(kp * np.float32(0.5), dtype), kf])
+    v = np.concatenate([oracle.round_to(vp * np.float32(1.25), dtype), vf])
+    assert_close(oracle.sdpa(q, k, v, H), to_np(out), dtype, "prefix dial")
+    assert not torch.equal(out, bd.sdpa_forward(dq, dkf, dvf, H, k_prefix=dkp, v_prefix=dvp))
