@@ -21,7 +21,7 @@ MI_MAX_SEGMENTS = 32
 EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
-    "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
+    "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_attention_map_avg", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
     "mi_linear_forward", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
     "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv",
@@ -54,8 +54,21 @@ class MiSdpaArgs(C.Structure):
         ("seg_causal", C.c_int32 * MI_MAX_SEGMENTS),
         ("rope_cos_q", C.c_void_p), ("rope_sin_q", C.c_void_p), ("rope_cos_k", C.c_void_p), ("rope_sin_k", C.c_void_p),
         ("rope_k_scratch", C.c_void_p),
+        ("logit_bias", C.c_void_p), ("bias_q0", C.c_int32), ("bias_cols", C.c_int32), ("bias_row_stride", C.c_int64),
+        ("lse_out", C.c_void_p),
         ("split_scratch", C.c_void_p), ("split_scratch_bytes", C.c_size_t),
         ("stream", C.c_void_p),
+    ]
+
+
+class MiAttentionMapArgs(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32), ("dtype", C.c_int32),
+        ("q", C.c_void_p), ("k", C.c_void_p), ("lse", C.c_void_p), ("map", C.c_void_p),
+        ("num_heads", C.c_int32), ("head_dim", C.c_int32), ("q_len", C.c_int32), ("kv_len", C.c_int32),
+        ("q_row_stride", C.c_int64), ("k_row_stride", C.c_int64), ("map_row_stride", C.c_int64),
+        ("scale", C.c_float), ("logit_bias", C.c_void_p), ("bias_q0", C.c_int32), ("bias_cols", C.c_int32),
+        ("bias_row_stride", C.c_int64), ("stream", C.c_void_p),
     ]
 
 
@@ -158,6 +171,7 @@ def lib() -> C.CDLL:
         L.mi_sdpa_split_scratch_bytes.restype = C.c_size_t
         L.mi_sdpa_supported.argtypes = [C.c_int32, C.c_int32]
         L.mi_sdpa_set_kernel_choice.argtypes = [C.c_int32]
+        L.mi_attention_map_avg.argtypes = [C.POINTER(MiAttentionMapArgs)]
         L.mi_rope_apply.argtypes = [C.POINTER(MiRopeArgs)]
         L.mi_headnorm_rope.argtypes = [C.POINTER(MiHeadnormRopeArgs)]
         L.mi_scale_rows.argtypes = [C.POINTER(MiScaleRowsArgs)]

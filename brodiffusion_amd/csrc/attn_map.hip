@@ -1,0 +1,143 @@
+// Head-averaged attention map for traced forwards: map[q][k] = (1/H) sum_h softmax_h(q, k), FP32, for batch 1.
+//
+// The flash kernels never materialise the softmax; a traced forward wants it averaged over heads. The attention
+// launch leaves the base-2 log of every row's denominator (lse, per head and query row); this kernel recomputes the
+// scores tile by tile and turns them into probabilities with it. One work group owns a (128 query rows x 64 keys)
+// tile of the map and loops over the heads, so every map element is accumulated in one register and written once —
+// no atomics, deterministic. Scores are computed transposed (S^T = K Q^T, as in the attention kernels): a lane owns
+// one query row, so lse and the bias row are per-lane scalars, and holds 4 consecutive keys per accumulator group,
+// which leave as 16-byte stores.
+// Per head a work group reads its K tile (64 x d, through LDS) and its Q rows (128 x d, straight into the B operands).
+#include "sdpa_common.h"
+
+namespace mi {
+namespace {
+
+using namespace sdpa;
+
+constexpr int kMapThreads = 256;
+constexpr int kMapRows = 128;
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    __shared__ __attribute__((aligned(16))) unsigned char Ks[G::K_BYTES];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    const int j0 = static_cast<int>(blockIdx.x) * kBN;
+    const int q0 = static_cast<int>(blockIdx.y) * kMapRows;
+    const int qrow = q0 + wave * 32 + lq;
+    const bool qvalid = qrow < p.Lq;
+    const int qr = qvalid ? qrow : p.Lq - 1;   // rows past the end repeat the last one and are never stored
+    const float* const bias_row = (p.bias && qvalid && qrow >= p.bias_q0 && j0 < p.bias_cols)
+                                      ? p.bias + static_cast<long>(qrow - p.bias_q0) * p.bias_rs : nullptr;
+    constexpr float kLog2e = 1.4426950408889634f;
+
+    // the zero pad of the head dimension (columns D .. DK-1) is written once; data chunks are rewritten per head
+    for (int i = tid; i < G::K_BYTES / 16; i += kMapThreads) reinterpret_cast<u32x4*>(Ks)[i] = u32x4{0u, 0u, 0u, 0u};
+    __syncthreads();
+
+    f32x16 avg[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) avg[kb][e] = 0.f;
+
+    const T* const qg = static_cast<const T*>(p.q);
+    const T* const kg = static_cast<const T*>(p.k);
+    for (int h = 0; h < p.H; ++h) {
+        // K tile of head h: rows past the last key stay zero (their probabilities are discarded below)
+        for (int idx = tid; idx < kBN * G::CPR; idx += kMapThreads) {
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            u32x4 v = u32x4{0u, 0u, 0u, 0u};
+            if (j0 + row < p.Lk) v = *reinterpret_cast<const u32x4*>(kg + static_cast<long>(j0 + row) * p.k_rs + h * D + cc * 8);
+            *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = v;
+        }
+        // this lane's query row as B operands: 8 contraction elements at 16 c + 8 lh
+        V8 qf[G::KC];
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) {
+            const int col = 16 * c + 8 * lh;
+            u32x4 v = u32x4{0u, 0u, 0u, 0u};
+            if (col < D) v = *reinterpret_cast<const u32x4*>(qg + static_cast<long>(qr) * p.q_rs + h * D + col);
+            qf[c] = __builtin_bit_cast(V8, v);
+        }
+        const float lse = p.lse[static_cast<long>(h) * p.Lq + qr];
+        __syncthreads();
+        f32x16 sacc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[kb][e] = 0.f;
+#pragma unroll
+            for (int c = 0; c < G::KC; ++c) {
+                const u32x4 a = *reinterpret_cast<const u32x4*>(Ks + (32 * kb + lq) * G::K_STRIDE + (2 * c + lh) * 16);
+                sacc[kb] = Mma<T>::run(__builtin_bit_cast(V8, a), qf[c], sacc[kb]);
+            }
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                float s2 = sacc[kb][e] * p.scale_log2;
+                if (bias_row && key < p.bias_cols) s2 = __builtin_fmaf(bias_row[key], kLog2e, s2);
+                avg[kb][e] += __builtin_amdgcn_exp2f(s2 - lse);
+            }
+        __syncthreads();   // all reads of this head's K tile are done before the next head overwrites it
+    }
+
+    if (!qvalid) return;
+    const float inv_h = 1.0f / static_cast<float>(p.H);
+    float* const row = p.map + static_cast<long>(qrow) * p.map_rs;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+            const int key = j0 + 32 * kb + 8 * bb + 4 * lh;
+            if (key + 3 < p.Lk && (p.map_rs & 3) == 0) {
+                *reinterpret_cast<f32x4*>(row + key) = f32x4{avg[kb][4 * bb] * inv_h, avg[kb][4 * bb + 1] * inv_h,
+                                                             avg[kb][4 * bb + 2] * inv_h, avg[kb][4 * bb + 3] * inv_h};
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (key + i < p.Lk) row[key + i] = avg[kb][4 * bb + i] * inv_h;
+            }
+        }
+}
+
+template <typename T, int D>
+int launch_map_d(const MapDev& p, hipStream_t st) {
+    const dim3 grid((p.Lk + kBN - 1) / kBN, (p.Lq + kMapRows - 1) / kMapRows);
+    hipLaunchKernelGGL((attn_map_kernel<T, D>), grid, dim3(kMapThreads), 0, st, p);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("mi_attention_map_avg launch: %s", hipGetErrorString(e));
+    return 0;
+}
+
+template <typename T>
+int launch_map_t(const MapDev& p, int head_dim, hipStream_t st) {
+    switch (head_dim) {
+        case 40: return launch_map_d<T, 40>(p, st);
+        case 64: return launch_map_d<T, 64>(p, st);
+        case 72: return launch_map_d<T, 72>(p, st);
+        case 80: return launch_map_d<T, 80>(p, st);
+        case 96: return launch_map_d<T, 96>(p, st);
+        case 112: return launch_map_d<T, 112>(p, st);
+        case 128: return launch_map_d<T, 128>(p, st);
+        case 160: return launch_map_d<T, 160>(p, st);
+        default: return fail("mi_attention_map_avg: head_dim %d has no kernel", head_dim);
+    }
+}
+
+}  // namespace
+
+int launch_attention_map(const MapDev& p, int dtype, int head_dim, hipStream_t stream) {
+    if (dtype == MI_DTYPE_BF16) return launch_map_t<__bf16>(p, head_dim, stream);
+    if (dtype == MI_DTYPE_F16) return launch_map_t<_Float16>(p, head_dim, stream);
+    return fail("mi_attention_map_avg: dtype %d not supported", dtype);
+}
+
+}  // namespace mi

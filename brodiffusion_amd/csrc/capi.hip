@@ -187,6 +187,20 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
     for (const void* t : tabs)
         if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
     p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
+    p.inv_scale = 1.0f / scale;
+    if (a->logit_bias) {
+        if (a->batch != 1) return fail("mi_sdpa_forward: logit_bias needs batch 1");
+        if (a->bias_q0 < 0 || a->bias_cols < 0 || a->bias_cols > Lk) return fail("mi_sdpa_forward: bias_q0 / bias_cols out of range");
+        p.bias = a->logit_bias; p.bias_q0 = a->bias_q0; p.bias_cols = a->bias_cols;
+        p.bias_rs = a->bias_row_stride ? a->bias_row_stride : a->bias_cols;
+        if (p.bias_rs < p.bias_cols) return fail("mi_sdpa_forward: bias_row_stride smaller than bias_cols");
+        if (reinterpret_cast<uintptr_t>(a->logit_bias) & 3u) return fail("mi_sdpa_forward: logit_bias must be 4-byte aligned");
+        if (a->bias_cols == 0 || a->bias_q0 >= a->q_len) p.bias = nullptr;   // nothing to add
+    }
+    if (a->lse_out) {
+        if (reinterpret_cast<uintptr_t>(a->lse_out) & 3u) return fail("mi_sdpa_forward: lse_out must be 4-byte aligned");
+        p.lse = a->lse_out;
+    }
     if (a->rope_k_scratch && !mi::aligned16(a->rope_k_scratch)) return fail("mi_sdpa_forward: rope_k_scratch must be 16-byte aligned");
     if (a->split_scratch && !mi::aligned16(a->split_scratch)) return fail("mi_sdpa_forward: split_scratch must be 16-byte aligned");
     // the grid pads batch*heads to a multiple of 8 for masked calls
@@ -242,6 +256,38 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
     p.split_scratch = static_cast<unsigned char*>(a->split_scratch);
     p.split_scratch_bytes = a->split_scratch ? a->split_scratch_bytes : 0;
     return mi::launch_sdpa(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
+}
+
+int mi_attention_map_avg(const mi_attention_map_args* a) {
+    mi::clear_error();
+    const char* op = "mi_attention_map_avg";
+    if (!a) return fail("%s: null args", op);
+    if (a->struct_size != sizeof(mi_attention_map_args)) return fail("%s: struct_size mismatch", op);
+    if (!mi::sdpa_supported(a->dtype, a->head_dim)) return fail("%s: no kernel for dtype %d head_dim %d", op, a->dtype, a->head_dim);
+    if (a->num_heads <= 0 || a->q_len < 0 || a->kv_len < 0) return fail("%s: bad shape", op);
+    if (a->q_len == 0 || a->kv_len == 0) return 0;
+    if (!a->q || !a->k || !a->lse || !a->map) return fail("%s: q, k, lse and map must not be null", op);
+    const long D = static_cast<long>(a->num_heads) * a->head_dim;
+    mi::MapDev p;
+    std::memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.lse = a->lse; p.map = a->map;
+    p.H = a->num_heads; p.Lq = a->q_len; p.Lk = a->kv_len;
+    p.q_rs = a->q_row_stride ? a->q_row_stride : D;
+    p.k_rs = a->k_row_stride ? a->k_row_stride : D;
+    p.map_rs = a->map_row_stride ? a->map_row_stride : a->kv_len;
+    if (p.q_rs < D || p.k_rs < D || p.map_rs < a->kv_len) return fail("%s: a row stride is smaller than its row", op);
+    if (p.q_rs % 8 || p.k_rs % 8) return fail("%s: q / k row strides must be multiples of 8 elements", op);
+    if (!mi::aligned16(a->q) || !mi::aligned16(a->k) || !mi::aligned16(a->map)) return fail("%s: q, k and map must be 16-byte aligned", op);
+    if ((reinterpret_cast<uintptr_t>(a->lse) | reinterpret_cast<uintptr_t>(a->logit_bias)) & 3u) return fail("%s: lse and logit_bias must be 4-byte aligned", op);
+    const float scale = a->scale > 0.f ? a->scale : 1.0f / std::sqrt(static_cast<float>(a->head_dim));
+    p.scale_log2 = scale * 1.4426950408889634f;
+    if (a->logit_bias && a->bias_cols > 0 && a->bias_q0 < a->q_len) {
+        if (a->bias_q0 < 0 || a->bias_cols > a->kv_len) return fail("%s: bias_q0 / bias_cols out of range", op);
+        p.bias = a->logit_bias; p.bias_q0 = a->bias_q0; p.bias_cols = a->bias_cols;
+        p.bias_rs = a->bias_row_stride ? a->bias_row_stride : a->bias_cols;
+        if (p.bias_rs < p.bias_cols) return fail("%s: bias_row_stride smaller than bias_cols", op);
+    }
+    return mi::launch_attention_map(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
 }
 
 }  // extern "C"

@@ -73,6 +73,10 @@ struct SdpaDev {
     const float* cos_q; const float* sin_q;
     const float* cos_k; const float* sin_k;
     int n_q_tiles; int n_blocks;  // logical work items = B*H*n_q_tiles
+    // additive logit bias (natural-log units, added to the scaled score) for query rows >= bias_q0 and keys < bias_cols
+    const float* bias; int bias_q0, bias_cols; long bias_rs;
+    float inv_scale;              // 1 / scale: the bias in units of the raw dot product
+    float* lse;                   // [B][H][Lq] base-2 log of the softmax denominator in exponent units, or null
     SplitGeo split;               // enabled != 0: split the last round along the key axis
     unsigned char* split_scratch; // partial slots, [8 groups][max_tail][max_parts] of SplitGeo::slot_bytes
     size_t split_scratch_bytes;   // what the caller lent
@@ -90,6 +94,18 @@ int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 // Scratch bytes with which launch_sdpa would split the last round of this launch (0: it would not split).
 size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim);
 bool sdpa_supported(int dtype, int head_dim);
+
+// Device-side view of the head-averaged attention map launch (batch 1).
+struct MapDev {
+    const void* q; const void* k;
+    const float* lse;             // [H][Lq], as written by the attention launch
+    float* map;                   // (Lq, Lk) FP32
+    int H, Lq, Lk;
+    long q_rs, k_rs, map_rs;
+    float scale_log2;
+    const float* bias; int bias_q0, bias_cols; long bias_rs;
+};
+int launch_attention_map(const MapDev& p, int dtype, int head_dim, hipStream_t stream);
 
 // One Y = X W^T + bias problem: X (M, K), W (N, K), Y (M, N), bias (N) or null; strides in elements.
 struct LinearProblem {

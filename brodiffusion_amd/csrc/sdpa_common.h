@@ -284,8 +284,19 @@ struct SoftmaxState {
 template <typename T, int D>
 __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
                                              SoftmaxState& st, float cl2, float lazy_raw, bool masked, int j0, int lo, int hi,
-                                             int lh, const float* mask_tile) {
+                                             int lh, const float* mask_tile, const float* bias_row = nullptr, int bias_cols = 0,
+                                             float bias_k = 0.f) {
     if (masked) {
+        // additive logit bias of this lane's query row (null: none) for keys below bias_cols, in raw-score units
+        if (bias_row) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                    if (key < bias_cols) sacc[kb][e] = __builtin_fmaf(bias_row[key], bias_k, sacc[kb][e]);
+                }
+        }
         // mask_tile: the 64 key-mask values of this tile staged in LDS (null when the call has no key mask)
         if (mask_tile) {
 #pragma unroll

@@ -244,6 +244,7 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
     const float* const key_mask = p.key_mask ? p.key_mask + b * p.key_mask_bs : nullptr;
+    const float* const bias_row = (p.bias && qvalid && qrow >= p.bias_q0) ? p.bias + static_cast<long>(qrow - p.bias_q0) * p.bias_rs : nullptr;
 
     int lo, hi;
     row_interval(p, b, qrow, qvalid, lo, hi);
@@ -303,8 +304,10 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
             f32x16 sacc[2];
             V8 pf[4];
             mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
-            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim)) && (key_mask == nullptr);
-            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, Ms);
+            const bool biased = p.bias != nullptr && j0 < p.bias_cols;
+            const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim)) && (key_mask == nullptr) && !biased;
+            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, Ms,
+                               biased ? bias_row : nullptr, p.bias_cols, p.inv_scale);
             mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
         }
         if (t + 1 < n_tiles) {
@@ -323,6 +326,10 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
 
     const float l_tot = exchange_sum(st.l);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    // base-2 log of the row's denominator in exponent units: p(key) = exp2(score * scale_log2 [+ bias * log2 e] - lse);
+    // +inf for a row without visible keys, so that every p is 0
+    if (p.lse && qvalid && lh == 0)
+        p.lse[(static_cast<long>(b) * p.H + h) * p.Lq + qrow] = l_tot > 0.f ? st.mc + __builtin_amdgcn_logf(l_tot) : __builtin_huge_valf();
     stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
     __syncthreads();
     write_output<T, D, kThreads4>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
@@ -1008,7 +1015,9 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int choice = sdpa_kernel_choice();
     // calls with a key mask stay on the 128-row kernel, which stages the mask tile in LDS
-    const bool pingpong = D <= 128 && p.key_mask == nullptr && (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
+    // ... and so do calls with a logit bias or a request for the softmax denominators
+    const bool pingpong = D <= 128 && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr &&
+                          (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
     if (pingpong) {
         p.n_q_tiles = (p.Lq + 255) / 256;
         p.n_blocks = static_cast<int>(tiles256);

@@ -384,6 +384,41 @@ void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Te
     run_sdpa(op, a);
 }
 
+void joint_attention_traced(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin,
+                            int head_dim, int num_heads, Tensor& out, Tensor& attn_avg, Tensor& Qr, Tensor& Kr, int txt_len,
+                            const Tensor* image_text_bias) {
+    const char* op = "joint_attention_traced";
+    bt::rope_apply(Q, cos, sin, head_dim, num_heads, Qr);
+    bt::rope_apply(K, cos, sin, head_dim, num_heads, Kr);
+    const int D = Q.cols, L = Q.rows;
+    if (head_dim <= 0 || num_heads <= 0 || D != head_dim * num_heads) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if (K.rows != L || V.rows != L || K.cols != D || V.cols != D) fail(std::string(op) + ": Q/K/V must share shape (L, D)");
+    const float* bias = nullptr;
+    if (image_text_bias != nullptr) {
+        if (txt_len < 0 || txt_len > L) fail(std::string(op) + ": txt_len out of range for bias");
+        if (image_text_bias->dtype != Dtype::FP32) fail(std::string(op) + ": image_text_bias must be FP32");
+        if (image_text_bias->rows != L - txt_len || image_text_bias->cols != txt_len) fail(std::string(op) + ": image_text_bias must be (img_len, txt_len)");
+        need_gpu(op, *image_text_bias);
+        if (txt_len > 0 && txt_len < L) bias = static_cast<const float*>(image_text_bias->data);
+    }
+    static thread_local Tensor* lse = new Tensor;   // per-thread scratch, never destroyed (see thread_scratch)
+    if (lse->data == nullptr || lse->size() < static_cast<std::size_t>(num_heads) * L) lse->resize(num_heads, L, Dtype::FP32, Device::GPU);
+    mi_sdpa_args a;
+    init_args(a, op, Qr, Kr, V, num_heads, num_heads, out);
+    a.logit_bias = bias; a.bias_q0 = txt_len; a.bias_cols = bias ? txt_len : 0;
+    a.lse_out = static_cast<float*>(lse->data);
+    check(op, mi_sdpa_forward(&a));
+    if (attn_avg.data == nullptr || attn_avg.rows != L || attn_avg.cols != L || attn_avg.dtype != Dtype::FP32) attn_avg.resize(L, L, Dtype::FP32, Q.device);
+    mi_attention_map_args m;
+    std::memset(&m, 0, sizeof(m));
+    m.struct_size = sizeof(m);
+    m.dtype = a.dtype;
+    m.q = Qr.data; m.k = Kr.data; m.lse = a.lse_out; m.map = static_cast<float*>(attn_avg.data);
+    m.num_heads = num_heads; m.head_dim = head_dim; m.q_len = L; m.kv_len = L;
+    m.logit_bias = bias; m.bias_q0 = txt_len; m.bias_cols = a.bias_cols;
+    check(op, mi_attention_map_avg(&m));
+}
+
 void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin, int head_dim,
                           int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out, Tensor& /*Qr*/, Tensor& Kr,
                           Tensor& /*Krep*/, Tensor& /*Vrep*/) {

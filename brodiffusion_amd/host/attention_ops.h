@@ -6,6 +6,7 @@
 //   bt::rope_apply / rope_apply_perhead    src/dit/common.cpp:192, src/triposplat/flow_model.cpp:374
 //   dit::joint_attention                   include/brodiffusion/dit/common.h:80-88
 //   dit::gqa_attention_masked              include/brodiffusion/dit/common.h:144-153
+//   dit::joint_attention_traced            include/brodiffusion/dit/common.h:117-129
 //   dit::build_axial_rope_tables           include/brodiffusion/dit/common.h:70-72
 //   bt::flash_attention_qkvo_forward       src/unet_blocks.cpp:264-272
 //   bt::flash_attention_q_with_kv_cached_forward  src/unet_blocks.cpp:311-317
@@ -89,6 +90,14 @@ void headnorm_rope(const Tensor& X, const Tensor& gain, float eps, const Tensor*
 // Qr is accepted and left untouched.
 void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin,
                      int head_dim, int num_heads, Tensor& out, Tensor& Qr, Tensor& Kr);
+
+// joint_attention with the softmax exposed, entirely on the device (the reference downloads Q, K, V and loops on the
+// host, src/dit/common.cpp:198-329): RoPE on Q and K into Qr / Kr, attention with the optional image->text steering
+// bias ((L - txt_len, txt_len) FP32, added to the scaled scores of image rows against text keys), `attn_avg` = the
+// (L, L) FP32 softmax averaged over the heads.
+void joint_attention_traced(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor& cos, const Tensor& sin,
+                            int head_dim, int num_heads, Tensor& out, Tensor& attn_avg, Tensor& Qr, Tensor& Kr,
+                            int txt_len = 0, const Tensor* image_text_bias = nullptr);
 
 void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* cos, const Tensor* sin,
                           int head_dim, int num_q_heads, int num_kv_heads, const float* d_mask, Tensor& out,

@@ -8,6 +8,7 @@ Names, argument order and error behaviour follow the brotensor operators the ref
     rope_apply(X, cos, sin, head_dim, num_heads, out)                        src/dit/common.cpp:192
     rope_apply_perhead(X, cos, sin, head_dim, num_heads, out)                src/triposplat/flow_model.cpp:374
     joint_attention(Q, K, V, cos, sin, head_dim, num_heads, out, Qr, Kr)     include/brodiffusion/dit/common.h:80-88
+    joint_attention_traced(..., out, attn_avg, Qr, Kr, txt_len, image_text_bias)  include/brodiffusion/dit/common.h:117-129
     gqa_attention_masked(...)                                                include/brodiffusion/dit/common.h:144-153
     build_axial_rope_tables(txt_len, hp, wp, head_dim, axes, theta)          src/dit/common.cpp:116-184
     flash_attention_qkvo_forward(X, Ctx, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out)
@@ -109,6 +110,7 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
                  rope_q: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  rope_k_scratch: Optional[torch.Tensor] = None, split_scratch=None,
+                 logit_bias: Optional[torch.Tensor] = None, bias_q0: int = 0, lse_out: Optional[torch.Tensor] = None,
                  op: str = "sdpa_forward") -> torch.Tensor:
     """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None).
     split_scratch: None = lend the module's own scratch (grown on demand, one per device, shared by all calls of the
@@ -197,6 +199,19 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
         if rope_k_scratch.dtype != q.dtype or not rope_k_scratch.is_contiguous() or rope_k_scratch.numel() < k.numel():
             _fail(op, "rope_k_scratch must be contiguous, of Q's dtype and at least as large as K")
         a.rope_k_scratch = rope_k_scratch.data_ptr()
+    if logit_bias is not None:
+        _dev(op, logit_bias)
+        if logit_bias.dtype != torch.float32 or logit_bias.dim() != 2 or logit_bias.stride(1) != 1:
+            _fail(op, "logit_bias must be a 2-D float32 tensor, contiguous along columns")
+        if logit_bias.shape[0] != Lq - bias_q0:
+            _fail(op, f"logit_bias must have one row per query row from bias_q0 on ({Lq - bias_q0}), has {logit_bias.shape[0]}")
+        a.logit_bias, a.bias_q0, a.bias_cols = logit_bias.data_ptr(), bias_q0, logit_bias.shape[1]
+        a.bias_row_stride = logit_bias.stride(0)
+    if lse_out is not None:
+        _dev(op, lse_out)
+        if lse_out.dtype != torch.float32 or lse_out.numel() != B * num_heads * Lq or not lse_out.is_contiguous():
+            _fail(op, "lse_out must be a contiguous float32 tensor of batch * heads * Lq values")
+        a.lse_out = lse_out.data_ptr()
     a.stream = _stream()
     if split_scratch is not False:
         need = int(capi.lib().mi_sdpa_split_scratch_bytes(C.byref(a)))
@@ -521,6 +536,66 @@ def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optio
     if Kr is not None and (Kr.shape != K.shape or Kr.dtype != K.dtype):
         _fail(op, "Kr must have K's shape and dtype")
     return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), rope_k_scratch=Kr, op=op)
+
+
+def attention_map_avg(q, k, lse, num_heads: int, *, scale: Optional[float] = None, logit_bias: Optional[torch.Tensor] = None,
+                      bias_q0: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(Lq, Lk) float32 map: the softmax of every head averaged over the heads. `lse` is what sdpa_forward wrote to
+    lse_out for the same q, k, scale and bias."""
+    op = "attention_map_avg"
+    _dev(op, q, k, lse, logit_bias, out)
+    if q.dim() != 2 or k.dim() != 2 or q.stride(1) != 1 or k.stride(1) != 1 or q.shape[1] != k.shape[1] or q.dtype != k.dtype:
+        _fail(op, "q and k must be 2-D (L, heads*head_dim) of one dtype, contiguous along columns")
+    Lq, Lk = q.shape[0], k.shape[0]
+    if lse.dtype != torch.float32 or lse.numel() != num_heads * Lq or not lse.is_contiguous():
+        _fail(op, "lse must be contiguous float32 (heads, Lq)")
+    if out is None:
+        out = torch.empty(Lq, Lk, dtype=torch.float32, device=q.device)
+    if out.dtype != torch.float32 or tuple(out.shape) != (Lq, Lk) or out.stride(1) != 1:
+        _fail(op, "out must be float32 (Lq, Lk)")
+    a = capi.MiAttentionMapArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, q)
+    a.q, a.k, a.lse, a.map = q.data_ptr(), k.data_ptr(), lse.data_ptr(), out.data_ptr()
+    a.num_heads, a.head_dim, a.q_len, a.kv_len = num_heads, q.shape[1] // num_heads, Lq, Lk
+    a.q_row_stride, a.k_row_stride, a.map_row_stride = q.stride(0), k.stride(0), out.stride(0)
+    a.scale = 0.0 if scale is None else float(scale)
+    if logit_bias is not None:
+        if logit_bias.dtype != torch.float32 or logit_bias.dim() != 2 or logit_bias.stride(1) != 1 or logit_bias.shape[0] != Lq - bias_q0:
+            _fail(op, "logit_bias must be float32 (Lq - bias_q0, cols)")
+        a.logit_bias, a.bias_q0, a.bias_cols, a.bias_row_stride = logit_bias.data_ptr(), bias_q0, logit_bias.shape[1], logit_bias.stride(0)
+    a.stream = _stream()
+    capi.check(capi.lib().mi_attention_map_avg(C.byref(a)), op)
+    return out
+
+
+def joint_attention_traced(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
+                           attn_avg: Optional[torch.Tensor] = None, Qr: Optional[torch.Tensor] = None,
+                           Kr: Optional[torch.Tensor] = None, txt_len: int = 0, image_text_bias: Optional[torch.Tensor] = None):
+    """dit::joint_attention_traced (src/dit/common.cpp:198-329) on the device: RoPE on Q and K into Qr / Kr, attention with
+    the optional image->text logit bias ((L - txt_len, txt_len) float32, added to the scaled scores of image rows against
+    text keys), and the head-averaged (L, L) float32 softmax map. Returns (out, attn_avg)."""
+    op = "joint_attention_traced"
+    _dev(op, Q, K, V, cos, sin, image_text_bias)
+    if Q.dim() != 2 or Q.shape[1] != head_dim * num_heads:
+        _fail(op, "D must equal head_dim * num_heads")
+    L = Q.shape[0]
+    if tuple(K.shape) != tuple(Q.shape) or tuple(V.shape) != tuple(Q.shape):
+        _fail(op, "Q/K/V must share shape (L, D)")
+    if image_text_bias is not None:
+        if txt_len < 0 or txt_len > L:
+            _fail(op, "txt_len out of range for bias")
+        if image_text_bias.dtype != torch.float32:
+            _fail(op, "image_text_bias must be FP32")
+        if tuple(image_text_bias.shape) != (L - txt_len, txt_len):
+            _fail(op, "image_text_bias must be (img_len, txt_len)")
+    Qr = rope_apply(Q, cos, sin, head_dim, num_heads, out=Qr)
+    Kr = rope_apply(K, cos, sin, head_dim, num_heads, out=Kr)
+    lse = torch.empty(num_heads, L, dtype=torch.float32, device=Q.device)
+    bias = image_text_bias if (image_text_bias is not None and txt_len > 0 and txt_len < L) else None
+    out = sdpa_forward(Qr, Kr, V, num_heads, out=out, logit_bias=bias, bias_q0=txt_len, lse_out=lse, op=op)
+    attn_avg = attention_map_avg(Qr, Kr, lse, num_heads, logit_bias=bias, bias_q0=txt_len, out=attn_avg)
+    return out, attn_avg
 
 
 def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num_kv_heads: int, d_mask,

@@ -12,6 +12,7 @@
  *                                          src/dit/qwenimage21_forward.cpp:584-585;
  *                                          src/triposplat/flow_model.cpp:374
  *   ReLU linear-attention core             src/dit/sana.cpp:470-586
+ *   dit::joint_attention_traced            src/dit/common.cpp:198-329 (bias + head-averaged map on device)
  *   bt::flash_attention_qkvo_forward,      src/unet_blocks.cpp:255-327; src/unet.cpp:470-480
  *   ..._q_with_kv_cached_forward, ..._project_kv
  *   bt::linear_forward_batched_fp16        include/brodiffusion/detail/compute.h:52-62
@@ -143,6 +144,15 @@ typedef struct mi_sdpa_args {
                                     K is rotated into it by one bandwidth-bound pass and attention reads the rotated copy
                                     (fastest form); afterwards it holds RoPE(K) like the Kr scratch of dit::joint_attention
                                     (src/dit/common.cpp:193). NULL: K is rotated tile by tile as it is loaded */
+    const float* logit_bias;     /* device FP32 or NULL: additive pre-softmax bias for query rows >= bias_q0 and keys
+                                    < bias_cols, element (row - bias_q0, key), added to the scaled score — the image->text
+                                    steering bias of dit::joint_attention_traced (src/dit/common.cpp:217-235, :279-281;
+                                    joint sequence [text ; image]: bias_q0 = bias_cols = txt_len). Batch 1 */
+    int32_t bias_q0, bias_cols;
+    int64_t bias_row_stride;     /* elements; 0 = bias_cols */
+    float* lse_out;              /* device FP32 [batch][num_heads][q_len] or NULL: receives per row the base-2 logarithm of the
+                                    softmax denominator in exponent units, lse = log2 sum_k 2^(score_k*scale*log2(e) + bias*log2(e))
+                                    (+inf for a row without visible keys); input of mi_attention_map_avg */
     void* split_scratch;         /* device, 16-byte aligned, or NULL: lets a launch whose last round of work groups would fill
                                     only part of the GPU cut the query tiles of that round along the key axis into equal
                                     pieces for all compute units (partial results in the scratch, merged by a second small
@@ -164,6 +174,29 @@ MI_API size_t mi_sdpa_split_scratch_bytes(const mi_sdpa_args* args);
 MI_API int mi_sdpa_set_kernel_choice(int32_t choice);
 /* 1 if (dtype, head_dim) has a compiled kernel, else 0. */
 MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);
+
+/* ── head-averaged attention map ───────────────────────────────────────────
+ * map[q][k] = (1/num_heads) * sum over heads of softmax_h(q, k), FP32 (q_len, kv_len): the trace artifact of
+ * dit::joint_attention_traced (src/dit/common.cpp:297, :308-312), which the reference computes in a host loop over
+ * downloaded tensors. q, k as given to mi_sdpa_forward (already rotated), unmasked attention, batch 1; `lse` is what
+ * that call wrote to lse_out with the same scale and bias. Every element is accumulated in one register over the
+ * heads and written once (no atomics). */
+typedef struct mi_attention_map_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* q;           /* (q_len, heads*head_dim) */
+    const void* k;           /* (kv_len, heads*head_dim) */
+    const float* lse;        /* [num_heads][q_len] */
+    float* map;              /* (q_len, kv_len) */
+    int32_t num_heads, head_dim, q_len, kv_len;
+    int64_t q_row_stride, k_row_stride, map_row_stride;
+    float scale;             /* <= 0: 1/sqrt(head_dim) */
+    const float* logit_bias;
+    int32_t bias_q0, bias_cols;
+    int64_t bias_row_stride;
+    void* stream;
+} mi_attention_map_args;
+MI_API int mi_attention_map_avg(const mi_attention_map_args* args);
 
 /* ── stand-alone RoPE ──────────────────────────────────────────────────────
  * Replaces bt::rope_apply(X,cos,sin,head_dim,num_heads,out) and

@@ -247,6 +247,32 @@ static void gpu_checks() {
         CHECK(within_bf16(e));
         CHECK(state.rows == Hl && state.cols == dl * dl + dl);
     }
+    {   // traced joint attention: output and head-averaged map against the checker's restatement of the host loop
+        const std::vector<int> axes = {16, 56, 56};
+        dit::RopeTables tabs = dit::build_axial_rope_tables(txt, hp, wp, d, axes);
+        std::vector<float> oc(static_cast<size_t>(L) * d / 2), os(oc.size());
+        orc_build_axial_rope_tables(txt, hp, wp, d, axes.data(), 3, 10000.0f, oc.data(), os.data());
+        std::vector<float> bias(static_cast<size_t>(L - txt) * txt);
+        orc_torch_randn_f32(7301, bias.size(), bias.data());
+        Tensor B = Tensor::from_host(bias.data(), L - txt, txt, Dtype::FP32), out, avg, Qr, Kr;
+        dit::joint_attention_traced(Q, K, V, tabs.cos, tabs.sin, d, H, out, avg, Qr, Kr, txt, &B);
+        std::vector<float> qr(q.size()), kr(k.size()), ref(q.size()), ref_avg(static_cast<size_t>(L) * L);
+        orc_rope_apply(q.data(), oc.data(), os.data(), L, H, d, 0, 1, qr.data());
+        orc_rope_apply(k.data(), oc.data(), os.data(), L, H, d, 0, 1, kr.data());
+        orc_sdpa(qr.data(), kr.data(), v.data(), L, L, H, d, -1.0, nullptr, nullptr, nullptr, nullptr, bias.data(), txt, txt, nullptr, 0,
+                 ref.data(), ref_avg.data(), 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("traced attention      rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        const std::vector<uint8_t> raw = avg.to_host_bytes();
+        const float* got = reinterpret_cast<const float*>(raw.data());
+        double worst = 0;
+        for (size_t i = 0; i < ref_avg.size(); ++i) worst = std::fmax(worst, std::fabs(static_cast<double>(got[i]) - ref_avg[i]));
+        std::printf("traced map            max_abs=%.3e\n", worst);
+        CHECK(avg.rows == L && avg.cols == L && worst <= 2e-5);
+        CHECK(throws_with([&] { Tensor b2 = Tensor::from_host(bias.data(), L - txt, txt - 1, Dtype::FP32);
+                                dit::joint_attention_traced(Q, K, V, tabs.cos, tabs.sin, d, H, out, avg, Qr, Kr, txt, &b2); }, "(img_len, txt_len)"));
+    }
     {   // headnorm + RoPE in one pass, with the prefix rows also written to a cache tensor
         const std::vector<int> axes = {16, 56, 56};
         dit::RopeTables tabs = dit::build_axial_rope_tables(txt, hp, wp, d, axes);

@@ -1,0 +1,98 @@
+"""Traced / steered joint attention on the device (dit::joint_attention_traced, src/dit/common.cpp:198-329): RoPE on
+Q and K, attention with the optional image->text logit bias, and the head-averaged softmax map. The reference does
+this in a host loop over downloaded tensors; the CPU checker restates that loop (orc_sdpa with bias and attn_avg).
+Output tolerance as for every attention call (helpers.TOL); the map is FP32 on both sides: probabilities are compared
+absolutely (<= 2e-5 on values <= 1; scores come from the same bf16 inputs with FP32 accumulation on both sides, the
+exponential on the GPU is the hardware exp2) and its rows must sum to 1."""
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import assert_close, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def tables(oracle, txt, hp, wp, d, axes):
+    cos, sin = oracle.build_axial_rope_tables(txt, hp, wp, d, axes)
+    return cos, sin, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+
+
+@pytest.mark.parametrize("dtype,H,d,txt,hp,wp,axes,with_bias", [
+    ("bf16", 4, 128, 37, 9, 11, (16, 56, 56), True),
+    ("bf16", 4, 128, 37, 9, 11, (16, 56, 56), False),
+    ("fp16", 3, 64, 64, 8, 8, (16, 24, 24), True),
+    ("bf16", 2, 72, 5, 20, 13, (8, 32, 32), True),        # 265 rows: ragged tiles on both axes
+])
+def test_traced_matches_checker(oracle, dtype, H, d, txt, hp, wp, axes, with_bias):
+    L = txt + hp * wp
+    q, k, v = (randn(9400 + i, (L, H * d), dtype) for i in range(3))
+    cos, sin, dcos, dsin = tables(oracle, txt, hp, wp, d, axes)
+    bias = (randn(9410, (L - txt, txt), "fp32") * 1.5).astype(np.float32) if with_bias else None
+    dbias = None if bias is None else torch.from_numpy(bias).cuda()
+    out, avg = bd.joint_attention_traced(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), dcos, dsin, d, H,
+                                         txt_len=txt, image_text_bias=dbias)
+    qr = oracle.rope_apply(q, cos, sin, H, d, round_to_dtype=dtype)
+    kr = oracle.rope_apply(k, cos, sin, H, d, round_to_dtype=dtype)
+    ref_o, ref_avg = oracle.sdpa(qr, kr, v, H, bias=bias, bias_q0=txt, return_attn_avg=True)
+    print(assert_close(ref_o, to_np(out), dtype, "traced output"))
+    got = to_np(avg)
+    assert got.shape == (L, L) and avg.dtype == torch.float32
+    assert np.abs(got - ref_avg).max() <= 2e-5, np.abs(got - ref_avg).max()
+    assert np.abs(got.sum(axis=1) - 1.0).max() <= 1e-4
+    if with_bias:
+        # the bias steers: without it the image rows put different mass on the text keys
+        _, avg0 = bd.joint_attention_traced(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), dcos, dsin, d, H)
+        assert np.abs(to_np(avg0)[txt:, :txt] - got[txt:, :txt]).max() > 1e-3
+        assert np.abs(to_np(avg0)[:txt] - got[:txt]).max() <= 1e-6          # text rows carry no bias
+
+
+def test_traced_equals_fused_path_without_bias(oracle):
+    """With no bias the traced output is the ordinary joint attention (same kernels up to the 128-row form)."""
+    dtype, H, d, txt, hp, wp = "bf16", 8, 128, 32, 16, 16
+    L = txt + hp * wp
+    q, k, v = (to_dev(randn(9500 + i, (L, H * d), dtype), dtype) for i in range(3))
+    _, _, dcos, dsin = tables(oracle, txt, hp, wp, d, (16, 56, 56))
+    out, avg = bd.joint_attention_traced(q, k, v, dcos, dsin, d, H)
+    bd.set_sdpa_kernel_choice(1)
+    try:
+        fused = bd.joint_attention(q, k, v, dcos, dsin, d, H, Kr=torch.empty_like(k))
+    finally:
+        bd.set_sdpa_kernel_choice(0)
+    assert (out.float() - fused.float()).abs().max().item() <= 2.0 ** -7
+    # a constant bias over all text keys of a row changes nothing only if it covers every key: here it covers the text
+    # keys alone, so it must move mass between text and image keys, by the closed form p_txt' = p_txt e^c / (p_txt e^c + 1 - p_txt)
+    c = 0.7
+    bias = torch.full((L - txt, txt), c, dtype=torch.float32, device="cuda")
+    _, avg_b = bd.joint_attention_traced(q, k, v, dcos, dsin, d, 1 * H, txt_len=txt, image_text_bias=bias)
+    # per head the closed form holds exactly; averaged over heads only the direction is fixed: text mass grows
+    assert (avg_b[txt:, :txt].sum(dim=1) > avg[txt:, :txt].sum(dim=1)).all()
+
+
+def test_single_head_bias_closed_form(oracle):
+    dtype, H, d, txt, hp, wp = "bf16", 1, 128, 40, 8, 8
+    L = txt + hp * wp
+    q, k, v = (to_dev(randn(9600 + i, (L, H * d), dtype), dtype) for i in range(3))
+    _, _, dcos, dsin = tables(oracle, txt, hp, wp, d, (16, 56, 56))
+    _, a0 = bd.joint_attention_traced(q, k, v, dcos, dsin, d, H)
+    c = -1.3
+    bias = torch.full((L - txt, txt), c, dtype=torch.float32, device="cuda")
+    _, a1 = bd.joint_attention_traced(q, k, v, dcos, dsin, d, H, txt_len=txt, image_text_bias=bias)
+    p = a0[txt:, :txt].sum(dim=1).double()
+    expect = p * np.exp(c) / (p * np.exp(c) + 1 - p)
+    assert (a1[txt:, :txt].sum(dim=1).double() - expect).abs().max().item() <= 1e-5
+
+
+def test_traced_errors():
+    z = lambda *s, dt=torch.bfloat16: torch.zeros(*s, device="cuda", dtype=dt)
+    q = z(16, 128)
+    cs = z(16, 64, dt=torch.float32)
+    with pytest.raises(RuntimeError, match=r"image_text_bias must be \(img_len, txt_len\)"):
+        bd.joint_attention_traced(q, q, q, cs, cs, 128, 1, txt_len=4, image_text_bias=z(12, 5, dt=torch.float32))
+    with pytest.raises(RuntimeError, match="image_text_bias must be FP32"):
+        bd.joint_attention_traced(q, q, q, cs, cs, 128, 1, txt_len=4, image_text_bias=z(12, 4))
+    with pytest.raises(RuntimeError, match="txt_len out of range"):
+        bd.joint_attention_traced(q, q, q, cs, cs, 128, 1, txt_len=40, image_text_bias=z(12, 4, dt=torch.float32))
+    with pytest.raises(RuntimeError, match="share shape"):
+        bd.joint_attention_traced(q, z(8, 128), q, cs, cs, 128, 1)
