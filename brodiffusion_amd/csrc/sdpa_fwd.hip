@@ -335,8 +335,157 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     write_output<T, D, kThreads4>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
 }
 
-// ───────────────────────── 8-wavefront ping-pong kernel ─────────────────────────
+// ───────────────────────── short key sequences (cross attention) ─────────────────────────
+// When all keys of a (batch, head) fit in LDS next to one query tile (cross attention to a text prompt: 77 to ~300
+// keys), the launch is pure overhead in the kernels above: every work group pays the prologue (Q staged, first K/V
+// tiles awaited) and the epilogue for a handful of key steps, and all work groups hit memory at the same moments.
+// Here a work group of 8 wavefronts loads the K and V of its (batch, head) ONCE, all tiles in flight together, and
+// then walks several 256-row query tiles: the Q rows of the next tile are already on their way (held in registers)
+// while the current tile is computed, the output of a tile drains while the next is computed, and the key loop has
+// no barrier at all (K and V never change), so the two wavefronts of a SIMD overlap their MFMA and softmax phases
+// freely. Unmasked calls (kv_valid_len allowed), no RoPE, no prefix.
 constexpr int kThreads8 = 512;
+constexpr int kShortMaxTiles = 5;   // 320 keys
+template <int D> constexpr int shortkv_lds_bytes(int n_kt) {
+    using G = HeadGeo<D>;
+    return 256 * G::O_STRIDE + n_kt * (G::K_BYTES + G::V_BYTES);
+}
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDev p, int n_kt, int n_strip, int strips_per_head) {
+    using G = HeadGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    constexpr int BM = 256;
+    constexpr int Q_BYTES = BM * G::O_STRIDE;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* const Qs = smem;
+    unsigned char* const Kall = smem + Q_BYTES;
+    unsigned char* const Vall = Kall + n_kt * G::K_BYTES;
+
+    const int logical = logical_block(p.n_blocks);
+    if (logical < 0) return;
+    const int bh = logical / strips_per_head;
+    const int strip = logical - bh * strips_per_head;
+    const int h = bh % p.H, b = bh / p.H;
+    const int hk = h / p.kv_group;
+
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+
+    // ── Q rows of a tile: fetched with full-row coalescing into registers, stored to LDS one tile later ──
+    constexpr int CPRK = G::DK / 8;
+    constexpr int NQ = (BM * CPRK + kThreads8 - 1) / kThreads8;
+    u32x4 qraw[NQ];
+    auto q_issue = [&](int q0) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = min(tid + kThreads8 * i, BM * CPRK - 1);
+            const int row = idx / CPRK, cc = min(idx - row * CPRK, G::CPR - 1);
+            qraw[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(min(q0 + row, p.Lq - 1)) * p.q_rs + cc * 8);
+        }
+    };
+    auto q_store = [&](int q0) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = tid + kThreads8 * i;
+            const int row = idx / CPRK, cc = idx - row * CPRK;
+            u32x4 v = qraw[i];
+            if (q0 + row >= p.Lq || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
+            if (idx < BM * CPRK) *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
+        }
+    };
+    const int qt_begin = strip * n_strip;
+    const int qt_end = min(qt_begin + n_strip, p.n_q_tiles);
+    q_issue(qt_begin * BM);
+
+    // ── all K and V tiles of this (batch, head): every load is issued before the first is stored ──
+    {
+        constexpr int NLD = (G::NCH + kThreads8 - 1) / kThreads8;
+        const unsigned char* const k_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D);
+        const unsigned char* const v_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D);
+        const unsigned k_rsb = static_cast<unsigned>(p.k_rs) * 2u, v_rsb = static_cast<unsigned>(p.v_rs) * 2u;
+        u32x4 kreg[kShortMaxTiles][NLD], vreg[kShortMaxTiles][NLD];
+#pragma unroll
+        for (int t = 0; t < kShortMaxTiles; ++t) {
+            if (t < n_kt) {
+                const int last = min(p.Lk - t * kBN, kBN) - 1;   // rows past the last key repeat it and are stored as zeros
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int idx = min(tid + kThreads8 * i, G::NCH - 1);
+                    const unsigned row = static_cast<unsigned>(t * kBN + min(idx / G::CPR, last));
+                    const unsigned cc = static_cast<unsigned>(idx % G::CPR);
+                    kreg[t][i] = *reinterpret_cast<const u32x4*>(k_base + (static_cast<unsigned long>(row) * k_rsb + cc * 16u));
+                    vreg[t][i] = *reinterpret_cast<const u32x4*>(v_base + (static_cast<unsigned long>(row) * v_rsb + cc * 16u));
+                }
+            }
+        }
+        zero_pads<D, kThreads8>(Kall, Vall, G::K_BYTES, G::V_BYTES, n_kt, tid);
+#pragma unroll
+        for (int t = 0; t < kShortMaxTiles; ++t) {
+            if (t < n_kt) {
+                const int nvalid = p.Lk - t * kBN;
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int idx = tid + kThreads8 * i;
+                    const int row = idx / G::CPR, cc = idx - row * G::CPR;
+                    if (idx < G::NCH) {
+                        const bool live = row < nvalid;
+                        *reinterpret_cast<u32x4*>(Kall + t * G::K_BYTES + row * G::K_STRIDE + cc * 16) = live ? kreg[t][i] : u32x4{0, 0, 0, 0};
+                        *reinterpret_cast<u32x4*>(Vall + t * G::V_BYTES + row * G::V_STRIDE + cc * 16) = live ? vreg[t][i] : u32x4{0, 0, 0, 0};
+                    }
+                }
+            }
+        }
+    }
+
+    const float cl2 = p.scale_log2;
+    const float lazy_raw = kLazyLog2 / cl2;
+    for (int qt = qt_begin; qt < qt_end; ++qt) {
+        const int q0 = qt * BM;
+        q_store(q0);
+        __syncthreads();   // Q tile (and, the first time, K and V) visible to all wavefronts
+        V8 qf[G::KC];
+        read_q_frags<T, D>(qf, Qs, wave * 32 + lq, lh);
+        __syncthreads();   // the staging area is free again
+        if (qt + 1 < qt_end) q_issue(q0 + BM);
+
+        const int qrow = q0 + wave * 32 + lq;
+        const bool qvalid = qrow < p.Lq;
+        int lo, hi;
+        row_interval(p, b, qrow, qvalid, lo, hi);
+        const WaveExtent we = wave_extent(lo, hi);
+        f32x16 oacc[G::VB];
+#pragma unroll
+        for (int vb = 0; vb < G::VB; ++vb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
+        SoftmaxState st;
+        for (int t = 0; t < n_kt; ++t) {
+            const int j0 = t * kBN;
+            if (j0 < we.hi_max && j0 + kBN > we.lo_min) {
+                const unsigned char* Ks = Kall + t * G::K_BYTES;
+                const unsigned char* Vs = Vall + t * G::V_BYTES;
+                f32x16 sacc[2];
+                V8 pf[4];
+                mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
+                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, p.Lk));
+                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, p.Lk), lh, nullptr);
+                mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
+            }
+        }
+        const float l_tot = exchange_sum(st.l);
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        stage_output<T, D>(Qs, wave * 32 + lq, lh, oacc, inv);
+        __syncthreads();
+        write_output<T, D, kThreads8>(Qs, o_base, p.o_rs, q0, p.Lq, BM, tid);
+        __syncthreads();   // staged rows are read before the next tile's Q overwrites them
+    }
+}
+
+// ───────────────────────── 8-wavefront ping-pong kernel ─────────────────────────
 template <int D> constexpr int lds_bytes_8() {
     using G = HeadGeo<D>;
     const int kv = 2 * (G::K_BYTES + G::V_BYTES);
@@ -1018,6 +1167,23 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     // ... and so do calls with a logit bias or a request for the softmax denominators
     const bool pingpong = D <= 128 && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr &&
                           (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
+    // short key sequences whose K and V fit in LDS next to a query tile: one work group walks several query tiles
+    const int n_kt = (p.Lk + kBN - 1) / kBN;
+    if (D <= 128 && choice == 0 && p.mask_mode == MI_MASK_NONE && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr &&
+        p.Lp == 0 && !rope_k && p.cos_q == nullptr && n_kt >= 1 && n_kt <= kShortMaxTiles && tiles256 >= n_cu &&
+        shortkv_lds_bytes<D>(n_kt) <= 160 * 1024) {
+        if constexpr (D <= 128) {
+            p.n_q_tiles = (p.Lq + 255) / 256;
+            const int n_strip = static_cast<int>(tiles256 / n_cu);   // query tiles per work group: about one work group per CU
+            const int strips_per_head = (p.n_q_tiles + n_strip - 1) / n_strip;
+            p.n_blocks = p.B * p.H * strips_per_head;
+            hipLaunchKernelGGL((sdpa_shortkv_kernel<T, D>), dim3(grid_blocks(p)), dim3(kThreads8), shortkv_lds_bytes<D>(n_kt), stream, p,
+                               n_kt, n_strip, strips_per_head);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail("sdpa_fwd launch: %s", hipGetErrorString(e));
+            return 0;
+        }
+    }
     if (pingpong) {
         p.n_q_tiles = (p.Lq + 255) / 256;
         p.n_blocks = static_cast<int>(tiles256);
