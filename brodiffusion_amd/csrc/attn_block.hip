@@ -85,6 +85,22 @@ int mi_linear_forward(const mi_linear_args* a) {
     return mi::launch_linear(b, 1, a->dtype, mi::resolve_stream(a->stream));
 }
 
+int mi_linear_geglu_forward(const mi_linear_args* a) {
+    mi::clear_error();
+    if (!a) return fail("mi_linear_geglu_forward: null args");
+    if (a->struct_size != sizeof(mi_linear_args))
+        return fail("mi_linear_geglu_forward: struct_size %u != %zu (header mismatch)", a->struct_size, sizeof(mi_linear_args));
+    if (a->rows < 0) return fail("mi_linear_geglu_forward: negative rows");
+    if (a->rows == 0) return 0;
+    mi::LinearBatch b;
+    std::memset(&b, 0, sizeof(b));
+    b.p[0] = mi::problem(a->x, a->w, a->bias, a->y, a->rows, a->out_features, a->in_features);
+    if (a->x_row_stride) b.p[0].ldx = a->x_row_stride;
+    if (a->w_row_stride) b.p[0].ldw = a->w_row_stride;
+    if (a->y_row_stride) b.p[0].ldy = a->y_row_stride;
+    return mi::launch_linear(b, 1, a->dtype, mi::resolve_stream(a->stream), true);
+}
+
 size_t mi_flash_attention_scratch_bytes(int32_t batch, int32_t q_len, int32_t kv_len, int32_t inner, int32_t with_kv) {
     if (batch <= 0 || q_len < 0 || kv_len < 0 || inner <= 0) return 0;
     const size_t q = mi::round_up(static_cast<size_t>(batch) * q_len * inner * 2);

@@ -116,6 +116,7 @@ struct LinearProblem {
 constexpr int kMaxLinearProblems = 3;
 struct LinearBatch { LinearProblem p[kMaxLinearProblems]; };
 // Validates and launches up to kMaxLinearProblems problems as one grid.
-int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t stream);
+// geglu: problem 0 has W (2 N, K) and bias (2 N), value half first; Y (M, N) = value * gelu_exact(gate).
+int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t stream, bool geglu = false);
 
 }  // namespace mi

@@ -45,7 +45,10 @@ constexpr int kRowBytes = kBK * 2 + 16;  // LDS row stride
 constexpr int kThreads = 256;
 
 // One 16-byte chunk column (tid % 8) and 32 rows per pass: ROWS / 32 loads per thread and tile.
-template <int ROWS>
+// GATED (the W tile of the GEGLU form): the tile's 32-row groups alternate between the value half and the gate half
+// of W — group 2j holds value features row0 + 32 j .., group 2j+1 the gate rows of the same features (n_rows further
+// down) — so that one wavefront's two 32-feature blocks are the value and the gate of the same outputs.
+template <int ROWS, bool GATED = false>
 __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
                                           int k0, int K, int tid) {
     const int kc = k0 + (tid & 7) * 8;
@@ -53,7 +56,9 @@ __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* bas
     const long col = k_ok ? kc : 0;
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
-        const int row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);  // rows past the end repeat the last one; never stored
+        int row;
+        if constexpr (GATED) row = min(row0 + (tid >> 3) + 32 * (i >> 1), n_rows - 1) + (i & 1) * n_rows;
+        else row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);  // rows past the end repeat the last one; never stored
         r[i] = *reinterpret_cast<const u32x4*>(base + (static_cast<long>(row) * ld + col) * 2);
     }
     if (!k_ok) {
@@ -68,18 +73,24 @@ __device__ __forceinline__ void store_tile(const u32x4 (&r)[ROWS / 32], char* ld
         *reinterpret_cast<u32x4*>(lds + ((tid >> 3) + 32 * i) * kRowBytes + (tid & 7) * 16) = r[i];
 }
 
-template <typename T, int BM, int BN>
+// GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
+// value * gelu_exact(gate) (diffusers' GEGLU with the erf form of GELU). A work group's 128 W-tile rows are 64 output
+// features times {value, gate}; each wavefront holds both accumulators of its 32 features, so the product of the two
+// halves never leaves registers and the (M, 2 N) intermediate does not exist.
+template <typename T, int BM, int BN, bool GEGLU = false>
 __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batch) {
     using M = Mma<T>;
     constexpr int TM = BM / 64, TN = BN / 64;  // 32 x 32 blocks per wavefront along tokens / features
+    static_assert(!GEGLU || TN == 2, "the GEGLU form pairs the two feature blocks of a wavefront");
+    constexpr int BN_OUT = GEGLU ? BN / 2 : BN;   // output features per tile
     constexpr int X_BYTES = BM * kRowBytes, W_BYTES = BN * kRowBytes;
     extern __shared__ __attribute__((aligned(16))) char lds[];  // [2][X tile ; W tile]
 
     const LinearProblem& p = batch.p[blockIdx.y];
-    const int tiles_n = (p.N + BN - 1) / BN;
+    const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
     const int tiles_m = (p.M + BM - 1) / BM;
     if (static_cast<int>(blockIdx.x) >= tiles_m * tiles_n) return;  // uniform: this problem has fewer tiles than the grid
-    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN_OUT;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, lh = lane >> 5;
@@ -97,7 +108,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
 
     u32x4 xr[BM / 32], wr[BN / 32];
     load_tile<BM>(xr, xg, p.ldx, m0, p.M, 0, p.K, tid);
-    load_tile<BN>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
+    load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
     store_tile<BM>(xr, lds, tid);
     store_tile<BN>(wr, lds + X_BYTES, tid);
     __syncthreads();
@@ -109,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
         const bool more = t + 1 < n_steps;
         if (more) {
             load_tile<BM>(xr, xg, p.ldx, m0, p.M, (t + 1) * kBK, p.K, tid);
-            load_tile<BN>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
+            load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
         }
         const char* xs = cur + (wm * TM * 32 + lq) * kRowBytes + lh * 16;
         const char* ws = cur + X_BYTES + (wn * TN * 32 + lq) * kRowBytes + lh * 16;
@@ -135,6 +146,35 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
     // acc[a][b][4g + i]: feature n0 + (wn*TN + a)*32 + 8g + 4*lh + i of token m0 + (wm*TM + b)*32 + lq
     char* yg = static_cast<char*>(p.y);
     const T* bias = static_cast<const T*>(p.bias);
+    if constexpr (GEGLU) {
+        // acc[0] = value, acc[1] = gate of features n0 + wn*32 + 8g + 4*lh + i
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = n0 + wn * 32 + 8 * g + 4 * lh;
+            if (n >= p.N) continue;
+            float bv[4] = {0.f, 0.f, 0.f, 0.f}, bg[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias) {
+                const typename M::v4 b4 = *reinterpret_cast<const typename M::v4*>(bias + n);
+                const typename M::v4 g4 = *reinterpret_cast<const typename M::v4*>(bias + p.N + n);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { bv[i] = static_cast<float>(b4[i]); bg[i] = static_cast<float>(g4[i]); }
+            }
+#pragma unroll
+            for (int b = 0; b < TM; ++b) {
+                const int m = m0 + (wm * TM + b) * 32 + lq;
+                if (m >= p.M) continue;
+                typename M::v4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float val = acc[0][b][4 * g + i] + bv[i];
+                    const float gate = acc[1][b][4 * g + i] + bg[i];
+                    o[i] = static_cast<T>(val * (0.5f * gate * (1.0f + erff(gate * 0.70710678118654752f))));
+                }
+                *reinterpret_cast<typename M::v4*>(yg + (static_cast<long>(m) * p.ldy + n) * 2) = o;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < TN; ++a) {
 #pragma unroll
@@ -160,16 +200,17 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
     }
 }
 
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, bool GEGLU = false>
 int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
+    constexpr int BN_OUT = GEGLU ? BN / 2 : BN;
     int max_tiles = 0;
     for (int i = 0; i < n_problems; ++i) {
         const LinearProblem& p = batch.p[i];
-        max_tiles = max(max_tiles, ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN));
+        max_tiles = max(max_tiles, ((p.M + BM - 1) / BM) * ((p.N + BN_OUT - 1) / BN_OUT));
     }
     constexpr size_t lds = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
     static_assert(lds <= 160 * 1024, "operand ring exceeds the LDS of a compute unit");
-    auto kern = linear_kernel<T, BM, BN>;
+    auto kern = linear_kernel<T, BM, BN, GEGLU>;
     if (lds > 64 * 1024) {
         static thread_local bool raised = false;
         if (!raised) {
@@ -183,7 +224,13 @@ int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
 }
 
 template <typename T>
-int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st) {
+int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool geglu) {
+    if (geglu) {
+        // 64-token tiles unless 128-token tiles alone fill the GPU twice over
+        const long big = static_cast<long>((batch.p[0].M + 127) / 128) * ((batch.p[0].N + 63) / 64);
+        if (big >= 2L * device_cu_count() && batch.p[0].K >= 1024) return launch_tiles<T, 128, 128, true>(batch, 1, st);
+        return launch_tiles<T, 64, 128, true>(batch, 1, st);
+    }
     // 128 x 128 tiles when they alone fill the GPU twice over and the contraction is long enough to pay for their
     // longer prologue, else 64 x 64 (more, smaller work groups: the projections of one attention block are small
     // problems; Q, K, V of 8192 x 320 x 320 in one launch: 15 us with 64 x 64 tiles, 22 us with 128 x 128)
@@ -199,7 +246,8 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st) {
 
 }  // namespace gemm
 
-int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t st) {
+int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t st, bool geglu) {
+    if (geglu && n_problems != 1) return fail("linear: the GEGLU form takes one problem per launch");
     if (n_problems < 1 || n_problems > kMaxLinearProblems) return fail("linear: %d problems in one launch (1..%d)", n_problems, kMaxLinearProblems);
     for (int i = 0; i < n_problems; ++i) {
         const LinearProblem& p = batch.p[i];
@@ -213,8 +261,8 @@ int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream
         if (al & 15u) return fail("linear: operands must be 16-byte aligned");
         if (static_cast<long>((p.M + 63) / 64) * ((p.N + 63) / 64) > 0x7fffffffL) return fail("linear: problem too large for one launch");
     }
-    if (dtype == MI_DTYPE_BF16) return gemm::launch_t<__bf16>(batch, n_problems, st);
-    if (dtype == MI_DTYPE_F16) return gemm::launch_t<_Float16>(batch, n_problems, st);
+    if (dtype == MI_DTYPE_BF16) return gemm::launch_t<__bf16>(batch, n_problems, st, geglu);
+    if (dtype == MI_DTYPE_F16) return gemm::launch_t<_Float16>(batch, n_problems, st, geglu);
     return fail("linear: dtype %d is neither MI_DTYPE_F16 nor MI_DTYPE_BF16", dtype);
 }
 

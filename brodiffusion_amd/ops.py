@@ -17,6 +17,8 @@ Names, argument order and error behaviour follow the brotensor operators the ref
                                                                              src/unet_blocks.cpp:311-317
     flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out, V_out)            src/unet.cpp:476-480
     linear_batched(W, bias, X, Y)                                            include/brodiffusion/detail/compute.h:52
+    fused_linear_geglu(X, W, b, Y), add_inplace_vec(Y, X), add_inplace_row_bias(Y, bias)
+                                                                             include/brodiffusion/fused_transformer.h:20-61
 
 Tensors are torch CUDA tensors (rows = tokens, cols = heads*head_dim), used for device memory
 and the current stream only; every computation is a call through the C ABI. Shape and dtype
@@ -303,6 +305,56 @@ def linear_batched(W, bias, X, Y: Optional[torch.Tensor] = None):
     a.rows, a.in_features, a.out_features = rows, W.shape[1], W.shape[0]
     a.stream = _stream()
     capi.check(capi.lib().mi_linear_forward(C.byref(a)), op)
+    return Y
+
+
+def fused_linear_geglu(X, W, b, Y: Optional[torch.Tensor] = None):
+    """Y = a * gelu_exact(g), [a | g] = X W^T + b with W (2*D_out, D_in), b (2*D_out): the fused FF1 + GEGLU of the
+    U-Net transformer block (brodiffusion::fused_linear_geglu, include/brodiffusion/fused_transformer.h:20-35)."""
+    op = "fused_linear_geglu"
+    _dev(op, X, W, b, Y)
+    if W.dim() != 2 or W.shape[0] % 2 != 0 or X.shape[-1] != W.shape[1]:
+        _fail(op, f"W must be (2*D_out, D_in) with D_in = {X.shape[-1]}, got {tuple(W.shape)}")
+    d_out = W.shape[0] // 2
+    _mat(op, W, "W", X.dtype)
+    _mat(op, X, "X", X.dtype)
+    rows = X.numel() // X.shape[-1]
+    if Y is None:
+        Y = torch.empty(*X.shape[:-1], d_out, dtype=X.dtype, device=X.device)
+    _mat(op, Y, "Y", X.dtype, cols=d_out)
+    if Y.numel() != rows * d_out:
+        _fail(op, "Y has the wrong number of rows")
+    a = capi.MiLinearArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, X)
+    a.x, a.w, a.y = X.data_ptr(), W.data_ptr(), Y.data_ptr()
+    a.bias = _bias(op, b, "b", X.dtype, W.shape[0])
+    a.rows, a.in_features, a.out_features = rows, W.shape[1], d_out
+    a.stream = _stream()
+    capi.check(capi.lib().mi_linear_geglu_forward(C.byref(a)), op)
+    return Y
+
+
+def add_inplace_vec(Y, X):
+    """Y += X, same shape and dtype (brodiffusion::add_inplace_vec, include/brodiffusion/fused_transformer.h:50-53)."""
+    op = "add_inplace_vec"
+    _dev(op, Y, X)
+    if tuple(Y.shape) != tuple(X.shape) or Y.dtype != X.dtype or not Y.is_contiguous() or not X.is_contiguous():
+        _fail(op, "Y and X must match in shape and dtype and be contiguous")
+    capi.check(capi.lib().mi_add_inplace(Y.data_ptr(), X.data_ptr(), Y.numel(), _dtype_code(op, Y), _stream()), op)
+    return Y
+
+
+def add_inplace_row_bias(Y, bias):
+    """Y[i, j] += bias[j]; bias holds Y's column count of values, any shape
+    (brodiffusion::add_inplace_row_bias, include/brodiffusion/fused_transformer.h:55-61)."""
+    op = "add_inplace_row_bias"
+    _dev(op, Y, bias)
+    if Y.dim() != 2 or Y.stride(1) != 1:
+        _fail(op, "Y must be 2-D, contiguous along columns")
+    if bias.dtype != Y.dtype or bias.numel() != Y.shape[1] or not bias.is_contiguous():
+        _fail(op, f"bias must hold {Y.shape[1]} values of Y's dtype")
+    capi.check(capi.lib().mi_add_row_bias(Y.data_ptr(), bias.data_ptr(), Y.shape[0], Y.shape[1], Y.stride(0), _dtype_code(op, Y), _stream()), op)
     return Y
 
 

@@ -321,6 +321,17 @@ typedef struct mi_linear_args {
     void* stream;
 } mi_linear_args;
 MI_API int mi_linear_forward(const mi_linear_args* args);
+/* Y (rows, out_features) = a * gelu_exact(g) with [a | g] = X W^T + bias, W (2*out_features, in_features) and bias
+ * (2*out_features): value half first, gate half second; gelu_exact(g) = 0.5 g (1 + erf(g / sqrt 2)). The fused FF1 +
+ * GEGLU of the U-Net transformer block, brodiffusion::fused_linear_geglu (include/brodiffusion/fused_transformer.h:20-35,
+ * src/fused_transformer.cu:56-68): the (rows, 2*out_features) intermediate never reaches memory. Same struct as
+ * mi_linear_forward. */
+MI_API int mi_linear_geglu_forward(const mi_linear_args* args);
+/* Y[i] += X[i] over n_elements of flat storage (brodiffusion::add_inplace_vec, fused_transformer.h:50-53) and
+ * Y[r][c] += bias[c] (brodiffusion::add_inplace_row_bias, fused_transformer.h:55-61). Any element count; 16-byte
+ * accesses when the addresses (and, for the bias form, cols and the row stride) allow. */
+MI_API int mi_add_inplace(void* y, const void* x, int64_t n_elements, int32_t dtype, void* stream);
+MI_API int mi_add_row_bias(void* y, const void* bias, int32_t rows, int32_t cols, int64_t y_row_stride, int32_t dtype, void* stream);
 
 /* ── attention with its projections ────────────────────────────────────────
  * The three operators the U-Net spatial transformer calls (src/unet_blocks.cpp:255-327,

@@ -73,6 +73,8 @@ _lib.orc_linear_attn_relu.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c
 _lib.orc_linear_attn_relu.restype = None
 _lib.orc_rms_norm.argtypes = [_f32p, _f32p, C.c_double, C.c_int, C.c_int, _f32p]
 _lib.orc_rms_norm.restype = None
+_lib.orc_geglu_exact.argtypes = [_f32p, C.c_int, C.c_int, _f32p]
+_lib.orc_geglu_exact.restype = None
 _lib.orc_linear.argtypes = [_f32p, _f32p, C.c_void_p, C.c_int, C.c_int, C.c_int, _f32p, C.c_int]
 _lib.orc_linear.restype = None
 _lib.orc_max_threads.restype = C.c_int
@@ -257,6 +259,15 @@ def headnorm_rope(x, gain, eps, cos, sin, num_heads, head_dim, round_to_dtype="f
     if cos is None:
         return round_to(y, round_to_dtype)
     return rope_apply(y, cos, sin, num_heads, head_dim, round_to_dtype=round_to_dtype)
+
+
+def geglu_exact(t):
+    """(rows, 2*d_out) -> (rows, d_out): value half times exact GELU of the gate half."""
+    t = _f32(t)
+    rows, two_d = t.shape
+    out = np.empty((rows, two_d // 2), dtype=np.float32)
+    _lib.orc_geglu_exact(t, rows, two_d // 2, out)
+    return out
 
 
 def linear(x, w, bias=None, n_threads=0):

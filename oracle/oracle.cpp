@@ -25,6 +25,8 @@
 //   orc_rms_norm               pinned: torch.nn.functional.rms_norm in float64, unit-RMS invariant, scale
 //                              invariance; eps placement (inside the square root) follows diffusers'
 //                              RMSNorm — brotensor's own is "parity unpinned"
+//   orc_geglu_exact            pinned: torch.nn.functional.gelu(approximate="none") in float64, gelu(0) = 0,
+//                              gelu(x) - gelu(-x) = x
 //   orc_linear                 pinned: numpy float64 matmul, identity weight, one-hot rows.
 //                              WHERE the fused projection operators round their intermediates
 //                              (Q, K, V, attention output to the tensor dtype) is "parity unpinned":
@@ -526,6 +528,19 @@ ORC_API void orc_linear(const float* x, const float* w, const float* bias, int M
             y[static_cast<size_t>(m) * N + n] = static_cast<float>(acc);
         }
     }
+}
+
+// ─── GEGLU ──────────────────────────────────────────────────────────────────
+// brotensor::geglu_exact_forward as brodiffusion::fused_linear_geglu states it
+// (include/brodiffusion/fused_transformer.h:20-29, src/fused_transformer.cu:66-68): t is (rows, 2*d_out),
+// value half a = t[:, :d_out], gate half g = t[:, d_out:], out = a * 0.5 g (1 + erf(g / sqrt 2)). Double arithmetic.
+ORC_API void orc_geglu_exact(const float* t, int rows, int d_out, float* out) {
+    for (int r = 0; r < rows; ++r)
+        for (int j = 0; j < d_out; ++j) {
+            const double a = t[static_cast<size_t>(r) * 2 * d_out + j];
+            const double g = t[static_cast<size_t>(r) * 2 * d_out + d_out + j];
+            out[static_cast<size_t>(r) * d_out + j] = static_cast<float>(a * 0.5 * g * (1.0 + std::erf(g * 0.70710678118654752440)));
+        }
 }
 
 ORC_API int orc_max_threads(void) {

@@ -1,0 +1,82 @@
+"""The SD1.5 transformer block's fused helpers (include/brodiffusion/fused_transformer.h:20-61): FF1 + exact GEGLU in
+one GEMM, Y += X, Y += row bias. Shapes and tolerances of the reference's own parity test come first
+(tests/test_fused_parity.cpp:172-200, :268-276: inputs uniform in [-1, 1] x scale rounded to fp16, fused against
+linear followed by geglu, relative 0.01 / absolute 0.008), then the real FF sizes against the CPU checker."""
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import TOL, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def uniform(seed, shape, scale, dtype, oracle, offset=0.0):
+    rng = np.random.default_rng(seed)
+    return oracle.round_to((rng.uniform(-1.0, 1.0, shape) * scale + offset).astype(np.float32), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("B,d_in,d_out", [(40, 64, 48), (128, 128, 96), (8192, 320, 1280), (2048, 640, 2560), (77, 1280, 5120), (1, 8, 8)])
+def test_fused_linear_geglu(oracle, dtype, B, d_in, d_out):
+    x = uniform(21, (B, d_in), 1.0, dtype, oracle)
+    w = uniform(22, (2 * d_out, d_in), 0.1, dtype, oracle)
+    b = uniform(23, (2 * d_out,), 0.2, dtype, oracle)
+    dx, dw, db = to_dev(x, dtype), to_dev(w, dtype), to_dev(b, dtype)
+    y = bd.fused_linear_geglu(dx, dw, db)
+    assert y.shape == (B, d_out)
+    ref = oracle.geglu_exact(oracle.linear(x, w, b))                      # exact: no intermediate rounding
+    err = np.abs(to_np(y) - ref)
+    assert err.max() <= 0.008 + 0.01 * np.abs(ref).max()                  # the reference's bound
+    unit = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    assert np.all(err <= unit * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)   # FP32 throughout, one rounding
+    # unfused composition on the device (what the reference compares against): linear, round, then geglu
+    t = bd.linear_batched(dw, db, dx)
+    unfused = oracle.geglu_exact(to_np(t))
+    assert np.abs(to_np(y) - unfused).max() <= 0.008 + 0.01 * np.abs(unfused).max()
+
+
+def test_geglu_halves_and_errors(oracle):
+    """Value half first, gate half second: a weight whose gate rows are zero and gate bias is large gives a * g."""
+    dtype, B, d_in, d_out = "fp16", 64, 64, 64
+    x = uniform(31, (B, d_in), 1.0, dtype, oracle)
+    w = np.zeros((2 * d_out, d_in), np.float32)
+    w[:d_out] = uniform(32, (d_out, d_in), 0.1, dtype, oracle)
+    b = np.zeros(2 * d_out, np.float32)
+    b[d_out:] = 8.0                                                        # gelu(8) = 8 to fp16 precision
+    y = bd.fused_linear_geglu(to_dev(x, dtype), to_dev(w, dtype), to_dev(b, dtype))
+    ref = oracle.round_to(oracle.linear(x, w[:d_out]) * np.float32(8.0), dtype)
+    assert np.abs(to_np(y) - ref).max() <= 2.0 ** -10 * np.abs(ref).max()
+    z = lambda *s: torch.zeros(*s, device="cuda", dtype=torch.float16)
+    with pytest.raises(RuntimeError, match=r"W must be \(2\*D_out, D_in\)"):
+        bd.fused_linear_geglu(z(4, 64), z(63, 64), z(63))
+    with pytest.raises(RuntimeError, match="b must be"):
+        bd.fused_linear_geglu(z(4, 64), z(64, 64), z(32))
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("rows,cols", [(10, 37), (64, 64), (8192, 320), (3, 1)])
+def test_add_inplace_vec(oracle, dtype, rows, cols):
+    y0 = uniform(31, (rows, cols), 1.0, dtype, oracle)
+    x = uniform(32, (rows, cols), 1.0, dtype, oracle)
+    y = to_dev(y0, dtype)
+    bd.add_inplace_vec(y, to_dev(x, dtype))
+    assert np.array_equal(to_np(y), oracle.round_to(y0 + x, dtype))        # one FP32 add, one rounding
+    # an unaligned view (offset by one element) takes the scalar path and gives the same values
+    buf = torch.zeros(rows * cols + 1, device="cuda", dtype=y.dtype)
+    buf[1:] = to_dev(y0, dtype).reshape(-1)
+    bd.add_inplace_vec(buf[1:], to_dev(x, dtype).reshape(-1))
+    assert torch.equal(buf[1:].reshape(rows, cols), y) and buf[0] == 0
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("rows,cols", [(13, 29), (48, 80), (8192, 320)])
+def test_add_inplace_row_bias(oracle, dtype, rows, cols):
+    y0 = uniform(41, (rows, cols), 1.0, dtype, oracle)
+    b = uniform(42, (cols,), 0.5, dtype, oracle)
+    y = to_dev(y0, dtype)
+    bd.add_inplace_row_bias(y, to_dev(b, dtype).reshape(cols, 1))          # (cols, 1) and (1, cols) both accepted
+    assert np.array_equal(to_np(y), oracle.round_to(y0 + b[None, :], dtype))
+    with pytest.raises(RuntimeError, match="bias must hold"):
+        bd.add_inplace_row_bias(y, to_dev(b, dtype)[:-1])

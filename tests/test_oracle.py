@@ -454,3 +454,17 @@ def test_headnorm_rope_is_norm_then_rotation(oracle):
             by_hand[l, h * d + 1:(h + 1) * d:2] = y[0::2] * sin[l] + y[1::2] * cos[l]
     assert np.allclose(got, by_hand, rtol=1e-5, atol=1e-6)
     assert np.allclose(oracle.headnorm_rope(x, g, 1e-6, None, None, H, d), oracle.rms_norm(x.reshape(L * H, d), g, 1e-6).reshape(L, H * d))
+
+
+def test_geglu_exact_vs_torch_float64(oracle):
+    rng = np.random.default_rng(21)
+    t = (rng.standard_normal((13, 2 * 24)) * 2).astype(np.float32)
+    td = torch.from_numpy(t).double()
+    ref = (td[:, :24] * torch.nn.functional.gelu(td[:, 24:], approximate="none")).numpy()
+    assert np.allclose(oracle.geglu_exact(t), ref, rtol=1e-6, atol=1e-7)
+    # gelu(0) = 0 and gelu(x) - gelu(-x) = x, seen through unit values
+    g = np.array([[1.0, 1.0, 1.0, 0.0, 1.7, -1.7]], np.float32)
+    out = oracle.geglu_exact(g)
+    assert out[0, 0] == 0.0 and abs((out[0, 1] - out[0, 2]) - 1.7) < 1e-6
+    # the value half is the first half: swapping the halves changes the result
+    assert not np.allclose(oracle.geglu_exact(t), oracle.geglu_exact(np.concatenate([t[:, 24:], t[:, :24]], axis=1)))
