@@ -104,6 +104,10 @@ def all_configs(torch, bd):
     yl = torch.empty(4608, 3072, dtype=torch.bfloat16, device="cuda")
     sdpa_entry("linear_4608x3072x3072_bf16", 2 * 4608 * 3072 * 3072, lambda: bd.linear_batched(wl, None, xl, yl), "bf16")
     del xl, wl, yl
+    # FF1 + exact GEGLU of the same block: 8192 tokens, 320 -> 2 x 1280
+    wg_, bg_ = rnd(2560, 320, dt=torch.float16) / 320 ** 0.5, rnd(2560, dt=torch.float16)
+    yg_ = torch.empty(8192, 1280, dtype=torch.float16, device="cuda")
+    sdpa_entry("sd15_unet_block_ff1_geglu_8192x320x2560_fp16", 2 * 8192 * 2560 * 320, lambda: bd.fused_linear_geglu(x2, wg_, bg_, yg_), "fp16")
     q, k, v = (rnd(2, 4096, 1152) for _ in range(3))
     sdpa_entry("cfg2a_pixart_selfattn_d72_bf16", 4 * 2 * 16 * 4096 * 4096 * 72, lambda: bd.flash_attention_forward(q, k, v, None, 16, False), "bf16")
     kc, vc = rnd(2, 300, 1152), rnd(2, 300, 1152)

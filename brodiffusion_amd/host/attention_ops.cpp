@@ -258,6 +258,36 @@ void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tenso
 
 }  // namespace bt
 
+void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y) {
+    const char* op = "fused_linear_geglu";
+    need_gpu(op, X); need_gpu(op, W); need_gpu(op, b);
+    if (W.rows % 2 != 0 || W.cols != X.cols || W.dtype != X.dtype) fail(std::string(op) + ": W must be (2*D_out, D_in) of X's dtype");
+    const int d_out = W.rows / 2;
+    if (b.dtype != X.dtype || b.size() != static_cast<std::size_t>(W.rows)) fail(std::string(op) + ": b must hold 2*D_out values of X's dtype");
+    if (Y.data == nullptr || Y.rows != X.rows || Y.cols != d_out || Y.dtype != X.dtype) Y.resize(X.rows, d_out, X.dtype, X.device);
+    mi_linear_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, X.dtype);
+    a.x = X.data; a.w = W.data; a.bias = b.data; a.y = Y.data;
+    a.rows = X.rows; a.in_features = X.cols; a.out_features = d_out;
+    check(op, mi_linear_geglu_forward(&a));
+}
+
+void add_inplace_vec(Tensor& Y, const Tensor& X) {
+    const char* op = "add_inplace_vec";
+    need_gpu(op, Y); need_gpu(op, X);
+    if (Y.rows != X.rows || Y.cols != X.cols || Y.dtype != X.dtype) fail(std::string(op) + ": Y and X must match in shape and dtype");
+    check(op, mi_add_inplace(Y.data, X.data, static_cast<int64_t>(Y.size()), dtype_code(op, Y.dtype), nullptr));
+}
+
+void add_inplace_row_bias(Tensor& Y, const Tensor& bias) {
+    const char* op = "add_inplace_row_bias";
+    need_gpu(op, Y); need_gpu(op, bias);
+    if (bias.dtype != Y.dtype || bias.size() != static_cast<std::size_t>(Y.cols)) fail(std::string(op) + ": bias must hold Y.cols values of Y's dtype");
+    check(op, mi_add_row_bias(Y.data, bias.data, Y.rows, Y.cols, 0, dtype_code(op, Y.dtype), nullptr));
+}
+
 namespace dit {
 
 RopeTables build_axial_rope_tables(int txt_len, int hp, int wp, int head_dim, const std::vector<int>& axes, float theta) {

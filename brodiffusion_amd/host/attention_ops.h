@@ -55,6 +55,14 @@ void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tenso
 
 }  // namespace bt
 
+// The fused helpers of the SD1.5 transformer block, names and argument order of include/brodiffusion/fused_transformer.h:
+//   fused_linear_geglu   Y(B, D_out) = a * gelu_exact(g), [a | g] = X W^T + b, W (2*D_out, D_in), b 2*D_out values  (:20-35)
+//   add_inplace_vec      Y += X, same shape                                                                        (:50-53)
+//   add_inplace_row_bias Y[i][j] += bias[j], bias holds Y.cols values in any shape                                  (:55-61)
+void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y);
+void add_inplace_vec(Tensor& Y, const Tensor& X);
+void add_inplace_row_bias(Tensor& Y, const Tensor& bias);
+
 namespace dit {
 
 struct RopeTables {

@@ -29,6 +29,7 @@ void orc_rows_block_causal(int Lq, int Lk, int q_offset, const int* seg_q_end, c
 void orc_linear_attn_relu(const float* q, const float* k, const float* v, int N, int H, int d, float eps, float* out,
                           float* S_out, float* z_out, int n_threads);
 void orc_rms_norm(const float* x, const float* gain, double eps, int rows, int cols, float* out);
+void orc_geglu_exact(const float* t, int rows, int d_out, float* out);
 void orc_linear(const float* x, const float* w, const float* bias, int M, int N, int K, float* y, int n_threads);
 }
 
@@ -335,6 +336,36 @@ static void gpu_checks() {
         CHECK(within_bf16(compare(lin(x, wo, bo.data(), Lx, C, C, false), download_bf16(Y))));
         CHECK(throws_with([&] { bt::flash_attention_qkvo_forward(X, &Ctx, Wq, nullptr, Wq, nullptr, Wv, nullptr, Wo, &Bo, nullptr, Hh, false, out); }, "Wk is (320, 320)"));
         CHECK(throws_with([&] { bt::flash_attention_qkvo_forward(X, nullptr, Wq, nullptr, Wq, nullptr, Wq, nullptr, Wo, &Bo, nullptr, 7, false, out); }, "does not divide"));
+    }
+    {   // the transformer block's fused helpers on the reference's own test shapes (tests/test_fused_parity.cpp:268-276)
+        const int B = 40, d_in = 64, d_out = 48;
+        std::vector<float> x = randn_bf16(7401, static_cast<size_t>(B) * d_in), w = randn_bf16(7402, static_cast<size_t>(2) * d_out * d_in),
+                           b = randn_bf16(7403, 2 * d_out);
+        for (float& e : w) e *= 0.1f;
+        orc_round_bf16(w.data(), w.size());
+        Tensor X = upload_bf16(x, B, d_in), W = upload_bf16(w, 2 * d_out, d_in), Bv = upload_bf16(b, 2 * d_out, 1), Y;
+        fused_linear_geglu(X, W, Bv, Y);
+        std::vector<float> t(static_cast<size_t>(B) * 2 * d_out), ref(static_cast<size_t>(B) * d_out);
+        orc_linear(x.data(), w.data(), b.data(), B, 2 * d_out, d_in, t.data(), 0);
+        orc_geglu_exact(t.data(), B, d_out, ref.data());
+        const Err e = compare(ref, download_bf16(Y));
+        std::printf("fused_linear_geglu    rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(Y.rows == B && Y.cols == d_out && e.rel_l2 <= 5e-3);
+        // Y += X on 10 x 37 and Y += row bias on 13 x 29: exact (one FP32 add, one rounding)
+        std::vector<float> y0 = randn_bf16(7404, 370), xa = randn_bf16(7405, 370), want(370);
+        for (int i = 0; i < 370; ++i) want[i] = y0[i] + xa[i];
+        orc_round_bf16(want.data(), want.size());
+        Tensor Ya = upload_bf16(y0, 10, 37), Xa = upload_bf16(xa, 10, 37);
+        add_inplace_vec(Ya, Xa);
+        CHECK(download_bf16(Ya) == want);
+        std::vector<float> y1 = randn_bf16(7406, 13 * 29), rb = randn_bf16(7407, 29), want1(13 * 29);
+        for (int i = 0; i < 13 * 29; ++i) want1[i] = y1[i] + rb[i % 29];
+        orc_round_bf16(want1.data(), want1.size());
+        Tensor Yb = upload_bf16(y1, 13, 29), Rb = upload_bf16(rb, 29, 1);
+        add_inplace_row_bias(Yb, Rb);
+        CHECK(download_bf16(Yb) == want1);
+        CHECK(throws_with([&] { add_inplace_vec(Ya, Xa.row_view(0, 5)); }, "must match in shape"));
+        CHECK(throws_with([&] { add_inplace_row_bias(Yb, Xa); }, "bias must hold"));
     }
     {   // GPU-side error path: unsupported head_dim surfaces the C ABI's message
         Tensor out;
