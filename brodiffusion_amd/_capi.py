@@ -122,7 +122,7 @@ class MiLinearArgs(C.Structure):
         ("x", C.c_void_p), ("w", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p),
         ("rows", C.c_int32), ("in_features", C.c_int32), ("out_features", C.c_int32),
         ("x_row_stride", C.c_int64), ("w_row_stride", C.c_int64), ("y_row_stride", C.c_int64),
-        ("stream", C.c_void_p),
+        ("w_scales", C.c_void_p), ("stream", C.c_void_p),
     ]
 
 
@@ -137,7 +137,9 @@ class MiAttnBlockArgs(C.Structure):
         ("channels", C.c_int32), ("ctx_channels", C.c_int32), ("inner", C.c_int32), ("out_channels", C.c_int32),
         ("num_heads", C.c_int32), ("causal", C.c_int32),
         ("key_mask", C.c_void_p), ("key_mask_batch_stride", C.c_int64),
-        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("stream", C.c_void_p),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t),
+        ("wq_scales", C.c_void_p), ("wk_scales", C.c_void_p), ("wv_scales", C.c_void_p), ("wo_scales", C.c_void_p),
+        ("stream", C.c_void_p),
     ]
 
 

@@ -40,9 +40,10 @@ int check_common(const mi_attn_block_args* a, const char* op, BlockDims& d, bool
     return 0;
 }
 
-LinearProblem problem(const void* x, const void* w, const void* bias, void* y, long M, int N, int K) {
+LinearProblem problem(const void* x, const void* w, const void* bias, void* y, long M, int N, int K, const float* w_scale = nullptr) {
     LinearProblem p;
     p.x = x; p.w = w; p.bias = bias; p.y = y;
+    p.w_scale = w_scale;
     p.M = static_cast<int>(M); p.N = N; p.K = K;
     p.ldx = K; p.ldw = K; p.ldy = N;
     return p;
@@ -78,7 +79,7 @@ int mi_linear_forward(const mi_linear_args* a) {
     if (a->rows == 0) return 0;
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(a->x, a->w, a->bias, a->y, a->rows, a->out_features, a->in_features);
+    b.p[0] = mi::problem(a->x, a->w, a->bias, a->y, a->rows, a->out_features, a->in_features, a->w_scales);
     if (a->x_row_stride) b.p[0].ldx = a->x_row_stride;
     if (a->w_row_stride) b.p[0].ldw = a->w_row_stride;
     if (a->y_row_stride) b.p[0].ldy = a->y_row_stride;
@@ -91,6 +92,7 @@ int mi_linear_geglu_forward(const mi_linear_args* a) {
     if (a->struct_size != sizeof(mi_linear_args))
         return fail("mi_linear_geglu_forward: struct_size %u != %zu (header mismatch)", a->struct_size, sizeof(mi_linear_args));
     if (a->rows < 0) return fail("mi_linear_geglu_forward: negative rows");
+    if (a->w_scales) return fail("mi_linear_geglu_forward: there is no INT8-weight form (the reference does not fuse it either)");
     if (a->rows == 0) return 0;
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
@@ -117,8 +119,8 @@ int mi_flash_attention_project_kv(const mi_attn_block_args* a) {
     if (!a->ctx || !a->wk || !a->wv || !a->k || !a->v) return fail("%s: ctx, wk, wv, k and v must not be null", op);
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(a->ctx, a->wk, a->bk, a->k, d.kv_rows, a->inner, a->ctx_channels);
-    b.p[1] = mi::problem(a->ctx, a->wv, a->bv, a->v, d.kv_rows, a->inner, a->ctx_channels);
+    b.p[0] = mi::problem(a->ctx, a->wk, a->bk, a->k, d.kv_rows, a->inner, a->ctx_channels, a->wk_scales);
+    b.p[1] = mi::problem(a->ctx, a->wv, a->bv, a->v, d.kv_rows, a->inner, a->ctx_channels, a->wv_scales);
     return mi::launch_linear(b, 2, a->dtype, mi::resolve_stream(a->stream));
 }
 
@@ -144,17 +146,17 @@ int mi_flash_attention_qkvo_forward(const mi_attn_block_args* a) {
 
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(a->x, a->wq, a->bq, sq, d.q_rows, a->inner, a->channels);
+    b.p[0] = mi::problem(a->x, a->wq, a->bq, sq, d.q_rows, a->inner, a->channels, a->wq_scales);
     int n = 1;
     if (d.kv_rows > 0) {
-        b.p[1] = mi::problem(src, a->wk, a->bk, sk, d.kv_rows, a->inner, kv_channels);
-        b.p[2] = mi::problem(src, a->wv, a->bv, sv, d.kv_rows, a->inner, kv_channels);
+        b.p[1] = mi::problem(src, a->wk, a->bk, sk, d.kv_rows, a->inner, kv_channels, a->wk_scales);
+        b.p[2] = mi::problem(src, a->wv, a->bv, sv, d.kv_rows, a->inner, kv_channels, a->wv_scales);
         n = 3;
     }
     if (mi::launch_linear(b, n, a->dtype, st) != 0) return -1;
     if (mi::attend(a, d, sq, sk, sv, sa, kv_len) != 0) return -1;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(sa, a->wo, a->bo, a->out, d.q_rows, a->out_channels, a->inner);
+    b.p[0] = mi::problem(sa, a->wo, a->bo, a->out, d.q_rows, a->out_channels, a->inner, a->wo_scales);
     return mi::launch_linear(b, 1, a->dtype, st);
 }
 
@@ -175,11 +177,11 @@ int mi_flash_attention_q_with_kv_cached_forward(const mi_attn_block_args* a) {
 
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(a->x, a->wq, a->bq, sq, d.q_rows, a->inner, a->channels);
+    b.p[0] = mi::problem(a->x, a->wq, a->bq, sq, d.q_rows, a->inner, a->channels, a->wq_scales);
     if (mi::launch_linear(b, 1, a->dtype, st) != 0) return -1;
     if (mi::attend(a, d, sq, a->k, a->v, sa, a->kv_len) != 0) return -1;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(sa, a->wo, a->bo, a->out, d.q_rows, a->out_channels, a->inner);
+    b.p[0] = mi::problem(sa, a->wo, a->bo, a->out, d.q_rows, a->out_channels, a->inner, a->wo_scales);
     return mi::launch_linear(b, 1, a->dtype, st);
 }
 

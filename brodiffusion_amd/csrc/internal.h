@@ -110,6 +110,7 @@ int launch_attention_map(const MapDev& p, int dtype, int head_dim, hipStream_t s
 // One Y = X W^T + bias problem: X (M, K), W (N, K), Y (M, N), bias (N) or null; strides in elements.
 struct LinearProblem {
     const void* x; const void* w; const void* bias; void* y;
+    const float* w_scale;   // non-null: w is INT8 (N, K) with one FP32 scale per row, Y = (X Wq^T) * scale + bias
     int M, N, K;
     long ldx, ldw, ldy;
 };

@@ -66,6 +66,32 @@ __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* bas
         for (int i = 0; i < ROWS / 32; ++i) r[i] = u32x4{0u, 0u, 0u, 0u};
     }
 }
+// INT8 weight tile: the same 8 contraction elements per thread and row are 8 bytes in memory; they are widened to T
+// (exactly: |w| <= 128) on their way to LDS, the per-row scale is applied to the accumulator in the epilogue.
+template <typename T, int ROWS>
+__device__ __forceinline__ void load_tile_int8(u32x4 (&r)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
+                                               int k0, int K, int tid) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    typedef signed char c8 __attribute__((ext_vector_type(8)));
+    const int kc = k0 + (tid & 7) * 8;
+    const bool k_ok = kc < K;
+    const long col = k_ok ? kc : 0;
+    u32x2 raw[ROWS / 32];
+#pragma unroll
+    for (int i = 0; i < ROWS / 32; ++i) {
+        const int row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);
+        raw[i] = *reinterpret_cast<const u32x2*>(base + static_cast<long>(row) * ld + col);
+    }
+#pragma unroll
+    for (int i = 0; i < ROWS / 32; ++i) {
+        const c8 q = __builtin_bit_cast(c8, raw[i]);
+        t8 w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w[e] = static_cast<T>(static_cast<float>(q[e]));
+        r[i] = k_ok ? __builtin_bit_cast(u32x4, w) : u32x4{0u, 0u, 0u, 0u};
+    }
+}
+
 template <int ROWS>
 __device__ __forceinline__ void store_tile(const u32x4 (&r)[ROWS / 32], char* lds, int tid) {
 #pragma unroll
@@ -77,11 +103,13 @@ __device__ __forceinline__ void store_tile(const u32x4 (&r)[ROWS / 32], char* ld
 // value * gelu_exact(gate) (diffusers' GEGLU with the erf form of GELU). A work group's 128 W-tile rows are 64 output
 // features times {value, gate}; each wavefront holds both accumulators of its 32 features, so the product of the two
 // halves never leaves registers and the (M, 2 N) intermediate does not exist.
-template <typename T, int BM, int BN, bool GEGLU = false>
+// W8: W is INT8 (N, K) with one FP32 scale per row (LinearProblem::w_scale): Y = (X Wq^T) * scale + bias.
+template <typename T, int BM, int BN, bool GEGLU = false, bool W8 = false>
 __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batch) {
     using M = Mma<T>;
     constexpr int TM = BM / 64, TN = BN / 64;  // 32 x 32 blocks per wavefront along tokens / features
     static_assert(!GEGLU || TN == 2, "the GEGLU form pairs the two feature blocks of a wavefront");
+    static_assert(!(GEGLU && W8), "no INT8-weight GEGLU form");
     constexpr int BN_OUT = GEGLU ? BN / 2 : BN;   // output features per tile
     constexpr int X_BYTES = BM * kRowBytes, W_BYTES = BN * kRowBytes;
     extern __shared__ __attribute__((aligned(16))) char lds[];  // [2][X tile ; W tile]
@@ -108,7 +136,8 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
 
     u32x4 xr[BM / 32], wr[BN / 32];
     load_tile<BM>(xr, xg, p.ldx, m0, p.M, 0, p.K, tid);
-    load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
+    if constexpr (W8) load_tile_int8<T, BN>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
+    else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
     store_tile<BM>(xr, lds, tid);
     store_tile<BN>(wr, lds + X_BYTES, tid);
     __syncthreads();
@@ -120,7 +149,8 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
         const bool more = t + 1 < n_steps;
         if (more) {
             load_tile<BM>(xr, xg, p.ldx, m0, p.M, (t + 1) * kBK, p.K, tid);
-            load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
+            if constexpr (W8) load_tile_int8<T, BN>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
+            else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
         }
         const char* xs = cur + (wm * TM * 32 + lq) * kRowBytes + lh * 16;
         const char* ws = cur + X_BYTES + (wn * TN * 32 + lq) * kRowBytes + lh * 16;
@@ -187,20 +217,28 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
 #pragma unroll
                 for (int i = 0; i < 4; ++i) bv[i] = static_cast<float>(b4[i]);
             }
+            float sc[4] = {1.f, 1.f, 1.f, 1.f};
+            if constexpr (W8) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[i] = p.w_scale[n + i];
+            }
 #pragma unroll
             for (int b = 0; b < TM; ++b) {
                 const int m = m0 + (wm * TM + b) * 32 + lq;
                 if (m >= p.M) continue;
                 typename M::v4 o;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] = static_cast<T>(acc[a][b][4 * g + i] + bv[i]);
+                for (int i = 0; i < 4; ++i) {
+                    if constexpr (W8) o[i] = static_cast<T>(__builtin_fmaf(acc[a][b][4 * g + i], sc[i], bv[i]));
+                    else o[i] = static_cast<T>(acc[a][b][4 * g + i] + bv[i]);
+                }
                 *reinterpret_cast<typename M::v4*>(yg + (static_cast<long>(m) * p.ldy + n) * 2) = o;
             }
         }
     }
 }
 
-template <typename T, int BM, int BN, bool GEGLU = false>
+template <typename T, int BM, int BN, bool GEGLU = false, bool W8 = false>
 int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
     constexpr int BN_OUT = GEGLU ? BN / 2 : BN;
     int max_tiles = 0;
@@ -210,7 +248,7 @@ int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
     }
     constexpr size_t lds = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
     static_assert(lds <= 160 * 1024, "operand ring exceeds the LDS of a compute unit");
-    auto kern = linear_kernel<T, BM, BN, GEGLU>;
+    auto kern = linear_kernel<T, BM, BN, GEGLU, W8>;
     if (lds > 64 * 1024) {
         static thread_local bool raised = false;
         if (!raised) {
@@ -240,8 +278,10 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool gegl
         big += static_cast<long>((batch.p[i].M + 127) / 128) * ((batch.p[i].N + 127) / 128);
         min_k = min(min_k, batch.p[i].K);
     }
-    if (big >= 2L * device_cu_count() && min_k >= 1024) return launch_tiles<T, 128, 128>(batch, n_problems, st);
-    return launch_tiles<T, 64, 64>(batch, n_problems, st);
+    const bool w8 = batch.p[0].w_scale != nullptr;
+    if (big >= 2L * device_cu_count() && min_k >= 1024)
+        return w8 ? launch_tiles<T, 128, 128, false, true>(batch, n_problems, st) : launch_tiles<T, 128, 128>(batch, n_problems, st);
+    return w8 ? launch_tiles<T, 64, 64, false, true>(batch, n_problems, st) : launch_tiles<T, 64, 64>(batch, n_problems, st);
 }
 
 }  // namespace gemm
@@ -253,6 +293,9 @@ int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream
         const LinearProblem& p = batch.p[i];
         if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("linear: empty problem %d (%d x %d x %d)", i, p.M, p.N, p.K);
         if (p.N % 8 || p.K % 8) return fail("linear: in_features %d and out_features %d must be multiples of 8", p.K, p.N);
+        if ((p.w_scale != nullptr) != (batch.p[0].w_scale != nullptr)) return fail("linear: INT8 and 16-bit weights cannot share a launch");
+        if (p.w_scale && geglu) return fail("linear: there is no INT8-weight GEGLU form");
+        if (reinterpret_cast<uintptr_t>(p.w_scale) & 3u) return fail("linear: weight scales must be 4-byte aligned");
         if (p.ldx % 8 || p.ldw % 8 || p.ldy % 8) return fail("linear: row strides must be multiples of 8 elements");
         if (p.ldx < p.K || p.ldw < p.K || p.ldy < p.N) return fail("linear: a row stride is smaller than the row");
         const uintptr_t al = reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.w) |

@@ -152,12 +152,22 @@ const void* bias_ptr(const char* op, const Tensor* b, const char* name, Dtype dt
     if (b->dtype != dt || b->size() != static_cast<std::size_t>(n)) fail(std::string(op) + ": " + name + " must hold " + std::to_string(n) + " values of X's dtype");
     return b->data;
 }
-void need_weight(const char* op, const Tensor& W, const char* name, Dtype dt, int rows, int cols) {
+// scales == nullptr: a weight of the activation dtype; otherwise an INT8 weight with FP32 per-output-row scales.
+// Returns the scales pointer for the C ABI.
+const float* need_weight(const char* op, const Tensor& W, const char* name, Dtype dt, int rows, int cols, const Tensor* scales = nullptr) {
     need_gpu(op, W);
-    if (W.dtype != dt) fail(std::string(op) + ": " + name + " must have X's dtype");
+    if (scales) {
+        need_gpu(op, *scales);
+        if (W.dtype != Dtype::INT8) fail(std::string(op) + ": " + name + " must be INT8");
+        if (scales->dtype != Dtype::FP32 || scales->size() != static_cast<std::size_t>(W.rows))
+            fail(std::string(op) + ": " + name + " scales must hold one FP32 value per output row");
+    } else if (W.dtype != dt) {
+        fail(std::string(op) + ": " + name + " must have X's dtype");
+    }
     if ((rows >= 0 && W.rows != rows) || W.cols != cols)
         fail(std::string(op) + ": " + name + " is (" + std::to_string(W.rows) + ", " + std::to_string(W.cols) + "), expected (" +
              (rows >= 0 ? std::to_string(rows) : std::string("out")) + ", " + std::to_string(cols) + ")");
+    return scales ? static_cast<const float*>(scales->data) : nullptr;
 }
 Tensor& thread_scratch() {
     // never destroyed: a destructor running at thread or process exit could call into a GPU runtime that is already gone
@@ -171,13 +181,14 @@ void lend_scratch(mi_attn_block_args& a, Tensor* scratch, bool with_kv) {
     a.scratch = s.data; a.scratch_bytes = s.bytes();
 }
 void init_block(mi_attn_block_args& a, const char* op, const Tensor& X, const Tensor& Wq, const Tensor* bq, const Tensor& Wo,
-                const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out) {
+                const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out, const Tensor* q_scales = nullptr,
+                const Tensor* o_scales = nullptr) {
     need_gpu(op, X);
     std::memset(&a, 0, sizeof(a));
     a.struct_size = sizeof(a);
     a.dtype = dtype_code(op, X.dtype);
-    need_weight(op, Wq, "Wq", X.dtype, -1, X.cols);
-    need_weight(op, Wo, "Wo", X.dtype, -1, Wq.rows);
+    a.wq_scales = need_weight(op, Wq, "Wq", X.dtype, -1, X.cols, q_scales);
+    a.wo_scales = need_weight(op, Wo, "Wo", X.dtype, -1, Wq.rows, o_scales);
     if (out.data == nullptr || out.rows != X.rows || out.cols != Wo.rows || out.dtype != X.dtype) out.resize(X.rows, Wo.rows, X.dtype, X.device);
     a.x = X.data; a.wq = Wq.data; a.wo = Wo.data; a.out = out.data;
     a.bq = bias_ptr(op, bq, "bq", X.dtype, Wq.rows);
@@ -188,10 +199,10 @@ void init_block(mi_attn_block_args& a, const char* op, const Tensor& X, const Te
 }
 }  // namespace
 
-void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor& Y) {
-    const char* op = "linear_batched";
+namespace {
+void linear_impl(const char* op, const Tensor& W, const Tensor* scales, const Tensor* bias, const Tensor& X, Tensor& Y) {
     need_gpu(op, X);
-    need_weight(op, W, "W", X.dtype, -1, X.cols);
+    const float* w_scales = need_weight(op, W, "W", X.dtype, -1, X.cols, scales);
     if (Y.data == nullptr || Y.rows != X.rows || Y.cols != W.rows || Y.dtype != X.dtype) Y.resize(X.rows, W.rows, X.dtype, X.device);
     mi_linear_args a;
     std::memset(&a, 0, sizeof(a));
@@ -200,19 +211,27 @@ void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor
     a.x = X.data; a.w = W.data; a.y = Y.data;
     a.bias = bias_ptr(op, bias, "bias", X.dtype, W.rows);
     a.rows = X.rows; a.in_features = X.cols; a.out_features = W.rows;
+    a.w_scales = w_scales;
     check(op, mi_linear_forward(&a));
 }
+}  // namespace
 
-void flash_attention_qkvo_forward(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor* bq, const Tensor& Wk,
-                                  const Tensor* bk, const Tensor& Wv, const Tensor* bv, const Tensor& Wo, const Tensor* bo,
-                                  const float* d_mask, int num_heads, bool causal, Tensor& out, Tensor* scratch) {
-    const char* op = "flash_attention_qkvo_forward";
+void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor& Y) { linear_impl("linear_batched", W, nullptr, bias, X, Y); }
+void linear_forward_batched_int8w_fp16(const Tensor& W_int8, const Tensor& scales, const Tensor* bias, const Tensor& X, Tensor& Y) {
+    linear_impl("linear_forward_batched_int8w_fp16", W_int8, &scales, bias, X, Y);
+}
+
+namespace {
+struct Scales { const Tensor* q; const Tensor* k; const Tensor* v; const Tensor* o; };
+void qkvo_impl(const char* op, const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor* bq, const Tensor& Wk,
+               const Tensor* bk, const Tensor& Wv, const Tensor* bv, const Tensor& Wo, const Tensor* bo, const float* d_mask,
+               int num_heads, bool causal, Tensor& out, Tensor* scratch, const Scales& sc) {
     mi_attn_block_args a;
-    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out);
+    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out, sc.q, sc.o);
     const Tensor& S = Ctx ? *Ctx : X;
     if (Ctx) { need_gpu(op, S); if (S.dtype != X.dtype) fail(std::string(op) + ": Ctx must have X's dtype"); }
-    need_weight(op, Wk, "Wk", X.dtype, Wq.rows, S.cols);
-    need_weight(op, Wv, "Wv", X.dtype, Wq.rows, S.cols);
+    a.wk_scales = need_weight(op, Wk, "Wk", X.dtype, Wq.rows, S.cols, sc.k);
+    a.wv_scales = need_weight(op, Wv, "Wv", X.dtype, Wq.rows, S.cols, sc.v);
     a.ctx = Ctx ? S.data : nullptr;
     a.wk = Wk.data; a.wv = Wv.data;
     a.bk = bias_ptr(op, bk, "bk", X.dtype, Wq.rows);
@@ -221,13 +240,11 @@ void flash_attention_qkvo_forward(const Tensor& X, const Tensor* Ctx, const Tens
     lend_scratch(a, scratch, true);
     check(op, mi_flash_attention_qkvo_forward(&a));
 }
-
-void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq, const Tensor* bq,
-                                              const Tensor& Wo, const Tensor* bo, const float* d_mask, int num_heads, bool causal,
-                                              Tensor& out, Tensor* scratch) {
-    const char* op = "flash_attention_q_with_kv_cached_forward";
+void kv_cached_impl(const char* op, const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq, const Tensor* bq,
+                    const Tensor& Wo, const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out, Tensor* scratch,
+                    const Scales& sc) {
     mi_attn_block_args a;
-    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out);
+    init_block(a, op, X, Wq, bq, Wo, bo, d_mask, num_heads, causal, out, sc.q, sc.o);
     need_gpu(op, K); need_gpu(op, V);
     if (K.dtype != X.dtype || V.dtype != X.dtype || K.cols != Wq.rows || V.cols != K.cols || V.rows != K.rows)
         fail(std::string(op) + ": K and V must be (Lk, " + std::to_string(Wq.rows) + ") of X's dtype");
@@ -235,13 +252,11 @@ void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, 
     lend_scratch(a, scratch, false);
     check(op, mi_flash_attention_q_with_kv_cached_forward(&a));
 }
-
-void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
-                                Tensor& K_out, Tensor& V_out) {
-    const char* op = "flash_attention_project_kv";
+void project_kv_impl(const char* op, const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
+                     Tensor& K_out, Tensor& V_out, const Scales& sc) {
     need_gpu(op, ctx);
-    need_weight(op, Wk, "Wk", ctx.dtype, -1, ctx.cols);
-    need_weight(op, Wv, "Wv", ctx.dtype, Wk.rows, ctx.cols);
+    const float* wk_scales = need_weight(op, Wk, "Wk", ctx.dtype, -1, ctx.cols, sc.k);
+    const float* wv_scales = need_weight(op, Wv, "Wv", ctx.dtype, Wk.rows, ctx.cols, sc.v);
     for (Tensor* t : {&K_out, &V_out})
         if (t->data == nullptr || t->rows != ctx.rows || t->cols != Wk.rows || t->dtype != ctx.dtype) t->resize(ctx.rows, Wk.rows, ctx.dtype, ctx.device);
     mi_attn_block_args a;
@@ -253,7 +268,42 @@ void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tenso
     a.bv = bias_ptr(op, bv, "bv", ctx.dtype, Wk.rows);
     a.k = K_out.data; a.v = V_out.data;
     a.batch = 1; a.kv_len = ctx.rows; a.ctx_channels = ctx.cols; a.inner = Wk.rows;
+    a.wk_scales = wk_scales; a.wv_scales = wv_scales;
     check(op, mi_flash_attention_project_kv(&a));
+}
+}  // namespace
+
+void flash_attention_qkvo_forward(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor* bq, const Tensor& Wk,
+                                  const Tensor* bk, const Tensor& Wv, const Tensor* bv, const Tensor& Wo, const Tensor* bo,
+                                  const float* d_mask, int num_heads, bool causal, Tensor& out, Tensor* scratch) {
+    qkvo_impl("flash_attention_qkvo_forward", X, Ctx, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch, Scales{});
+}
+void flash_attention_qkvo_int8w_fp16(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor& Wq_scales, const Tensor* bq,
+                                     const Tensor& Wk, const Tensor& Wk_scales, const Tensor* bk, const Tensor& Wv,
+                                     const Tensor& Wv_scales, const Tensor* bv, const Tensor& Wo, const Tensor& Wo_scales,
+                                     const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out, Tensor* scratch) {
+    qkvo_impl("flash_attention_qkvo_int8w_fp16", X, Ctx, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch,
+              Scales{&Wq_scales, &Wk_scales, &Wv_scales, &Wo_scales});
+}
+void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq, const Tensor* bq,
+                                              const Tensor& Wo, const Tensor* bo, const float* d_mask, int num_heads, bool causal,
+                                              Tensor& out, Tensor* scratch) {
+    kv_cached_impl("flash_attention_q_with_kv_cached_forward", X, K, V, Wq, bq, Wo, bo, d_mask, num_heads, causal, out, scratch, Scales{});
+}
+void flash_attention_q_with_kv_cached_int8w_fp16(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq,
+                                                 const Tensor& Wq_scales, const Tensor* bq, const Tensor& Wo, const Tensor& Wo_scales,
+                                                 const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out,
+                                                 Tensor* scratch) {
+    kv_cached_impl("flash_attention_q_with_kv_cached_int8w_fp16", X, K, V, Wq, bq, Wo, bo, d_mask, num_heads, causal, out, scratch,
+                   Scales{&Wq_scales, nullptr, nullptr, &Wo_scales});
+}
+void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
+                                Tensor& K_out, Tensor& V_out) {
+    project_kv_impl("flash_attention_project_kv", ctx, Wk, bk, Wv, bv, K_out, V_out, Scales{});
+}
+void flash_attention_project_kv_int8w_fp16(const Tensor& ctx, const Tensor& Wk, const Tensor& Wk_scales, const Tensor* bk,
+                                           const Tensor& Wv, const Tensor& Wv_scales, const Tensor* bv, Tensor& K_out, Tensor& V_out) {
+    project_kv_impl("flash_attention_project_kv_int8w_fp16", ctx, Wk, bk, Wv, bv, K_out, V_out, Scales{nullptr, &Wk_scales, &Wv_scales, nullptr});
 }
 
 }  // namespace bt

@@ -53,6 +53,21 @@ void flash_attention_q_with_kv_cached_forward(const Tensor& X, const Tensor& K, 
 void flash_attention_project_kv(const Tensor& ctx, const Tensor& Wk, const Tensor* bk, const Tensor& Wv, const Tensor* bv,
                                 Tensor& K_out, Tensor& V_out);
 
+// W8A16 forms (INT8 weight (out, in) + FP32 per-output-row scales (out, 1)), argument order of the brotensor operators
+// the quantised U-Net calls (src/unet_blocks.cpp:238-240, :256-262, :305-310; src/unet.cpp:470-474).
+void linear_forward_batched_int8w_fp16(const Tensor& W_int8, const Tensor& scales, const Tensor* bias, const Tensor& X, Tensor& Y);
+void flash_attention_qkvo_int8w_fp16(const Tensor& X, const Tensor* Ctx, const Tensor& Wq, const Tensor& Wq_scales, const Tensor* bq,
+                                     const Tensor& Wk, const Tensor& Wk_scales, const Tensor* bk, const Tensor& Wv,
+                                     const Tensor& Wv_scales, const Tensor* bv, const Tensor& Wo, const Tensor& Wo_scales,
+                                     const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out,
+                                     Tensor* scratch = nullptr);
+void flash_attention_q_with_kv_cached_int8w_fp16(const Tensor& X, const Tensor& K, const Tensor& V, const Tensor& Wq,
+                                                 const Tensor& Wq_scales, const Tensor* bq, const Tensor& Wo, const Tensor& Wo_scales,
+                                                 const Tensor* bo, const float* d_mask, int num_heads, bool causal, Tensor& out,
+                                                 Tensor* scratch = nullptr);
+void flash_attention_project_kv_int8w_fp16(const Tensor& ctx, const Tensor& Wk, const Tensor& Wk_scales, const Tensor* bk,
+                                           const Tensor& Wv, const Tensor& Wv_scales, const Tensor* bv, Tensor& K_out, Tensor& V_out);
+
 }  // namespace bt
 
 // The fused helpers of the SD1.5 transformer block, names and argument order of include/brodiffusion/fused_transformer.h:

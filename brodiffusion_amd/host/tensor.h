@@ -14,10 +14,10 @@
 
 namespace bdamd {
 
-enum class Dtype { FP32, FP16, BF16 };
+enum class Dtype { FP32, FP16, BF16, INT8 };
 enum class Device { CPU, GPU };
 
-inline std::size_t dtype_size(Dtype d) { return d == Dtype::FP32 ? 4 : 2; }
+inline std::size_t dtype_size(Dtype d) { return d == Dtype::FP32 ? 4 : (d == Dtype::INT8 ? 1 : 2); }
 
 [[noreturn]] inline void fail(const std::string& msg) { throw std::runtime_error(msg); }
 

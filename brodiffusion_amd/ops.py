@@ -274,6 +274,18 @@ def _mat(op: str, t, name: str, dtype, rows=None, cols=None):
         _fail(op, f"{name} has {t.shape[-1]} columns, expected {cols}")
 
 
+def _weight(op: str, W, scales, name: str, dtype, rows=None, cols=None) -> int:
+    """A weight operand: of the activation dtype, or INT8 with FP32 per-output-row scales. Returns the scales pointer (0: none)."""
+    if scales is None:
+        _mat(op, W, name, dtype, rows=rows, cols=cols)
+        return 0
+    _mat(op, W, name, torch.int8, rows=rows, cols=cols)
+    _dev(op, scales)
+    if scales.dtype != torch.float32 or scales.numel() != W.shape[0] or not scales.is_contiguous():
+        _fail(op, f"{name} scales must hold {W.shape[0]} contiguous float32 values (one per output row)")
+    return scales.data_ptr()
+
+
 def _bias(op: str, b, name: str, dtype, n: int):
     if b is None:
         return 0
@@ -283,13 +295,14 @@ def _bias(op: str, b, name: str, dtype, n: int):
     return b.data_ptr()
 
 
-def linear_batched(W, bias, X, Y: Optional[torch.Tensor] = None):
-    """Y = X W^T + bias; W (out_features, in_features), X (..., in_features)."""
-    op = "linear_batched"
+def linear_batched(W, bias, X, Y: Optional[torch.Tensor] = None, W_scales: Optional[torch.Tensor] = None,
+                   op: str = "linear_batched"):
+    """Y = X W^T + bias; W (out_features, in_features), X (..., in_features). With W_scales, W is INT8 and
+    Y = (X W^T) * scales + bias (see linear_forward_batched_int8w_fp16)."""
     _dev(op, W, X)
     if W.dim() != 2 or X.shape[-1] != W.shape[1]:
         _fail(op, f"X has {X.shape[-1]} columns, W is {tuple(W.shape)}")
-    _mat(op, W, "W", X.dtype)
+    w_scales = _weight(op, W, W_scales, "W", X.dtype)
     _mat(op, X, "X", X.dtype)
     rows = X.numel() // X.shape[-1]
     if Y is None:
@@ -303,9 +316,16 @@ def linear_batched(W, bias, X, Y: Optional[torch.Tensor] = None):
     a.x, a.w, a.y = X.data_ptr(), W.data_ptr(), Y.data_ptr()
     a.bias = _bias(op, bias, "bias", X.dtype, W.shape[0])
     a.rows, a.in_features, a.out_features = rows, W.shape[1], W.shape[0]
+    a.w_scales = w_scales
     a.stream = _stream()
     capi.check(capi.lib().mi_linear_forward(C.byref(a)), op)
     return Y
+
+
+def linear_forward_batched_int8w_fp16(W_int8, scales, bias, X, Y: Optional[torch.Tensor] = None):
+    """W8A16 linear layer, argument order of bt::linear_forward_batched_int8w_fp16 (src/unet_blocks.cpp:238-240):
+    W_int8 (out, in) INT8, scales (out, 1) FP32, bias of X's dtype or None."""
+    return linear_batched(W_int8, bias, X, Y, W_scales=scales, op="linear_forward_batched_int8w_fp16")
 
 
 def fused_linear_geglu(X, W, b, Y: Optional[torch.Tensor] = None):
@@ -362,7 +382,8 @@ def flash_attention_scratch_bytes(batch: int, q_len: int, kv_len: int, inner: in
     return int(capi.lib().mi_flash_attention_scratch_bytes(batch, q_len, kv_len, inner, int(with_kv)))
 
 
-def _attn_block(op: str, fn_name: str, X, Ctx, K, V, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch):
+def _attn_block(op: str, fn_name: str, X, Ctx, K, V, Wq, bq, Wk, bk, Wv, bv, Wo, bo, d_mask, num_heads, causal, out, scratch,
+                scales=(None, None, None, None)):
     _dev(op, X, Ctx, K, V, Wq, Wk, Wv, Wo, d_mask, out, scratch)
     dt = X.dtype
     B, Lq, Cx, _, _ = _as3(op, X, "X")
@@ -371,10 +392,10 @@ def _attn_block(op: str, fn_name: str, X, Ctx, K, V, Wq, bq, Wk, bk, Wv, bv, Wo,
     if Wq.dim() != 2 or Wo.dim() != 2:
         _fail(op, "Wq and Wo must be 2-D (out_features, in_features)")
     inner, Cout = Wq.shape[0], Wo.shape[0]
-    _mat(op, Wq, "Wq", dt, cols=Cx)
-    _mat(op, Wo, "Wo", dt, cols=inner)
     a = capi.MiAttnBlockArgs()
     a.struct_size = C.sizeof(a)
+    a.wq_scales = _weight(op, Wq, scales[0], "Wq", dt, cols=Cx)
+    a.wo_scales = _weight(op, Wo, scales[3], "Wo", dt, cols=inner)
     a.dtype = _dtype_code(op, X)
     a.x, a.wq, a.wo = X.data_ptr(), Wq.data_ptr(), Wo.data_ptr()
     a.bq, a.bo = _bias(op, bq, "bq", dt, inner), _bias(op, bo, "bo", dt, Cout)
@@ -394,8 +415,8 @@ def _attn_block(op: str, fn_name: str, X, Ctx, K, V, Wq, bq, Wk, bk, Wv, bv, Wo,
                 _fail(op, f"Ctx has batch {Bc}, X has {B}")
             _mat(op, Ctx, "Ctx", dt)
             a.ctx = Ctx.data_ptr()
-        for W, nm in ((Wk, "Wk"), (Wv, "Wv")):
-            _mat(op, W, nm, dt, rows=inner, cols=Cc)
+        a.wk_scales = _weight(op, Wk, scales[1], "Wk", dt, rows=inner, cols=Cc)
+        a.wv_scales = _weight(op, Wv, scales[2], "Wv", dt, rows=inner, cols=Cc)
         a.wk, a.wv = Wk.data_ptr(), Wv.data_ptr()
         a.bk, a.bv = _bias(op, bk, "bk", dt, inner), _bias(op, bv, "bv", dt, inner)
         a.ctx_channels = Cc
@@ -439,9 +460,35 @@ def flash_attention_q_with_kv_cached_forward(X, K, V, Wq, bq, Wo, bo, d_mask, nu
                        Wq, bq, None, None, None, None, Wo, bo, d_mask, num_heads, causal, out, scratch)
 
 
-def flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out: Optional[torch.Tensor] = None, V_out: Optional[torch.Tensor] = None):
+def flash_attention_qkvo_int8w_fp16(X, Ctx, Wq_int8, Wq_scales, bq, Wk_int8, Wk_scales, bk, Wv_int8, Wv_scales, bv,
+                                    Wo_int8, Wo_scales, bo, d_mask, num_heads: int, causal: bool,
+                                    out: Optional[torch.Tensor] = None, scratch: Optional[torch.Tensor] = None):
+    """flash_attention_qkvo_forward with INT8 weights and FP32 per-output-row scales (W8A16), argument order of
+    bt::flash_attention_qkvo_int8w_fp16 (src/unet_blocks.cpp:256-262)."""
+    return _attn_block("flash_attention_qkvo_int8w_fp16", "mi_flash_attention_qkvo_forward", X, Ctx, None, None,
+                       Wq_int8, bq, Wk_int8, bk, Wv_int8, bv, Wo_int8, bo, d_mask, num_heads, causal, out, scratch,
+                       scales=(Wq_scales, Wk_scales, Wv_scales, Wo_scales))
+
+
+def flash_attention_q_with_kv_cached_int8w_fp16(X, K, V, Wq_int8, Wq_scales, bq, Wo_int8, Wo_scales, bo, d_mask, num_heads: int,
+                                                causal: bool, out: Optional[torch.Tensor] = None,
+                                                scratch: Optional[torch.Tensor] = None):
+    """W8A16 form of flash_attention_q_with_kv_cached_forward (src/unet_blocks.cpp:305-310)."""
+    return _attn_block("flash_attention_q_with_kv_cached_int8w_fp16", "mi_flash_attention_q_with_kv_cached_forward", X, None, K, V,
+                       Wq_int8, bq, None, None, None, None, Wo_int8, bo, d_mask, num_heads, causal, out, scratch,
+                       scales=(Wq_scales, None, None, Wo_scales))
+
+
+def flash_attention_project_kv_int8w_fp16(ctx, Wk_int8, Wk_scales, bk, Wv_int8, Wv_scales, bv,
+                                          K_out: Optional[torch.Tensor] = None, V_out: Optional[torch.Tensor] = None):
+    """W8A16 form of flash_attention_project_kv (src/unet.cpp:470-474)."""
+    return flash_attention_project_kv(ctx, Wk_int8, bk, Wv_int8, bv, K_out, V_out, scales=(Wk_scales, Wv_scales),
+                                      op="flash_attention_project_kv_int8w_fp16")
+
+
+def flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out: Optional[torch.Tensor] = None, V_out: Optional[torch.Tensor] = None,
+                               scales=(None, None), op: str = "flash_attention_project_kv"):
     """K_out = ctx Wk^T + bk, V_out = ctx Wv^T + bv in one launch (fills the cross-attention K/V cache)."""
-    op = "flash_attention_project_kv"
     _dev(op, ctx, Wk, Wv, K_out, V_out)
     dt = ctx.dtype
     B, Lk, Cc, _, _ = _as3(op, ctx, "ctx")
@@ -449,8 +496,8 @@ def flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out: Optional[torch.Tensor
     if Wk.dim() != 2 or tuple(Wv.shape) != tuple(Wk.shape):
         _fail(op, "Wk and Wv must be 2-D and alike")
     inner = Wk.shape[0]
-    _mat(op, Wk, "Wk", dt, cols=Cc)
-    _mat(op, Wv, "Wv", dt, cols=Cc)
+    wk_scales = _weight(op, Wk, scales[0], "Wk", dt, cols=Cc)
+    wv_scales = _weight(op, Wv, scales[1], "Wv", dt, cols=Cc)
     if K_out is None:
         K_out = torch.empty(*ctx.shape[:-1], inner, dtype=dt, device=ctx.device)
     if V_out is None:
@@ -465,6 +512,7 @@ def flash_attention_project_kv(ctx, Wk, bk, Wv, bv, K_out: Optional[torch.Tensor
     a.ctx, a.wk, a.wv = ctx.data_ptr(), Wk.data_ptr(), Wv.data_ptr()
     a.bk, a.bv = _bias(op, bk, "bk", dt, inner), _bias(op, bv, "bv", dt, inner)
     a.k, a.v = K_out.data_ptr(), V_out.data_ptr()
+    a.wk_scales, a.wv_scales = wk_scales, wv_scales
     a.batch, a.kv_len, a.ctx_channels, a.inner = B, Lk, Cc, inner
     a.stream = _stream()
     capi.check(capi.lib().mi_flash_attention_project_kv(C.byref(a)), op)

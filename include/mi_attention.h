@@ -318,6 +318,11 @@ typedef struct mi_linear_args {
     void* y;
     int32_t rows, in_features, out_features;
     int64_t x_row_stride, w_row_stride, y_row_stride;
+    const float* w_scales;   /* NULL: w has `dtype`. Otherwise w is INT8 (out_features, in_features) and w_scales holds one FP32
+                                scale per output feature: Y = (X Wq^T) * scale + bias, the W8A16 form
+                                bt::linear_forward_batched_int8w_fp16 (src/unet_blocks.cpp:238-240; weights as
+                                include/brodiffusion/detail/unet_blocks.h:28-35). The bytes are widened exactly on their way
+                                to LDS and the scale is applied to the FP32 accumulator */
     void* stream;
 } mi_linear_args;
 MI_API int mi_linear_forward(const mi_linear_args* args);
@@ -376,6 +381,10 @@ typedef struct mi_attn_block_args {
     int64_t key_mask_batch_stride;   /* 0 = shared */
     void* scratch;
     size_t scratch_bytes;
+    const float* wq_scales;          /* each NULL (weight of `dtype`) or FP32 per-output-row scales of an INT8 weight: the */
+    const float* wk_scales;          /* ..._int8w_fp16 forms of the three operators (src/unet_blocks.cpp:256-262, :305-310, */
+    const float* wv_scales;          /* src/unet.cpp:470-474). The weights of one projection launch (Q/K/V) must be of one kind */
+    const float* wo_scales;
     void* stream;
 } mi_attn_block_args;
 /* Scratch bytes of the qkvo form (with_kv != 0) or the kv_cached form (with_kv == 0); project_kv needs none. */

@@ -330,6 +330,43 @@ static void gpu_checks() {
         bt::flash_attention_q_with_kv_cached_forward(X, Kc, Vc, Wq, nullptr, Wo, &Bo, nullptr, Hh, false, out2, &own_scratch);
         CHECK(out.to_host_bytes() == out2.to_host_bytes());
         CHECK(own_scratch.bytes() >= mi_flash_attention_scratch_bytes(1, Lx, Lc, C, 0));
+        // W8A16 forms: INT8 weights with per-row scales against the checker fed the dequantised weights; the cached form
+        // after project_kv equals the full form bit for bit
+        {
+            auto quant = [](uint64_t seed, int rows, int cols, std::vector<int8_t>& q, std::vector<float>& sc, std::vector<float>& deq) {
+                std::vector<float> r(static_cast<size_t>(rows) * cols);
+                orc_torch_randn_f32(seed, r.size(), r.data());
+                q.resize(r.size()); sc.resize(rows); deq.resize(r.size());
+                for (int i = 0; i < rows; ++i) sc[i] = (0.75f + 0.5f * static_cast<float>(i % 7) / 7.0f) / (42.0f * std::sqrt(static_cast<float>(cols)));
+                for (size_t i = 0; i < r.size(); ++i) {
+                    const float v = std::fmax(-127.f, std::fmin(127.f, std::nearbyint(r[i] * 42.0f)));
+                    q[i] = static_cast<int8_t>(v);
+                    deq[i] = v * sc[i / cols];
+                }
+            };
+            std::vector<int8_t> qq, qk, qv, qo;
+            std::vector<float> sq, sk, sv, so, dq, dk, dv, dO;
+            quant(7111, C, C, qq, sq, dq); quant(7112, C, Cc, qk, sk, dk); quant(7113, C, Cc, qv, sv, dv); quant(7114, C, C, qo, so, dO);
+            auto up8 = [](const std::vector<int8_t>& q, int r, int c) { return Tensor::from_host(q.data(), r, c, Dtype::INT8); };
+            auto upf = [](const std::vector<float>& f, int r) { return Tensor::from_host(f.data(), r, 1, Dtype::FP32); };
+            Tensor Wq8 = up8(qq, C, C), Wk8 = up8(qk, C, Cc), Wv8 = up8(qv, C, Cc), Wo8 = up8(qo, C, C);
+            Tensor Sq = upf(sq, C), Sk = upf(sk, C), Sv = upf(sv, C), So = upf(so, C), o8, K8, V8, o8c;
+            bt::flash_attention_qkvo_int8w_fp16(X, &Ctx, Wq8, Sq, nullptr, Wk8, Sk, nullptr, Wv8, Sv, nullptr, Wo8, So, &Bo, nullptr, Hh, false, o8);
+            const std::vector<float> q8 = lin(x, dq, nullptr, Lx, C, C, true), k8 = lin(ctx, dk, nullptr, Lc, C, Cc, true), v8 = lin(ctx, dv, nullptr, Lc, C, Cc, true);
+            std::vector<float> a8(q8.size());
+            orc_sdpa(q8.data(), k8.data(), v8.data(), Lx, Lc, Hh, C / Hh, -1.0, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr, 0, a8.data(), nullptr, 0);
+            orc_round_bf16(a8.data(), a8.size());
+            const Err e8 = compare(lin(a8, dO, bo.data(), Lx, C, C, false), download_bf16(o8));
+            std::printf("qkvo int8 weights     rel_l2=%.3e max_abs=%.3e\n", e8.rel_l2, e8.max_abs);
+            CHECK(within_bf16(e8));
+            bt::flash_attention_project_kv_int8w_fp16(Ctx, Wk8, Sk, nullptr, Wv8, Sv, nullptr, K8, V8);
+            bt::flash_attention_q_with_kv_cached_int8w_fp16(X, K8, V8, Wq8, Sq, nullptr, Wo8, So, &Bo, nullptr, Hh, false, o8c);
+            CHECK(o8.to_host_bytes() == o8c.to_host_bytes());
+            Tensor Y8;
+            bt::linear_forward_batched_int8w_fp16(Wo8, So, &Bo, X, Y8);
+            CHECK(within_bf16(compare(lin(x, dO, bo.data(), Lx, C, C, false), download_bf16(Y8))));
+            CHECK(throws_with([&] { bt::linear_forward_batched_int8w_fp16(Wo, So, &Bo, X, Y8); }, "must be INT8"));
+        }
         // the linear layer alone
         Tensor Y;
         bt::linear_batched(Wo, &Bo, X, Y);

@@ -192,3 +192,81 @@ def test_attn_block_argument_errors():
         bd.flash_attention_q_with_kv_cached_forward(x, z(5, 32), z(5, 32), w, None, w, None, None, 1, False)
     # empty query set is a no-op with an empty result
     assert bd.flash_attention_qkvo_forward(z(0, 64), None, w, None, w, None, w, None, w, None, None, 1, False).shape == (0, 64)
+
+
+# ── INT8 weights with per-output-row scales (W8A16) ──────────────────────────
+def quantised(seed, n_out, n_in, pow2=False):
+    rng = np.random.default_rng(seed)
+    q = rng.integers(-127, 128, (n_out, n_in)).astype(np.int8)
+    if pow2:
+        scales = np.full(n_out, 2.0 ** -8, np.float32) * (2.0 ** rng.integers(-1, 2, n_out)).astype(np.float32)
+    else:
+        scales = (rng.uniform(0.5, 1.5, n_out) / (73.0 * np.sqrt(n_in))).astype(np.float32)     # rows of unit-variance weights
+    return q, scales, q.astype(np.float32) * scales[:, None]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(77, 320, 768), (8192, 320, 320), (300, 72, 1000), (257, 1280, 1280)])
+def test_linear_int8w_matches_checker(oracle, dtype, M, N, K):
+    x = randn(31 + M, (M, K), dtype)
+    q, scales, w = quantised(32 + N, N, K)
+    b = randn(33 + K, (N,), dtype)
+    dq, ds = torch.from_numpy(q).cuda(), torch.from_numpy(scales).cuda()
+    y = bd.linear_forward_batched_int8w_fp16(dq, ds, to_dev(b, dtype), to_dev(x, dtype))
+    ref = oracle.linear(x, w, b)                                             # the dequantised weight in FP32
+    assert_close(ref, to_np(y), dtype, f"int8w linear {M}x{N}x{K}")
+    unit = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    assert np.all(np.abs(to_np(y) - ref) <= unit * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)
+    with pytest.raises(RuntimeError, match="scales must hold"):
+        bd.linear_forward_batched_int8w_fp16(dq, ds[:-1], None, to_dev(x, dtype))
+    with pytest.raises(RuntimeError, match="dtype"):
+        bd.linear_forward_batched_int8w_fp16(dq.to(torch.int16), ds, None, to_dev(x, dtype))
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_int8w_equals_16bit_weights_when_exactly_representable(dtype):
+    """Power-of-two scales: the dequantised weight is exact in fp16 / bf16 and scaling the accumulator by a power of
+    two is exact, so the W8A16 path and the 16-bit path must give the same bits."""
+    M, N, K = 1000, 320, 768
+    q, scales, w = quantised(41, N, K, pow2=True)
+    x = to_dev(randn(42, (M, K), dtype), dtype)
+    b = to_dev(randn(43, (N,), dtype), dtype)
+    dq, ds = torch.from_numpy(q).cuda(), torch.from_numpy(scales).cuda()
+    assert torch.equal(bd.linear_forward_batched_int8w_fp16(dq, ds, None, x), bd.linear_batched(to_dev(w, dtype), None, x))
+    # with a bias the two epilogues (fused multiply-add, then conversion / add and conversion in one mixed-precision
+    # instruction) may round a value that sits on a tie differently: at most one unit in the last place, rarely
+    y8, y16 = bd.linear_forward_batched_int8w_fp16(dq, ds, b, x), bd.linear_batched(to_dev(w, dtype), b, x)
+    unit = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    diff = (y8.float() - y16.float()).abs()
+    assert (diff <= unit * y16.float().abs().clamp(min=1.0)).all() and (diff > 0).float().mean().item() < 1e-3
+
+
+def test_qkvo_int8w_block_and_kv_cache(oracle):
+    dtype, B, L, C, H, Lc, Cc = "fp16", 2, 1024, 320, 8, 77, 768
+    x, ctx = randn(7601, (B, L, C), dtype), randn(7602, (B, Lc, Cc), dtype)
+    (qq, sq, wq), (qk, sk, wk), (qv, sv, wv), (qo, so, wo) = (quantised(7610 + i, C, cin) for i, cin in enumerate((C, Cc, Cc, C)))
+    bo = randn(7620, (C,), dtype) * 0.25
+    bo = oracle.round_to(bo, dtype)
+    g = lambda a: torch.from_numpy(a).cuda()
+    dx, dctx, dbo = to_dev(x, dtype), to_dev(ctx, dtype), to_dev(bo, dtype)
+    out = bd.flash_attention_qkvo_int8w_fp16(dx, dctx, g(qq), g(sq), None, g(qk), g(sk), None, g(qv), g(sv), None, g(qo), g(so), dbo,
+                                             None, H, False)
+    for b in range(B):
+        ref = oracle.attention_qkvo(x[b], ctx[b], wq, None, wk, None, wv, None, wo, bo, H, dtype)
+        print("int8w qkvo", assert_close(ref, to_np(out[b]), dtype, f"int8w qkvo batch {b}"))
+    K, V = bd.flash_attention_project_kv_int8w_fp16(dctx, g(qk), g(sk), None, g(qv), g(sv), None)
+    cached = bd.flash_attention_q_with_kv_cached_int8w_fp16(dx, K, V, g(qq), g(sq), None, g(qo), g(so), dbo, None, H, False)
+    assert torch.equal(cached, out)
+    # self-attention form: Q, K, V all from X in one INT8 launch
+    (_, _, wk1), (_, _, wv1) = quantised(7630, C, C), quantised(7631, C, C)
+    qk1, sk1, _ = quantised(7630, C, C)
+    qv1, sv1, _ = quantised(7631, C, C)
+    out_self = bd.flash_attention_qkvo_int8w_fp16(dx, None, g(qq), g(sq), None, g(qk1), g(sk1), None, g(qv1), g(sv1), None,
+                                                  g(qo), g(so), dbo, None, H, False)
+    ref = oracle.attention_qkvo(x[0], None, wq, None, wk1, None, wv1, None, wo, bo, H, dtype)
+    assert_close(ref, to_np(out_self[0]), dtype, "int8w qkvo self")
+    # mixing an INT8 Q weight with 16-bit K / V weights in the one projection launch is refused
+    with pytest.raises(RuntimeError, match="cannot share a launch"):
+        bd.ops._attn_block("flash_attention_qkvo_int8w_fp16", "mi_flash_attention_qkvo_forward", dx, None, None, None,
+                           g(qq), None, to_dev(wk1, dtype), None, to_dev(wv1, dtype), None, g(qo), dbo, None, H, False, None, None,
+                           scales=(g(sq), None, None, g(so)))
