@@ -197,6 +197,16 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
         if (reinterpret_cast<uintptr_t>(a->logit_bias) & 3u) return fail("mi_sdpa_forward: logit_bias must be 4-byte aligned");
         if (a->bias_cols == 0 || a->bias_q0 >= a->q_len) p.bias = nullptr;   // nothing to add
     }
+    if ((a->cu_seqlens_q == nullptr) != (a->cu_seqlens_k == nullptr)) return fail("mi_sdpa_forward: cu_seqlens_q and cu_seqlens_k must be given together");
+    if (a->cu_seqlens_q) {
+        if (a->prefix_len > 0 || a->key_mask || a->kv_valid_len || a->rope_cos_q || a->rope_cos_k || a->logit_bias || a->lse_out)
+            return fail("mi_sdpa_forward: packed variable-length sequences take no prefix, key mask, kv_valid_len, RoPE, bias or lse_out");
+        if (a->mask_mode == MI_MASK_BLOCK_CAUSAL || (a->mask_mode == MI_MASK_CAUSAL && a->window != 0))
+            return fail("mi_sdpa_forward: packed variable-length sequences support MI_MASK_NONE and unwindowed MI_MASK_CAUSAL");
+        if ((reinterpret_cast<uintptr_t>(a->cu_seqlens_q) | reinterpret_cast<uintptr_t>(a->cu_seqlens_k)) & 3u)
+            return fail("mi_sdpa_forward: cu_seqlens must be 4-byte aligned");
+        p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+    }
     if (a->lse_out) {
         if (reinterpret_cast<uintptr_t>(a->lse_out) & 3u) return fail("mi_sdpa_forward: lse_out must be 4-byte aligned");
         p.lse = a->lse_out;

@@ -76,6 +76,7 @@ struct SdpaDev {
     // additive logit bias (natural-log units, added to the scaled score) for query rows >= bias_q0 and keys < bias_cols
     const float* bias; int bias_q0, bias_cols; long bias_rs;
     float inv_scale;              // 1 / scale: the bias in units of the raw dot product
+    const int* cu_q; const int* cu_k;   // packed variable-length sequences: [B + 1] row offsets, or null
     float* lse;                   // [B][H][Lq] base-2 log of the softmax denominator in exponent units, or null
     SplitGeo split;               // enabled != 0: split the last round along the key axis
     unsigned char* split_scratch; // partial slots, [8 groups][max_tail][max_parts] of SplitGeo::slot_bytes

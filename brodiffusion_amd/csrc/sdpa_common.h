@@ -150,12 +150,13 @@ __device__ __forceinline__ WaveExtent wave_extent(int lo, int hi) {
 // chunk are fetched from a clamped address and blanked at the store.
 // q_scale != 1 folds a factor (softmax scale times log2 e) into Q before its single rounding to T.
 template <typename T, int D, int NT, int ROWS>
-__device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p, const T* q_base, int q0, int tid, float q_scale = 1.f) {
+__device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p, const T* q_base, int q0, int tid, float q_scale = 1.f,
+                                             int last_row_override = -1) {
     using G = HeadGeo<D>;
     constexpr int CPRK = G::DK / 8;            // chunks per staged row (data chunks, then the zero pad)
     constexpr int NCH = ROWS * CPRK;
     constexpr int NI = (NCH + NT - 1) / NT;
-    const int last_row = p.Lq - 1;
+    const int last_row = last_row_override >= 0 ? last_row_override : p.Lq - 1;   // (a packed sequence has its own length)
     const bool rope = p.cos_q != nullptr;
     u32x4 raw[NI];
     f32x4 cs[NI], sn[NI];

@@ -218,8 +218,11 @@ template <int D> constexpr int lds_bytes_4() {
     return kv > o ? kv : o;
 }
 
-template <typename T, int D, bool ROPE_K>
-__global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(const SdpaDev p) {
+// VARLEN: the batch items are sequences of different lengths packed back to back along the row axis
+// (cu_q / cu_k: device arrays of batch + 1 row offsets, the cu_seqlens convention); Lq and Lk of the launch are the
+// longest sequence and only size the grid. Each work group rebuilds the launch view for its own sequence.
+template <typename T, int D, bool ROPE_K, bool VARLEN = false>
+__global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(const SdpaDev p_in) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
     constexpr int BM = 128;
@@ -228,9 +231,21 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     constexpr int STAGE = G::K_BYTES + G::V_BYTES + kBN * 4;   // K tile, V tile, 64 key-mask floats
 
     int qt, bh;
-    if (!block_to_tile(p, qt, bh)) return;
-    const int h = bh % p.H;
-    const int b = bh / p.H;
+    if (!block_to_tile(p_in, qt, bh)) return;
+    const int h = bh % p_in.H;
+    const SdpaDev& p = p_in;
+    // this work group's sequence: row offsets into the packed tensors, its own lengths and causal offset
+    int b = bh / p.H, Lq = p.Lq, Lk = p.Lk, q_offset = p.q_offset;
+    long q_row0 = 0, k_row0 = 0;
+    if constexpr (VARLEN) {
+        const int qs = p.cu_q[b], ks = p.cu_k[b];
+        Lq = p.cu_q[b + 1] - qs;
+        Lk = p.cu_k[b + 1] - ks;
+        if (qt * BM >= Lq) return;
+        q_row0 = qs; k_row0 = ks;
+        q_offset = Lk - Lq;   // causal: the last query meets the last key, per sequence
+        b = 0;                // batch strides do not apply to packed rows
+    }
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in a scalar register
@@ -239,19 +254,25 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     const int lh = lane >> 5;
     const int q0 = qt * BM;
     const int qrow = q0 + wave * 32 + lq;
-    const bool qvalid = qrow < p.Lq;
+    const bool qvalid = qrow < Lq;
     const int hk = h / p.kv_group;
-    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
-    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + q_row0 * p.q_rs + h * D;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + q_row0 * p.o_rs + h * D;
     const float* const key_mask = p.key_mask ? p.key_mask + b * p.key_mask_bs : nullptr;
     const float* const bias_row = (p.bias && qvalid && qrow >= p.bias_q0) ? p.bias + static_cast<long>(qrow - p.bias_q0) * p.bias_rs : nullptr;
 
     int lo, hi;
-    row_interval(p, b, qrow, qvalid, lo, hi);
+    if constexpr (VARLEN) {
+        lo = 0;
+        hi = p.mask_mode == MI_MASK_CAUSAL ? min(Lk, q_offset + qrow + 1) : Lk;
+        if (!qvalid || hi <= lo) { lo = 0; hi = 0; }
+    } else {
+        row_interval(p, b, qrow, qvalid, lo, hi);
+    }
     const WaveExtent we = wave_extent(lo, hi);
     if (lane == 0) { red[wave] = we.lo_min; red[4 + wave] = we.hi_max; }
     V8 qf[G::KC];
-    stage_q_tile<T, D, kThreads4, BM>(smem, p, q_base, q0, tid);
+    stage_q_tile<T, D, kThreads4, BM>(smem, p, q_base, q0, tid, 1.f, Lq - 1);
     __syncthreads();
     read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
     __syncthreads();
@@ -271,8 +292,8 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     const float lazy_raw = kLazyLog2 / cl2;
 
     TileMover<T, D, kThreads4, ROPE_K> mv{p, plan,
-                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D),
-                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + k_row0 * p.k_rs + hk * D),
+                                          reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + k_row0 * p.v_rs + hk * D),
                                           reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.kp) + b * p.kp_bs + hk * D),
                                           reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.vp) + b * p.vp_bs + hk * D),
                                           tid, {}, {}, 1.f};
@@ -329,10 +350,10 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     // base-2 log of the row's denominator in exponent units: p(key) = exp2(score * scale_log2 [+ bias * log2 e] - lse);
     // +inf for a row without visible keys, so that every p is 0
     if (p.lse && qvalid && lh == 0)
-        p.lse[(static_cast<long>(b) * p.H + h) * p.Lq + qrow] = l_tot > 0.f ? st.mc + __builtin_amdgcn_logf(l_tot) : __builtin_huge_valf();
+        p.lse[(static_cast<long>(b) * p.H + h) * Lq + qrow] = l_tot > 0.f ? st.mc + __builtin_amdgcn_logf(l_tot) : __builtin_huge_valf();
     stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
     __syncthreads();
-    write_output<T, D, kThreads4>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
+    write_output<T, D, kThreads4>(smem, o_base, p.o_rs, q0, Lq, BM, tid);
 }
 
 // ───────────────────────── short key sequences (cross attention) ─────────────────────────
@@ -1112,7 +1133,7 @@ template <int D>
 bool plan_split(SdpaDev& p, int n_cu) {
     p.split = SplitGeo{};
     if constexpr (!dma_kernel_available<D>()) return false;
-    if (p.mask_mode != MI_MASK_NONE || p.kv_valid_len || p.key_mask || p.Lp > 0 || p.cos_k) return false;
+    if (p.mask_mode != MI_MASK_NONE || p.kv_valid_len || p.key_mask || p.Lp > 0 || p.cos_k || p.cu_q) return false;
     if (n_cu < 8 || n_cu % 8 != 0 || sdpa_kernel_choice() == 1 || sdpa_kernel_choice() == 3) return false;
     const long tiles = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int T = (p.Lk + kBN - 1) / kBN;
@@ -1143,6 +1164,14 @@ size_t split_scratch_bytes_d(SdpaDev p, int n_cu) {
 template <typename T, int D>
 int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     const bool rope_k = p.cos_k != nullptr;
+    if (p.cu_q != nullptr) {
+        p.n_q_tiles = (p.Lq + 127) / 128;
+        p.n_blocks = p.B * p.H * p.n_q_tiles;
+        hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false, true>), dim3(grid_blocks(p)), dim3(kThreads4), lds_bytes_4<D>(), stream, p);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail("sdpa_fwd launch: %s", hipGetErrorString(e));
+        return 0;
+    }
     if constexpr (dma_kernel_available<D>()) {
         if (p.split_scratch != nullptr && plan_split<D>(p, n_cu) &&
             p.split_scratch_bytes >= static_cast<size_t>(8) * p.split.max_tail * p.split.max_parts * SplitGeo::slot_bytes(D)) {

@@ -85,6 +85,31 @@ void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Te
     run_sdpa(op, a);
 }
 
+void flash_attention_gqa_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* key_mask, int num_q_heads,
+                                 int num_kv_heads, bool causal, Tensor& out) {
+    const char* op = "flash_attention_gqa_forward";
+    if (num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) fail(std::string(op) + ": num_kv_heads must divide num_q_heads");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_q_heads, num_kv_heads, out);
+    a.key_mask = key_mask;
+    if (causal) { a.mask_mode = MI_MASK_CAUSAL; a.q_offset = K.rows - Q.rows; }
+    run_sdpa(op, a);
+}
+
+void flash_attention_varlen_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const int32_t* cu_q, const int32_t* cu_k,
+                                    int n_seqs, int max_q, int max_k, int num_heads, int head_dim, bool causal, Tensor& out) {
+    const char* op = "flash_attention_varlen_forward";
+    if (!cu_q || !cu_k || n_seqs <= 0 || max_q < 0 || max_k < 0) fail(std::string(op) + ": cu_q, cu_k and a positive n_seqs are required");
+    if (head_dim <= 0 || Q.cols != num_heads * head_dim) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    mi_sdpa_args a;
+    init_args(a, op, Q, K, V, num_heads, num_heads, out);
+    a.batch = n_seqs; a.q_len = max_q; a.kv_len = max_k;
+    a.q_batch_stride = a.k_batch_stride = a.v_batch_stride = a.o_batch_stride = 8;   // ignored for packed sequences
+    a.cu_seqlens_q = cu_q; a.cu_seqlens_k = cu_k;
+    if (causal) a.mask_mode = MI_MASK_CAUSAL;
+    run_sdpa(op, a);
+}
+
 static void rope_impl(const char* op, const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads,
                       Tensor& out, bool per_head) {
     need_gpu(op, X); need_gpu(op, cos); need_gpu(op, sin);

@@ -3,6 +3,8 @@
 // the brodiffusion wrappers the reference calls (paths in the reference repository):
 //   bt::flash_attention_forward            src/dit/common.cpp:194
 //   bt::flash_attention_windowed_forward   src/dit/qwenimage21_forward.cpp:662
+//   bt::flash_attention_gqa_forward        src/ardy/denoiser_backbone.cpp:179
+//   bt::flash_attention_varlen_forward     src/dit/krea2.cpp:574
 //   bt::rope_apply / rope_apply_perhead    src/dit/common.cpp:192, src/triposplat/flow_model.cpp:374
 //   dit::joint_attention                   include/brodiffusion/dit/common.h:80-88
 //   dit::gqa_attention_masked              include/brodiffusion/dit/common.h:144-153
@@ -26,6 +28,13 @@ void flash_attention_forward(const Tensor& Q, const Tensor& K, const Tensor& V, 
                              int num_heads, bool causal, Tensor& out);
 void flash_attention_windowed_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* d_mask,
                                       int num_heads, int window, Tensor& out);
+// Grouped-query attention with an optional key mask (src/ardy/denoiser_backbone.cpp:179) and packed variable-length
+// attention (src/dit/krea2.cpp:574: sequence i owns query rows [cu_q[i], cu_q[i+1]) and key rows [cu_k[i], cu_k[i+1]);
+// cu_q / cu_k are device int32 arrays of n_seqs + 1 offsets).
+void flash_attention_gqa_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const float* key_mask, int num_q_heads,
+                                 int num_kv_heads, bool causal, Tensor& out);
+void flash_attention_varlen_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const int32_t* cu_q, const int32_t* cu_k,
+                                    int n_seqs, int max_q, int max_k, int num_heads, int head_dim, bool causal, Tensor& out);
 void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
 void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
 

@@ -5,6 +5,8 @@ Names, argument order and error behaviour follow the brotensor operators the ref
 
     flash_attention_forward(Q, K, V, d_mask, num_heads, causal, out)        src/dit/common.cpp:194
     flash_attention_windowed_forward(Q, K, V, d_mask, num_heads, window, out) src/dit/qwenimage21_forward.cpp:662
+    flash_attention_varlen_forward(q, k, v, cu_q, cu_k, n_seqs, max_q, max_k, num_heads, head_dim, causal, out)
+                                                                             src/dit/krea2.cpp:574
     rope_apply(X, cos, sin, head_dim, num_heads, out)                        src/dit/common.cpp:192
     rope_apply_perhead(X, cos, sin, head_dim, num_heads, out)                src/triposplat/flow_model.cpp:374
     joint_attention(Q, K, V, cos, sin, head_dim, num_heads, out, Qr, Kr)     include/brodiffusion/dit/common.h:80-88
@@ -247,6 +249,42 @@ def flash_attention_forward(Q, K, V, d_mask, num_heads: int, causal: bool, out: 
     Lq, Lk = Q.shape[-2], K.shape[-2]
     mask = SdpaMask.causal(Lk - Lq) if causal else None
     return sdpa_forward(Q, K, V, num_heads, out=out, key_mask=d_mask, mask=mask, op=op)
+
+
+def flash_attention_varlen_forward(q, k, v, cu_q, cu_k, n_seqs: int, max_q: int, max_k: int, num_heads: int, head_dim: int,
+                                   causal: bool, out: Optional[torch.Tensor] = None):
+    """Attention over n_seqs sequences of different lengths packed along the row axis: sequence i owns query rows
+    [cu_q[i], cu_q[i+1]) of q / out and key rows [cu_k[i], cu_k[i+1]) of k / v (device int32 arrays of n_seqs + 1 offsets);
+    max_q / max_k bound the sequence lengths. Argument order of bt::flash_attention_varlen_forward (src/dit/krea2.cpp:574)."""
+    op = "flash_attention_varlen_forward"
+    _dev(op, q, k, v, cu_q, cu_k, out)
+    dt = _dtype_code(op, q)
+    if q.dim() != 2 or k.dim() != 2 or v.dim() != 2 or q.stride(1) != 1 or k.stride(1) != 1 or v.stride(1) != 1:
+        _fail(op, "q, k, v must be 2-D packed (total rows, heads*head_dim), contiguous along columns")
+    if k.dtype != q.dtype or v.dtype != q.dtype or q.shape[1] != num_heads * head_dim or k.shape[1] != q.shape[1] or tuple(v.shape) != tuple(k.shape):
+        _fail(op, "q, k, v must share dtype and heads*head_dim columns; k and v the same shape")
+    for t, nm in ((cu_q, "cu_q"), (cu_k, "cu_k")):
+        if t.dtype != torch.int32 or t.numel() != n_seqs + 1 or not t.is_contiguous():
+            _fail(op, f"{nm} must be a contiguous int32 tensor of n_seqs + 1 offsets")
+    if n_seqs <= 0 or max_q < 0 or max_k < 0:
+        _fail(op, "n_seqs must be positive, max_q and max_k non-negative")
+    if out is None:
+        out = torch.empty_like(q)
+    if out.shape != q.shape or out.dtype != q.dtype or out.stride(1) != 1:
+        _fail(op, "out must have q's shape and dtype")
+    a = capi.MiSdpaArgs()
+    a.struct_size = C.sizeof(capi.MiSdpaArgs)
+    a.dtype = dt
+    a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.batch, a.num_heads, a.head_dim = n_seqs, num_heads, head_dim
+    a.q_len, a.kv_len = max_q, max_k
+    a.q_row_stride, a.k_row_stride, a.v_row_stride, a.o_row_stride = q.stride(0), k.stride(0), v.stride(0), out.stride(0)
+    a.q_batch_stride = a.k_batch_stride = a.v_batch_stride = a.o_batch_stride = 8      # ignored for packed sequences
+    a.mask_mode = capi.MI_MASK_CAUSAL if causal else capi.MI_MASK_NONE
+    a.cu_seqlens_q, a.cu_seqlens_k = cu_q.data_ptr(), cu_k.data_ptr()
+    a.stream = _stream()
+    capi.check(capi.lib().mi_sdpa_forward(C.byref(a)), op)
+    return out
 
 
 def flash_attention_windowed_forward(Q, K, V, d_mask, num_heads: int, window: int, out: Optional[torch.Tensor] = None):

@@ -153,6 +153,13 @@ typedef struct mi_sdpa_args {
     float* lse_out;              /* device FP32 [batch][num_heads][q_len] or NULL: receives per row the base-2 logarithm of the
                                     softmax denominator in exponent units, lse = log2 sum_k 2^(score_k*scale*log2(e) + bias*log2(e))
                                     (+inf for a row without visible keys); input of mi_attention_map_avg */
+    const int32_t* cu_seqlens_q; /* device int32 [batch + 1], or NULL. With both given, the batch items are sequences of different */
+    const int32_t* cu_seqlens_k; /* lengths packed along the row axis: item b owns query rows [cu_seqlens_q[b], cu_seqlens_q[b+1]) of q / o
+                                    and key rows [cu_seqlens_k[b], cu_seqlens_k[b+1]) of k / v; q_len and kv_len are the LONGEST
+                                    sequence (they size the launch), batch strides are ignored. bt::flash_attention_varlen_forward
+                                    (q, k, v, cu_q, cu_k, n_seqs, max_q, max_k, num_heads, head_dim, causal, out),
+                                    src/dit/krea2.cpp:574. MI_MASK_NONE or MI_MASK_CAUSAL (window 0; each sequence aligns its last
+                                    query with its last key); no prefix, key mask, kv_valid_len, RoPE, bias */
     void* split_scratch;         /* device, 16-byte aligned, or NULL: lets a launch whose last round of work groups would fill
                                     only part of the GPU cut the query tiles of that round along the key axis into equal
                                     pieces for all compute units (partial results in the scratch, merged by a second small

@@ -404,6 +404,27 @@ static void gpu_checks() {
         CHECK(throws_with([&] { add_inplace_vec(Ya, Xa.row_view(0, 5)); }, "must match in shape"));
         CHECK(throws_with([&] { add_inplace_row_bias(Yb, Xa); }, "bias must hold"));
     }
+    {   // packed variable-length attention: each sequence equals a call on its own rows; GQA wrapper equals the plain op at kv = q heads
+        const std::vector<int32_t> cu = {0, 19, 19, 50, L};
+        int32_t* d_cu = static_cast<int32_t*>(mi_malloc(cu.size() * sizeof(int32_t)));
+        CHECK(d_cu != nullptr && mi_memcpy_h2d(d_cu, cu.data(), cu.size() * sizeof(int32_t)) == 0);
+        Tensor o_var;
+        bt::flash_attention_varlen_forward(Q, K, V, d_cu, d_cu, 4, L - 50, L - 50, H, d, false, o_var);
+        const std::vector<uint8_t> all = o_var.to_host_bytes();
+        for (size_t i = 0; i + 1 < cu.size(); ++i) {
+            const int r0 = cu[i], n = cu[i + 1] - cu[i];
+            if (n == 0) continue;
+            Tensor o_seq;
+            bt::flash_attention_forward(Q.row_view(r0, n), K.row_view(r0, n), V.row_view(r0, n), nullptr, H, false, o_seq);
+            const std::vector<uint8_t> one = o_seq.to_host_bytes();
+            CHECK(std::memcmp(all.data() + static_cast<size_t>(r0) * D * 2, one.data(), one.size()) == 0);
+        }
+        mi_free(d_cu);
+        Tensor o_gqa, o_plain;
+        bt::flash_attention_gqa_forward(Q, K, V, nullptr, H, H, false, o_gqa);
+        bt::flash_attention_forward(Q, K, V, nullptr, H, false, o_plain);
+        CHECK(o_gqa.to_host_bytes() == o_plain.to_host_bytes());
+    }
     {   // GPU-side error path: unsupported head_dim surfaces the C ABI's message
         Tensor out;
         CHECK(throws_with([&] { bt::flash_attention_forward(Q, K, V, nullptr, 8, false, out); }, "no kernel"));
