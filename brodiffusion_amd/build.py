@@ -60,6 +60,7 @@ def build(save_temps: bool = False, verbose: bool = False) -> str:
 HOST_DIR = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIB_DIR, "libbrodiffusion_amd_host.so")
 HOST_TEST = os.path.join(LIB_DIR, "test_host_ops")
+SPLIT_TEST = os.path.join(LIB_DIR, "test_split_geo")
 CXX = os.environ.get("CXX", "g++")
 
 
@@ -82,6 +83,14 @@ def build_host(with_test: bool = True, verbose: bool = False) -> str:
         if r.returncode != 0:
             sys.stderr.write(r.stdout + r.stderr)
             raise RuntimeError("host test build failed")
+    if with_test:
+        # host-only check of the launch-planning arithmetic shared by host and device code (needs the HIP headers: hipcc)
+        cmd = [HIPCC, "-std=c++20", "-O1", "-Wall", "--offload-host-only", "-x", "hip", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+               os.path.join(ROOT, "tests", "cpp", "test_split_geo.cpp"), "-o", SPLIT_TEST]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            sys.stderr.write(r.stdout + r.stderr)
+            raise RuntimeError("split-geometry test build failed")
     if verbose:
         print("built", HOST_LIB)
     return HOST_LIB

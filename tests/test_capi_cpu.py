@@ -141,3 +141,13 @@ def test_host_cpp_layer_error_paths():
         build.build_host()
     r = subprocess.run([build.HOST_TEST, "--cpu"], capture_output=True, text=True)
     assert r.returncode == 0 and "test_host_ops: OK" in r.stdout, r.stdout + r.stderr
+
+
+def test_split_planning_arithmetic_brute_force():
+    """tests/cpp/test_split_geo.cpp: the formulas that cut the last round of an attention launch into pieces (shared by
+    the host planner and the kernels) against their definition, over 180 (tiles, key steps, slots) configurations."""
+    from brodiffusion_amd import build
+    if not os.path.exists(build.SPLIT_TEST):
+        build.build_host()
+    r = subprocess.run([build.SPLIT_TEST], capture_output=True, text=True)
+    assert r.returncode == 0 and "test_split_geo: OK" in r.stdout, r.stdout + r.stderr
