@@ -415,8 +415,11 @@ int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st)
     {
         LinDev ps = p;
         const int tiles = (ps.N + kStateTile - 1) / kStateTile;
+        // the largest split that still gives every group a CU of its own and at least two tiles (40 heads on 256 CUs: 6;
+        // two groups per CU measured slower, a power of two leaves a third of the CUs idle)
         int split = 1;
-        while (split * 2 <= max_split && BH * split * 2 <= n_cu && tiles / (split * 2) >= 2) split *= 2;
+        for (int s2 = 2; s2 <= max_split; ++s2)
+            if (BH * s2 <= n_cu && tiles / s2 >= 2) split = s2;
         ps.tokens_per_group = ((tiles + split - 1) / split) * kStateTile;
         ps.n_chunks = (ps.N + ps.tokens_per_group - 1) / ps.tokens_per_group;
         ps.n_blocks = BH * ps.n_chunks;
