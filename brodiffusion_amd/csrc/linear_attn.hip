@@ -80,9 +80,6 @@ __device__ __forceinline__ u32x4 relu8(u32x4 raw) {
     return __builtin_bit_cast(u32x4, x);
 }
 
-__global__ void __launch_bounds__(256) fill_zero_kernel(f32x4* p, long n4) {
-    for (long i = blockIdx.x * 256L + threadIdx.x; i < n4; i += gridDim.x * 256L) p[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-}
 
 // Work group -> (batch*head, token chunk). Hardware work-group ids go round the 8 XCDs, each with its own L2: the
 // logical index is arranged so that one XCD gets a contiguous range of heads with all their chunks. Then the heads

@@ -1,18 +1,21 @@
-// Flash-style softmax attention forward for gfx950 (MI355X), hand-written. Two kernels share the
-// building blocks of sdpa_common.h:
+// Flash-style softmax attention forward for gfx950 (MI355X), hand-written. Four kernels share the building blocks of
+// sdpa_common.h; launch_d picks one per call:
 //
-//   sdpa_fwd_pp_kernel   8 wavefronts = 256 query rows per work group, 2 wavefronts per SIMD. The two
-//                        wavefronts of a SIMD run half a tile apart: while one issues the MFMAs of
-//                        O += V^T P (tile t) and S = K Q^T (tile t+1), the other does the softmax of
-//                        its own tile on the VALU, so the matrix and vector pipes of the SIMD are busy
-//                        at the same time. The phase shift is set up once by one extra barrier for the
-//                        second group and kept by the two work-group barriers of every iteration.
-//   sdpa_fwd_kernel      4 wavefronts = 128 query rows per work group, 2 work groups per CU; used when
-//                        the problem has too few 256-row tiles to fill the chip.
+//   sdpa_fwd_kernel         4 wavefronts = 128 query rows per work group, K/V tiles through registers into padded LDS,
+//                           double buffered. Small problems, head_dim 160, calls with a key mask, a logit bias, a
+//                           request for the softmax denominators, or packed variable-length sequences.
+//   sdpa_fwd_pp_kernel      8 wavefronts = 256 query rows, 2 wavefronts per SIMD, one work-group barrier per key tile:
+//                           between two barriers every wavefront runs the MFMA stream (O += V^T P of tile t, then
+//                           S = K Q^T of tile t+1) and one softmax, in opposite order in the two groups of four, so the
+//                           matrix pipe and the VALU of a SIMD are busy at the same time.
+//   sdpa_fwd_pp_dma_kernel  the same schedule with K/V tiles moved global -> LDS by DMA (head_dim 72 and 128), optionally
+//                           with the last, partly filled round of work groups cut along the key axis (SPLIT) and merged
+//                           by sdpa_combine_kernel.
+//   sdpa_shortkv_kernel     short key sequences (cross attention): K and V of a head stay in LDS, a work group walks
+//                           several query tiles, no barrier in the key loop.
 //
-// Key/value tiles of 64 rows are staged in LDS (double buffered, loaded one tile ahead through
-// registers). Not in HBM: scores, probabilities, rotated Q/K (RoPE is applied as Q and K are loaded),
-// the [prefix ; fresh] K/V concatenation (two source pointers), any mask tensor (per-row visible-key
+// Not in HBM: scores, probabilities, rotated Q (RoPE is applied as Q is loaded; K either the same way or by one pass into
+// a caller scratch), the [prefix ; fresh] K/V concatenation (two source pointers), any mask tensor (per-row visible-key
 // intervals; key tiles outside every row's interval are skipped).
 #include <type_traits>
 
