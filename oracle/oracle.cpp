@@ -396,10 +396,14 @@ ORC_API void orc_sdpa(const float* q, const float* k, const float* v, int Lq, in
 // with q_offset = Lk - Lq (or any offset) query row r attends keys [0, q_offset + r];
 // window > 0 keeps only the last `window` of those.
 ORC_API void orc_rows_causal(int Lq, int Lk, int q_offset, int window, int* row_lo, int* row_hi) {
+    // The window is counted in positions, from the query's own position back: a query that sits beyond the last key
+    // (q_offset + r >= Lk, outside what the reference ever calls) sees fewer than `window` keys, possibly none.
     for (int r = 0; r < Lq; ++r) {
-        const int hi = std::min(Lk, q_offset + r + 1);
-        row_hi[r] = std::max(hi, 0);
-        row_lo[r] = window > 0 ? std::max(0, hi - window) : 0;
+        const int pos1 = q_offset + r + 1;
+        const int hi = std::max(std::min(Lk, pos1), 0);
+        const int lo = window > 0 ? std::max(0, pos1 - window) : 0;
+        row_hi[r] = hi;
+        row_lo[r] = std::min(lo, hi);
     }
 }
 // Block-causal segments, following include/brodiffusion/dit/qwenimage21.h:31-33 and the

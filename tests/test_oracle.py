@@ -468,3 +468,12 @@ def test_geglu_exact_vs_torch_float64(oracle):
     assert out[0, 0] == 0.0 and abs((out[0, 1] - out[0, 2]) - 1.7) < 1e-6
     # the value half is the first half: swapping the halves changes the result
     assert not np.allclose(oracle.geglu_exact(t), oracle.geglu_exact(np.concatenate([t[:, 24:], t[:, :24]], axis=1)))
+
+
+def test_window_is_counted_in_positions(oracle):
+    """A windowed query at position p sees keys (p - window, p] that exist: hand-worked for queries that run past the
+    last key (outside what the reference calls: there q_offset = Lk - Lq and both readings coincide)."""
+    lo, hi = oracle.rows_causal(5, 3, 0, 2)
+    assert list(zip(lo, hi)) == [(0, 1), (0, 2), (1, 3), (2, 3), (3, 3)]
+    lo, hi = oracle.rows_causal(3, 10, 7, 4)          # q_offset = Lk - Lq: the last 4 keys up to the diagonal
+    assert list(zip(lo, hi)) == [(4, 8), (5, 9), (6, 10)]
