@@ -38,7 +38,7 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-configs", action="store_true")
     ap.add_argument("--traffic-probe", action="store_true",
-                    help="few launches of the headline step plus one 256 MiB tensor copy; run under rocprofv3 --pmc "
+                    help="few launches of the headline step and of cfg5 plus one 256 MiB tensor copy; run under rocprofv3 --pmc "
                          "FETCH_SIZE (or WRITE_SIZE): the copy calibrates the counter, the step gives HBM bytes per launch")
     return ap.parse_args()
 
@@ -204,11 +204,16 @@ def main():
     if args.traffic_probe:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)
+        # cfg5 (Sana ReLU linear attention, B=2 H=20 d=112 N=4096) rides along: its kernels are the HBM-bound ones
+        lq, lk, lv = (torch.randn(2, 4096, 2240, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(3))
+        lo = torch.empty_like(lq)
+        lws = torch.empty(2 * 20 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
         for _ in range(3):
             dst.copy_(src)
             step()
+            bd.linear_attention_relu_forward(lq, lk, lv, 20, out=lo, workspace=lws)
         torch.cuda.synchronize()
-        print(json.dumps({"traffic_probe": "3 x (256 MiB copy, headline step)"}))
+        print(json.dumps({"traffic_probe": "3 x (256 MiB copy, headline step, Sana linear attention N=4096)"}))
         return
     preheat(torch, step)
     for _ in range(args.warmup):
