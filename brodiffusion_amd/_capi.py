@@ -69,7 +69,7 @@ class MiAttentionMapArgs(C.Structure):
         ("num_heads", C.c_int32), ("head_dim", C.c_int32), ("q_len", C.c_int32), ("kv_len", C.c_int32),
         ("q_row_stride", C.c_int64), ("k_row_stride", C.c_int64), ("map_row_stride", C.c_int64),
         ("scale", C.c_float), ("logit_bias", C.c_void_p), ("bias_q0", C.c_int32), ("bias_cols", C.c_int32),
-        ("bias_row_stride", C.c_int64), ("stream", C.c_void_p),
+        ("bias_row_stride", C.c_int64), ("key_mask", C.c_void_p), ("stream", C.c_void_p),
     ]
 
 

@@ -1,4 +1,5 @@
-// Head-averaged attention map for traced forwards: map[q][k] = (1/H) sum_h softmax_h(q, k), FP32, for batch 1.
+// Head-averaged attention map for traced forwards: map[q][k] = (1/H) sum_h softmax_h(q, k), FP32, for batch 1
+// (0 in the columns of keys that a key mask hides).
 //
 // The flash kernels never materialise the softmax; a traced forward wants it averaged over heads. The attention
 // launch leaves the base-2 log of every row's denominator (lse, per head and query row); this kernel recomputes the
@@ -44,6 +45,15 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) avg[kb][e] = 0.f;
+    // bit 16 kb + e: this lane's key (kb, e) counts (inside the sequence and not masked)
+    unsigned live = 0;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+            if (key < p.Lk && (p.key_mask == nullptr || p.key_mask[key] != 0.f)) live |= 1u << (16 * kb + e);
+        }
 
     const T* const qg = static_cast<const T*>(p.q);
     const T* const kg = static_cast<const T*>(p.k);
@@ -84,7 +94,7 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
                 const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
                 float s2 = sacc[kb][e] * p.scale_log2;
                 if (bias_row && key < p.bias_cols) s2 = __builtin_fmaf(bias_row[key], kLog2e, s2);
-                avg[kb][e] += __builtin_amdgcn_exp2f(s2 - lse);
+                if (live & (1u << (16 * kb + e))) avg[kb][e] += __builtin_amdgcn_exp2f(s2 - lse);
             }
         __syncthreads();   // all reads of this head's K tile are done before the next head overwrites it
     }

@@ -288,7 +288,8 @@ int mi_attention_map_avg(const mi_attention_map_args* a) {
     if (p.q_rs < D || p.k_rs < D || p.map_rs < a->kv_len) return fail("%s: a row stride is smaller than its row", op);
     if (p.q_rs % 8 || p.k_rs % 8) return fail("%s: q / k row strides must be multiples of 8 elements", op);
     if (!mi::aligned16(a->q) || !mi::aligned16(a->k) || !mi::aligned16(a->map)) return fail("%s: q, k and map must be 16-byte aligned", op);
-    if ((reinterpret_cast<uintptr_t>(a->lse) | reinterpret_cast<uintptr_t>(a->logit_bias)) & 3u) return fail("%s: lse and logit_bias must be 4-byte aligned", op);
+    if ((reinterpret_cast<uintptr_t>(a->lse) | reinterpret_cast<uintptr_t>(a->logit_bias) | reinterpret_cast<uintptr_t>(a->key_mask)) & 3u)
+        return fail("%s: lse, logit_bias and key_mask must be 4-byte aligned", op);
     const float scale = a->scale > 0.f ? a->scale : 1.0f / std::sqrt(static_cast<float>(a->head_dim));
     p.scale_log2 = scale * 1.4426950408889634f;
     if (a->logit_bias && a->bias_cols > 0 && a->bias_q0 < a->q_len) {
@@ -297,6 +298,7 @@ int mi_attention_map_avg(const mi_attention_map_args* a) {
         p.bias_rs = a->bias_row_stride ? a->bias_row_stride : a->bias_cols;
         if (p.bias_rs < p.bias_cols) return fail("%s: bias_row_stride smaller than bias_cols", op);
     }
+    p.key_mask = a->key_mask;
     return mi::launch_attention_map(p, a->dtype, a->head_dim, mi::resolve_stream(a->stream));
 }
 

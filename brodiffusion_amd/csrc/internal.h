@@ -105,6 +105,7 @@ struct MapDev {
     long q_rs, k_rs, map_rs;
     float scale_log2;
     const float* bias; int bias_q0, bias_cols; long bias_rs;
+    const float* key_mask;        // [Lk] or null
 };
 int launch_attention_map(const MapDev& p, int dtype, int head_dim, hipStream_t stream);
 

@@ -331,6 +331,47 @@ void flash_attention_project_kv_int8w_fp16(const Tensor& ctx, const Tensor& Wk, 
     project_kv_impl("flash_attention_project_kv_int8w_fp16", ctx, Wk, bk, Wv, bv, K_out, V_out, Scales{nullptr, &Wk_scales, &Wv_scales, nullptr});
 }
 
+void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const Tensor& Wq, const Tensor& Wk, const Tensor& Wv,
+                                       const Tensor& Wo, const float* d_mask, const Tensor* logit_bias, int num_heads,
+                                       Tensor& out, Tensor& AttnAvg) {
+    const char* op = "cross_attention_forward_with_attn";
+    need_gpu(op, X); need_gpu(op, Ctx);
+    if (Ctx.dtype != X.dtype) fail(std::string(op) + ": Ctx must have X's dtype");
+    const int Lq = X.rows, Lk = Ctx.rows;
+    if (num_heads <= 0 || Wq.rows % num_heads != 0) fail(std::string(op) + ": num_heads must divide the projection width");
+    const float* bias = nullptr;
+    if (logit_bias != nullptr) {
+        need_gpu(op, *logit_bias);
+        if (logit_bias->dtype != Dtype::FP32 || logit_bias->rows != Lq || logit_bias->cols != Lk) fail(std::string(op) + ": logit_bias must be FP32 (Lq, Lk)");
+        bias = static_cast<const float*>(logit_bias->data);
+    }
+    // per-thread scratch, never destroyed (see thread_scratch): projected Q, K, V, the attention output, the denominators
+    struct Work { Tensor q, k, v, a, lse; };
+    static thread_local Work* w = new Work;
+    linear_impl(op, Wq, nullptr, nullptr, X, w->q);
+    linear_impl(op, Wk, nullptr, nullptr, Ctx, w->k);
+    linear_impl(op, Wv, nullptr, nullptr, Ctx, w->v);
+    if (w->k.cols != w->q.cols || w->v.cols != w->q.cols) fail(std::string(op) + ": Wq, Wk and Wv must project to one width");
+    if (w->lse.data == nullptr || w->lse.size() < static_cast<std::size_t>(num_heads) * Lq) w->lse.resize(num_heads, Lq, Dtype::FP32, Device::GPU);
+    mi_sdpa_args a;
+    init_args(a, op, w->q, w->k, w->v, num_heads, num_heads, w->a);
+    a.key_mask = d_mask;
+    a.logit_bias = bias; a.bias_q0 = 0; a.bias_cols = bias ? Lk : 0;
+    a.lse_out = static_cast<float*>(w->lse.data);
+    check(op, mi_sdpa_forward(&a));
+    if (AttnAvg.data == nullptr || AttnAvg.rows != Lq || AttnAvg.cols != Lk || AttnAvg.dtype != Dtype::FP32) AttnAvg.resize(Lq, Lk, Dtype::FP32, X.device);
+    mi_attention_map_args m;
+    std::memset(&m, 0, sizeof(m));
+    m.struct_size = sizeof(m);
+    m.dtype = a.dtype;
+    m.q = w->q.data; m.k = w->k.data; m.lse = a.lse_out; m.map = static_cast<float*>(AttnAvg.data);
+    m.num_heads = num_heads; m.head_dim = a.head_dim; m.q_len = Lq; m.kv_len = Lk;
+    m.logit_bias = bias; m.bias_q0 = 0; m.bias_cols = a.bias_cols;
+    m.key_mask = d_mask;
+    check(op, mi_attention_map_avg(&m));
+    linear_impl(op, Wo, nullptr, nullptr, w->a, out);
+}
+
 }  // namespace bt
 
 void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y) {

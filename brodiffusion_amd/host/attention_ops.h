@@ -13,6 +13,7 @@
 //   bt::flash_attention_qkvo_forward       src/unet_blocks.cpp:264-272
 //   bt::flash_attention_q_with_kv_cached_forward  src/unet_blocks.cpp:311-317
 //   bt::flash_attention_project_kv         src/unet.cpp:476-480
+//   bt::cross_attention_forward_with_attn  src/unet_blocks.cpp:282-290
 //   detail::linear_batched                 include/brodiffusion/detail/compute.h:52-62
 //   headnorm + bt::rope_apply              src/dit/qwenimage21_forward.cpp:53-63, :582-585
 // Precondition failures throw std::runtime_error("<op>: <message>"); a CPU tensor is refused.
@@ -76,6 +77,14 @@ void flash_attention_q_with_kv_cached_int8w_fp16(const Tensor& X, const Tensor& 
                                                  Tensor* scratch = nullptr);
 void flash_attention_project_kv_int8w_fp16(const Tensor& ctx, const Tensor& Wk, const Tensor& Wk_scales, const Tensor* bk,
                                            const Tensor& Wv, const Tensor& Wv_scales, const Tensor* bv, Tensor& K_out, Tensor& V_out);
+
+// The U-Net's traced cross attention (src/unet_blocks.cpp:282-290): Q = X Wq^T, K = Ctx Wk^T, V = Ctx Wv^T (no biases),
+// attention with the optional additive logit bias (FP32 (Lq, Lk)) and key mask, out = A Wo^T (no bias: the caller adds
+// it), AttnAvg = the FP32 (Lq, Lk) softmax averaged over the heads. Everything stays on the device; the projected
+// tensors live in a per-thread scratch.
+void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const Tensor& Wq, const Tensor& Wk, const Tensor& Wv,
+                                       const Tensor& Wo, const float* d_mask, const Tensor* logit_bias, int num_heads,
+                                       Tensor& out, Tensor& AttnAvg);
 
 }  // namespace bt
 

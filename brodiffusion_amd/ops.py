@@ -677,11 +677,11 @@ def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optio
 
 
 def attention_map_avg(q, k, lse, num_heads: int, *, scale: Optional[float] = None, logit_bias: Optional[torch.Tensor] = None,
-                      bias_q0: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      bias_q0: int = 0, key_mask: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """(Lq, Lk) float32 map: the softmax of every head averaged over the heads. `lse` is what sdpa_forward wrote to
-    lse_out for the same q, k, scale and bias."""
+    lse_out for the same q, k, scale, bias and key_mask (float32 (Lk,), 1 = valid; masked columns of the map are 0)."""
     op = "attention_map_avg"
-    _dev(op, q, k, lse, logit_bias, out)
+    _dev(op, q, k, lse, logit_bias, key_mask, out)
     if q.dim() != 2 or k.dim() != 2 or q.stride(1) != 1 or k.stride(1) != 1 or q.shape[1] != k.shape[1] or q.dtype != k.dtype:
         _fail(op, "q and k must be 2-D (L, heads*head_dim) of one dtype, contiguous along columns")
     Lq, Lk = q.shape[0], k.shape[0]
@@ -702,6 +702,10 @@ def attention_map_avg(q, k, lse, num_heads: int, *, scale: Optional[float] = Non
         if logit_bias.dtype != torch.float32 or logit_bias.dim() != 2 or logit_bias.stride(1) != 1 or logit_bias.shape[0] != Lq - bias_q0:
             _fail(op, "logit_bias must be float32 (Lq - bias_q0, cols)")
         a.logit_bias, a.bias_q0, a.bias_cols, a.bias_row_stride = logit_bias.data_ptr(), bias_q0, logit_bias.shape[1], logit_bias.stride(0)
+    if key_mask is not None:
+        if key_mask.dtype != torch.float32 or key_mask.numel() != Lk or not key_mask.is_contiguous():
+            _fail(op, "key_mask must be contiguous float32 (Lk,)")
+        a.key_mask = key_mask.data_ptr()
     a.stream = _stream()
     capi.check(capi.lib().mi_attention_map_avg(C.byref(a)), op)
     return out
@@ -733,6 +737,40 @@ def joint_attention_traced(Q, K, V, cos, sin, head_dim: int, num_heads: int, out
     bias = image_text_bias if (image_text_bias is not None and txt_len > 0 and txt_len < L) else None
     out = sdpa_forward(Qr, Kr, V, num_heads, out=out, logit_bias=bias, bias_q0=txt_len, lse_out=lse, op=op)
     attn_avg = attention_map_avg(Qr, Kr, lse, num_heads, logit_bias=bias, bias_q0=txt_len, out=attn_avg)
+    return out, attn_avg
+
+
+def cross_attention_forward_with_attn(X, Ctx, Wq, Wk, Wv, Wo, d_mask, logit_bias, num_heads: int,
+                                      out: Optional[torch.Tensor] = None, attn_avg: Optional[torch.Tensor] = None):
+    """bt::cross_attention_forward_with_attn as the U-Net's traced cross attention calls it (src/unet_blocks.cpp:282-290):
+    Q = X Wq^T, K = Ctx Wk^T, V = Ctx Wv^T (no biases), attention with the optional additive logit bias (float32
+    (Lq, Lk)) and key mask (float32 (Lk,), 1 = valid), output projection with Wo (no bias: the caller adds it), and
+    the softmax averaged over the heads as a float32 (Lq, Lk) map. All on the device. Returns (out, attn_avg)."""
+    op = "cross_attention_forward_with_attn"
+    _dev(op, X, Ctx, Wq, Wk, Wv, Wo, d_mask, logit_bias, out, attn_avg)
+    if X.dim() != 2 or Ctx.dim() != 2:
+        _fail(op, "X and Ctx must be 2-D (rows, channels)")
+    Lq, Lk = X.shape[0], Ctx.shape[0]
+    inner = Wq.shape[0]
+    if inner % num_heads != 0:
+        _fail(op, "num_heads must divide the projection width")
+    if logit_bias is not None and (logit_bias.dtype != torch.float32 or tuple(logit_bias.shape) != (Lq, Lk)):
+        _fail(op, "logit_bias must be float32 (Lq, Lk)")
+    if d_mask is not None and (d_mask.dtype != torch.float32 or d_mask.numel() != Lk):
+        _fail(op, "d_mask must be float32 (Lk,)")
+    q = torch.empty(Lq, inner, dtype=X.dtype, device=X.device)
+    k = torch.empty(Lk, inner, dtype=X.dtype, device=X.device)
+    v = torch.empty(Lk, inner, dtype=X.dtype, device=X.device)
+    linear_batched(Wq, None, X, q, op=op)
+    linear_batched(Wk, None, Ctx, k, op=op)
+    linear_batched(Wv, None, Ctx, v, op=op)
+    lse = torch.empty(num_heads, Lq, dtype=torch.float32, device=X.device)
+    mask = None if d_mask is None else d_mask.reshape(Lk).contiguous()
+    a = sdpa_forward(q, k, v, num_heads, logit_bias=logit_bias, key_mask=mask, lse_out=lse, op=op)
+    attn_avg = attention_map_avg(q, k, lse, num_heads, logit_bias=logit_bias, key_mask=mask, out=attn_avg)
+    if out is None:
+        out = torch.empty(Lq, Wo.shape[0], dtype=X.dtype, device=X.device)
+    linear_batched(Wo, None, a, out, op=op)
     return out, attn_avg
 
 

@@ -185,9 +185,10 @@ MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);
 /* ── head-averaged attention map ───────────────────────────────────────────
  * map[q][k] = (1/num_heads) * sum over heads of softmax_h(q, k), FP32 (q_len, kv_len): the trace artifact of
  * dit::joint_attention_traced (src/dit/common.cpp:297, :308-312), which the reference computes in a host loop over
- * downloaded tensors. q, k as given to mi_sdpa_forward (already rotated), unmasked attention, batch 1; `lse` is what
- * that call wrote to lse_out with the same scale and bias. Every element is accumulated in one register over the
- * heads and written once (no atomics). */
+ * downloaded tensors, and of bt::cross_attention_forward_with_attn (src/unet_blocks.cpp:282-290). q, k as given to
+ * mi_sdpa_forward (already rotated), batch 1, no mask other than key_mask; `lse` is what that call wrote to lse_out
+ * with the same scale, bias and key_mask. Every element is accumulated in one register over the heads and written
+ * once (no atomics). */
 typedef struct mi_attention_map_args {
     uint32_t struct_size;
     int32_t dtype;
@@ -201,6 +202,7 @@ typedef struct mi_attention_map_args {
     const float* logit_bias;
     int32_t bias_q0, bias_cols;
     int64_t bias_row_stride;
+    const float* key_mask;   /* null, or [kv_len]: 1 = valid, 0 = masked (those map columns are 0) */
     void* stream;
 } mi_attention_map_args;
 MI_API int mi_attention_map_avg(const mi_attention_map_args* args);

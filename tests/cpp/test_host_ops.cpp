@@ -274,6 +274,51 @@ static void gpu_checks() {
         CHECK(throws_with([&] { Tensor b2 = Tensor::from_host(bias.data(), L - txt, txt - 1, Dtype::FP32);
                                 dit::joint_attention_traced(Q, K, V, tabs.cos, tabs.sin, d, H, out, avg, Qr, Kr, txt, &b2); }, "(img_len, txt_len)"));
     }
+    {   // the U-Net's traced cross attention: projections, logit bias + key mask, output projection, head-averaged map
+        const int Lq = 200, Lk = 50, C = 128, Cc = 96, Hc = 2, dc = C / Hc;
+        auto weight = [&](uint64_t seed, int rows, int cols) {
+            std::vector<float> w(static_cast<size_t>(rows) * cols);
+            orc_torch_randn_f32(seed, w.size(), w.data());
+            for (float& x : w) x /= std::sqrt(static_cast<float>(cols));
+            orc_round_bf16(w.data(), w.size());
+            return w;
+        };
+        const std::vector<float> x = randn_bf16(7401, static_cast<size_t>(Lq) * C), ctx = randn_bf16(7402, static_cast<size_t>(Lk) * Cc);
+        const std::vector<float> wq = weight(7403, C, C), wk = weight(7404, C, Cc), wv = weight(7405, C, Cc), wo = weight(7406, C, C);
+        std::vector<float> bias(static_cast<size_t>(Lq) * Lk), mask(Lk, 1.f);
+        orc_torch_randn_f32(7407, bias.size(), bias.data());
+        mask[3] = 0.f;
+        for (int j = Lk - 7; j < Lk; ++j) mask[j] = 0.f;
+        Tensor X = upload_bf16(x, Lq, C), Ctx = upload_bf16(ctx, Lk, Cc), Wq = upload_bf16(wq, C, C), Wk = upload_bf16(wk, C, Cc),
+               Wv = upload_bf16(wv, C, Cc), Wo = upload_bf16(wo, C, C), B = Tensor::from_host(bias.data(), Lq, Lk, Dtype::FP32),
+               M = Tensor::from_host(mask.data(), 1, Lk, Dtype::FP32), out, avg;
+        bt::cross_attention_forward_with_attn(X, Ctx, Wq, Wk, Wv, Wo, static_cast<const float*>(M.data), &B, Hc, out, avg);
+        std::vector<float> qp(static_cast<size_t>(Lq) * C), kp(static_cast<size_t>(Lk) * C), vp(kp.size()), a(qp.size()), ref(qp.size()),
+            ref_avg(static_cast<size_t>(Lq) * Lk);
+        orc_linear(x.data(), wq.data(), nullptr, Lq, C, C, qp.data(), 0);
+        orc_linear(ctx.data(), wk.data(), nullptr, Lk, C, Cc, kp.data(), 0);
+        orc_linear(ctx.data(), wv.data(), nullptr, Lk, C, Cc, vp.data(), 0);
+        orc_round_bf16(qp.data(), qp.size()); orc_round_bf16(kp.data(), kp.size()); orc_round_bf16(vp.data(), vp.size());
+        orc_sdpa(qp.data(), kp.data(), vp.data(), Lq, Lk, Hc, dc, -1.0, mask.data(), nullptr, nullptr, nullptr, bias.data(), 0, Lk, nullptr, 0,
+                 a.data(), ref_avg.data(), 0);
+        orc_round_bf16(a.data(), a.size());
+        orc_linear(a.data(), wo.data(), nullptr, Lq, C, C, ref.data(), 0);
+        const Err e = compare(ref, download_bf16(out));
+        std::printf("traced cross attn     rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
+        CHECK(within_bf16(e));
+        const std::vector<uint8_t> raw = avg.to_host_bytes();
+        const float* got = reinterpret_cast<const float*>(raw.data());
+        // projected Q / K elements may round the other way on the two sides (one unit in the last place), which moves a
+        // probability by about that fraction
+        bool ok = avg.rows == Lq && avg.cols == Lk;
+        for (size_t i = 0; i < ref_avg.size() && ok; ++i) {
+            ok = std::fabs(static_cast<double>(got[i]) - ref_avg[i]) <= 5e-5 + 2.0 * 0.00390625 * ref_avg[i];
+            if (mask[i % Lk] == 0.f) ok = ok && got[i] == 0.f;
+        }
+        CHECK(ok);
+        CHECK(throws_with([&] { Tensor b2 = Tensor::from_host(bias.data(), Lq, Lk - 1, Dtype::FP32);
+                                bt::cross_attention_forward_with_attn(X, Ctx, Wq, Wk, Wv, Wo, nullptr, &b2, Hc, out, avg); }, "logit_bias must be FP32 (Lq, Lk)"));
+    }
     {   // headnorm + RoPE in one pass, with the prefix rows also written to a cache tensor
         const std::vector<int> axes = {16, 56, 56};
         dit::RopeTables tabs = dit::build_axial_rope_tables(txt, hp, wp, d, axes);

@@ -96,3 +96,44 @@ def test_traced_errors():
         bd.joint_attention_traced(q, q, q, cs, cs, 128, 1, txt_len=40, image_text_bias=z(12, 4, dt=torch.float32))
     with pytest.raises(RuntimeError, match="share shape"):
         bd.joint_attention_traced(q, z(8, 128), q, cs, cs, 128, 1)
+
+
+@pytest.mark.parametrize("dtype,Lq,Lk,C,Cctx,H,with_bias,with_mask", [
+    ("fp16", 1024, 77, 320, 768, 8, True, False),      # SD1.5 level 0 cross attention, traced and steered
+    ("fp16", 256, 77, 640, 768, 8, False, False),      # level 1 (head_dim 80), plain trace
+    ("bf16", 300, 50, 128, 96, 2, True, True),         # ragged sizes, bias and key mask together
+])
+def test_cross_attention_with_attn(oracle, dtype, Lq, Lk, C, Cctx, H, with_bias, with_mask):
+    """bt::cross_attention_forward_with_attn as src/unet_blocks.cpp:282-290 calls it: projections, attention with logit
+    bias / key mask, output projection, head-averaged map."""
+    x, ctx = randn(9501, (Lq, C), dtype), randn(9502, (Lk, Cctx), dtype)
+    wq = oracle.round_to(randn(9503, (C, C), "fp32") / np.sqrt(C), dtype)
+    wk = oracle.round_to(randn(9504, (C, Cctx), "fp32") / np.sqrt(Cctx), dtype)
+    wv = oracle.round_to(randn(9505, (C, Cctx), "fp32") / np.sqrt(Cctx), dtype)
+    wo = oracle.round_to(randn(9506, (C, C), "fp32") / np.sqrt(C), dtype)
+    bias = (randn(9507, (Lq, Lk), "fp32") * 1.5).astype(np.float32) if with_bias else None
+    mask = None
+    if with_mask:
+        mask = np.ones(Lk, np.float32)
+        mask[Lk - 7:] = 0
+        mask[3] = 0
+    d = lambda a: to_dev(a, dtype)
+    out, avg = bd.cross_attention_forward_with_attn(
+        d(x), d(ctx), d(wq), d(wk), d(wv), d(wo), None if mask is None else torch.from_numpy(mask).cuda(),
+        None if bias is None else torch.from_numpy(bias).cuda(), H)
+    q = oracle.round_to(oracle.linear(x, wq), dtype)
+    k = oracle.round_to(oracle.linear(ctx, wk), dtype)
+    v = oracle.round_to(oracle.linear(ctx, wv), dtype)
+    ref_a, ref_avg = oracle.sdpa(q, k, v, H, key_mask=mask, bias=bias, return_attn_avg=True)
+    ref = oracle.linear(oracle.round_to(ref_a, dtype), wo)
+    assert_close(ref, to_np(out), dtype, "cross attention with map: output")
+    got = to_np(avg)
+    # The projected Q and K are rounded to the tensor dtype on both sides, and a sum that lands near a rounding
+    # boundary goes either way: single elements differ by one unit in the last place, which moves a score, and with
+    # it a probability, by about that fraction. (Attention and map alone, on identical Q and K, agree to 1e-6:
+    # test_traced_matches_checker.)
+    unit = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    assert np.all(np.abs(got - ref_avg) <= 5e-5 + 2 * unit * ref_avg)
+    assert np.abs(got.sum(axis=1) - 1.0).max() <= 1e-4
+    if with_mask:
+        assert (got[:, mask == 0] == 0).all()
