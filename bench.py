@@ -137,6 +137,15 @@ def all_configs(torch, bd):
     out["headnorm_rope_4608x24x128_bf16"] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
                                              "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16",
                                              "mbytes": round(nbytes / 1e6, 2)}
+    # measured ceiling for the HBM-bound rows: a device-to-device copy of the size of cfg5b's four streams
+    # (73.4 MB read + 73.4 MB written), by the same timing method
+    csrc = torch.empty(73_400_320, dtype=torch.uint8, device="cuda").fill_(1)
+    cdst = torch.empty_like(csrc)
+    mn, av = event_ms(torch, lambda: cdst.copy_(csrc), 20)
+    copy_gbs = 2 * csrc.numel() / (mn * 1e-3) / 1e9
+    out["hbm_copy_ceiling_147mb"] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(copy_gbs, 1),
+                                     "frac_hbm_peak": round(copy_gbs / PEAK_HBM_GBS, 4)}
+    del csrc, cdst
     for name, n in (("cfg5a_sana_linear_n1024_d112_bf16", 1024), ("cfg5b_sana_linear_n4096_d112_bf16", 4096)):
         ql, kl, vl_ = (rnd(2, n, 2240) for _ in range(3))
         ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
@@ -145,7 +154,8 @@ def all_configs(torch, bd):
         mn, av = event_ms(torch, lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc), 20)
         nbytes = 4 * 2 * n * 2240 * 2
         out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
-                     "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16 in, f32 accumulate",
+                     "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                     "frac_copy_ceiling": round(nbytes / (mn * 1e-3) / 1e9 / copy_gbs, 4), "dtype": "bf16 in, f32 accumulate",
                      "mbytes": round(nbytes / 1e6, 2)}
     return out
 
