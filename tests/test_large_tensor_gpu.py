@@ -77,3 +77,49 @@ def test_keys_beyond_2_31_elements(oracle):
     rows = [0, 1000, Lq - 1]
     ref = oracle.sdpa(to_np(q[rows]), to_np(k0), to_np(v0), H)
     assert_close(ref, to_np(out[rows]), "bf16", "sampled rows against one period of the keys")
+
+
+def test_elementwise_and_rope_beyond_2_31_elements(oracle):
+    """RoPE, head norm + RoPE, row scaling, the two adds and the linear layer on (1 100 000, 2048) = 2.25e9 elements;
+    rows on both sides of element 2^31 against the checker (or plain arithmetic)."""
+    H, d, L = 16, 128, 1_100_000
+    x = _big_randn(L, H * d, 41)
+    rows = [0, 5, (1 << 20) - 1, 1 << 20, (1 << 20) + 7, L - 1]
+    idx = torch.tensor(rows, device="cuda")
+    ang = torch.rand(L, d // 2, device="cuda", generator=torch.Generator(device="cuda").manual_seed(42)) * 6.28
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    xs = to_np(x[idx])
+    unit = 2.0 ** -8
+
+    r = bd.rope_apply(x, cos, sin, d, H)
+    ref = oracle.rope_apply(xs, cos[idx].cpu().numpy(), sin[idx].cpu().numpy(), H, d, round_to_dtype="bf16")
+    assert np.abs(to_np(r[idx]) - ref).max() <= unit * max(1.0, np.abs(ref).max())
+    del r
+
+    gain = oracle.round_to(1 + 0.3 * np.arange(d, dtype=np.float32) / d, "bf16")
+    hn = bd.headnorm_rope(x, torch.from_numpy(gain).cuda().to(torch.bfloat16), 1e-6, cos, sin, d, H)
+    ref = oracle.headnorm_rope(xs, gain, 1e-6, cos[idx].cpu().numpy(), sin[idx].cpu().numpy(), H, d)
+    assert np.all(np.abs(to_np(hn[idx]) - ref) <= unit * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)
+    del hn
+
+    rs = torch.rand(L, 1, device="cuda", generator=torch.Generator(device="cuda").manual_seed(43))
+    sr = bd.scale_rows(x, 0.75, rs)
+    ref = oracle.round_to(xs * (0.75 * rs[idx].cpu().numpy()), "bf16")
+    assert np.abs(to_np(sr[idx]) - ref).max() <= unit * max(1.0, np.abs(ref).max())
+
+    y = sr                                            # reuse the buffer: y += x, then y += bias per row
+    before = to_np(y[idx])
+    bd.add_inplace_vec(y, x)
+    ref = oracle.round_to(before + xs, "bf16")
+    assert np.array_equal(to_np(y[idx]), ref)
+    bias = _big_randn(1, H * d, 44).reshape(H * d)
+    before = to_np(y[idx])
+    bd.add_inplace_row_bias(y, bias)
+    assert np.array_equal(to_np(y[idx]), oracle.round_to(before + to_np(bias)[None, :], "bf16"))
+    del y, sr
+
+    w = (_big_randn(256, H * d, 45) / np.sqrt(H * d)).to(torch.bfloat16)
+    out = bd.linear_batched(w, None, x)               # (1 100 000, 256): the input offsets are the large ones
+    ref = oracle.linear(xs, to_np(w))
+    got = to_np(out[idx])
+    assert np.all(np.abs(got - ref) <= unit * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)
