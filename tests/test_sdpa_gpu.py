@@ -308,3 +308,26 @@ def test_errors():
         bd.flash_attention_forward(q.float(), q.float(), q.float(), None, 2, False)
     with pytest.raises(RuntimeError, match="K and V must be"):
         bd.flash_attention_forward(q, q[:, :128], q, None, 2, False)
+
+
+def test_block_causal_maximum_segment_count(oracle, kernel_choice):
+    """The segment table holds 32 entries: 32 alternating text / image segments of ragged lengths behind a cached
+    prefix, in one launch; one more segment is refused."""
+    dtype, H, d, prefix = "bf16", 2, 64, 37
+    lens = [5 + (7 * i) % 23 + (29 if i % 2 else 0) for i in range(32)]
+    kinds = [("t" if i % 2 == 0 else "i", n) for i, n in enumerate(lens)]
+    L = sum(lens)
+    sq = [int(x) for x in np.cumsum(lens)]
+    sk = [prefix + e for e in sq]
+    sc = [1 if kd == "t" else 0 for kd, _ in kinds]
+    q = randn(301, (L, H * d), dtype); k = randn(302, (L, H * d), dtype); v = randn(303, (L, H * d), dtype)
+    kp = randn(304, (prefix, H * d), dtype); vp = randn(305, (prefix, H * d), dtype)
+    mask = bd.SdpaMask.block_causal(prefix, sq, sk, sc)
+    out = bd.sdpa_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, mask=mask,
+                          k_prefix=to_dev(kp, dtype), v_prefix=to_dev(vp, dtype))
+    lo, hi = oracle.rows_block_causal(L, prefix + L, prefix, sq, sk, sc)
+    ref = oracle.sdpa(q, np.concatenate([kp, k]), np.concatenate([vp, v]), H, row_lo=lo, row_hi=hi)
+    assert_close(ref, to_np(out), dtype, "32 segments")
+    with pytest.raises(RuntimeError, match="segments"):
+        bd.sdpa_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H,
+                        mask=bd.SdpaMask.block_causal(0, sq + [L + 1], sq + [L + 1], sc + [0]))
