@@ -376,12 +376,20 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
                                                  RelSoftmaxState& st, f32x16& neg_ref, bool masked, bool dead_row, int j0, int lo,
                                                  int hi, int lh) {
     if (masked) {
+        // Keys outside [lo, hi) become -inf by integer arithmetic on the lane's own values (the sign of
+        // (key - lo) | (hi - 1 - key) selects the bits of -inf): 32 compares would put 32 lane masks into scalar
+        // registers at once, and the scalars that live through the key loop would be spilled around them.
+        const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                if (key < lo || key >= hi) sacc[kb][e] = kNegInf;
+                const int x = d0 + 32 * kb + 8 * (e >> 2) + (e & 3);
+                const unsigned out = static_cast<unsigned>((x | (top - x)) >> 31);   // all ones when outside
+                const float score = sacc[kb][e];   // a scalar copy first: a bit cast of a vector element expression
+                                                   // reads element 0 for every index with this compiler
+                const unsigned bits = __builtin_bit_cast(unsigned, score);
+                sacc[kb][e] = __builtin_bit_cast(float, (bits & ~out) | (0xff800000u & out));
             }
     }
     auto exponentiate = [&]() -> float {
