@@ -268,6 +268,17 @@ __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsig
     }
 }
 
+// score, or -inf when `x` is outside [0, top] (x = key - lo, top = hi - 1 - lo) or `extra` is negative: the sign of
+// x | (top - x) | extra selects the bits of -inf. Integer arithmetic on the lane's own values on purpose: 32 compares
+// would put 32 lane masks into scalar registers at once, and the scalars that live through the key loop would be
+// spilled around them. (The score is taken by value: a bit cast of a vector element expression reads element 0 for
+// every index with this compiler.)
+__device__ __forceinline__ float blank_outside(float score, int x, int top, int extra = 0) {
+    const unsigned out = static_cast<unsigned>((x | (top - x) | extra) >> 31);   // all ones when blanked
+    const unsigned bits = __builtin_bit_cast(unsigned, score);
+    return __builtin_bit_cast(float, (bits & ~out) | (0xff800000u & out));
+}
+
 // Online-softmax state of one lane (one query row, shared with lane l^32).
 // m is the reference the exponentials are taken against; it is raised only when a tile's maximum
 // exceeds it by more than 2^kLazyLog2, so most tiles skip the rescale of l and O. The result does
@@ -308,17 +319,20 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
                     const f32x4 mk = *reinterpret_cast<const f32x4*>(mask_tile + kbase);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int key = j0 + kbase + i;
-                        if (key < lo || key >= hi || mk[i] == 0.f) sacc[kb][4 * bb + i] = kNegInf;
+                        const float score = sacc[kb][4 * bb + i], mv = mk[i];
+                        // a key-mask value of +-0 hides the key: (bits of |m|) - 1 is negative exactly then
+                        const int hidden = static_cast<int>(__builtin_bit_cast(unsigned, mv) & 0x7fffffffu) - 1;
+                        sacc[kb][4 * bb + i] = blank_outside(score, j0 + kbase + i - lo, hi - 1 - lo, hidden);
                     }
                 }
         } else {
+            const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                    if (key < lo || key >= hi) sacc[kb][e] = kNegInf;
+                    const float score = sacc[kb][e];
+                    sacc[kb][e] = blank_outside(score, d0 + 32 * kb + 8 * (e >> 2) + (e & 3), top);
                 }
         }
     }
@@ -376,20 +390,13 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
                                                  RelSoftmaxState& st, f32x16& neg_ref, bool masked, bool dead_row, int j0, int lo,
                                                  int hi, int lh) {
     if (masked) {
-        // Keys outside [lo, hi) become -inf by integer arithmetic on the lane's own values (the sign of
-        // (key - lo) | (hi - 1 - key) selects the bits of -inf): 32 compares would put 32 lane masks into scalar
-        // registers at once, and the scalars that live through the key loop would be spilled around them.
-        const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;
+        const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;   // keys outside [lo, hi) become -inf
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int x = d0 + 32 * kb + 8 * (e >> 2) + (e & 3);
-                const unsigned out = static_cast<unsigned>((x | (top - x)) >> 31);   // all ones when outside
-                const float score = sacc[kb][e];   // a scalar copy first: a bit cast of a vector element expression
-                                                   // reads element 0 for every index with this compiler
-                const unsigned bits = __builtin_bit_cast(unsigned, score);
-                sacc[kb][e] = __builtin_bit_cast(float, (bits & ~out) | (0xff800000u & out));
+                const float score = sacc[kb][e];
+                sacc[kb][e] = blank_outside(score, d0 + 32 * kb + 8 * (e >> 2) + (e & 3), top);
             }
     }
     auto exponentiate = [&]() -> float {
