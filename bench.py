@@ -26,8 +26,8 @@ sys.path.insert(0, ROOT)
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, published
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --traffic-probe`: (69372 KiB x 2.00 calibration) fetched + 27648 KiB written.
-TRAFFIC_BYTES_PER_LAUNCH = (69372 * 2 + 27648) * 1024
+# `bench.py --traffic-probe`: (69300 KiB x 2.00 calibration) fetched + 27648 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (69300 * 2 + 27648) * 1024
 
 
 def parse():
