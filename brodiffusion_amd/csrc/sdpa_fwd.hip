@@ -604,7 +604,9 @@ template <int D> constexpr int lds_bytes_8() {
 // In the shadow of the stream the wavefront stores its share of tiles K_{t+2}, V_{t+1} into the LDS buffers
 // of K_t, V_{t-1} (last read in step t-1) and issues the global loads of K_{t+3}, V_{t+2}; two buffers per
 // operand suffice.
-template <typename T, int D, bool ROPE_K>
+// DENSE: as in the DMA form below (no mask, no prefix, whole key tiles only); instantiated for head_dim up to 64, where
+// it measures 2-3 % faster (at 80 the compiler's allocation of that instance goes wrong: twice as slow).
+template <typename T, int D, bool ROPE_K, bool DENSE = false>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev p) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
@@ -632,10 +634,13 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
 
-    int lo, hi;
-    row_interval(p, b, qrow, qvalid, lo, hi);
-    const WaveExtent we = wave_extent(lo, hi);
-    if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    int lo = 0, hi = p.Lk;   // DENSE: rows past the end of Q repeat its last row and are never stored
+    if constexpr (!DENSE) row_interval(p, b, qrow, qvalid, lo, hi);
+    WaveExtent we{0, 0, p.Lk, p.Lk};
+    if constexpr (!DENSE) {
+        we = wave_extent(lo, hi);
+        if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
+    }
     V8 qf[G::KC];
     stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid, p.scale_log2);   // Q carries scale * log2(e)
     __syncthreads();
@@ -646,11 +651,14 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     zero_pads<D, kThreads8>(Kbuf, Vbuf, G::K_BYTES, G::V_BYTES, 2, tid);
     for (int i = tid; i < 2 * G::V_BYTES / 16; i += kThreads8) *reinterpret_cast<u32x4*>(Vbuf + i * 16) = u32x4{0, 0, 0, 0};
     __syncthreads();
-    int g_lo = red[0], kv_stop = red[8];
+    int g_lo = 0, kv_stop = p.Lk;
+    if constexpr (!DENSE) {
+        g_lo = red[0]; kv_stop = red[8];
 #pragma unroll
-    for (int w = 1; w < 8; ++w) { g_lo = min(g_lo, red[w]); kv_stop = max(kv_stop, red[8 + w]); }
-    g_lo = __builtin_amdgcn_readfirstlane(g_lo);
-    kv_stop = __builtin_amdgcn_readfirstlane(kv_stop);
+        for (int w = 1; w < 8; ++w) { g_lo = min(g_lo, red[w]); kv_stop = max(kv_stop, red[8 + w]); }
+        g_lo = __builtin_amdgcn_readfirstlane(g_lo);
+        kv_stop = __builtin_amdgcn_readfirstlane(kv_stop);
+    }
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
     const int n_tiles = plan.n_tiles;
 
@@ -714,7 +722,13 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         }
         __syncthreads();
         auto softmax_of = [&](int tt) {
-            if (tile_active(tt)) {
+            if constexpr (DENSE) {
+                if (tt >= 0 && tt < n_tiles) {
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, false, false, 0, 0, p.Lk, lh);
+                    return;
+                }
+            }
+            if (!DENSE && tile_active(tt)) {
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
@@ -1310,6 +1324,9 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
                     if (dense) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false, true>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                     else hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                 }
+            }
+            else if (D <= 64 && p.mask_mode == MI_MASK_NONE && p.kv_valid_len == nullptr && p.Lp == 0 && p.Lk % kBN == 0) {
+                if constexpr (D <= 64) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false, true>), grid, block, lds_bytes_8<D>(), stream, p);
             }
             else hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false>), grid, block, lds_bytes_8<D>(), stream, p);
         }
