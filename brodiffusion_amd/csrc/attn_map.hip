@@ -45,14 +45,19 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) avg[kb][e] = 0.f;
-    // bit 16 kb + e: this lane's key (kb, e) counts (inside the sequence and not masked)
-    unsigned live = 0;
+    // What is added to the scaled score of this lane's key (kb, e), the same for every head, fetched once: the logit
+    // bias in exponent units, 0 without one, -inf for keys past the end of the sequence or hidden by the key mask
+    // (their probability is then 0). The head loop is left with one fused multiply-add per score and no condition.
+    f32x16 pre[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-            if (key < p.Lk && (p.key_mask == nullptr || p.key_mask[key] != 0.f)) live |= 1u << (16 * kb + e);
+            float v = 0.f;
+            if (bias_row && key < p.bias_cols) v = bias_row[key] * kLog2e;
+            if (key >= p.Lk || (p.key_mask != nullptr && p.key_mask[min(key, p.Lk - 1)] == 0.f)) v = kNegInf;
+            pre[kb][e] = v;
         }
 
     const T* const qg = static_cast<const T*>(p.q);
@@ -91,10 +96,7 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int key = j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                float s2 = sacc[kb][e] * p.scale_log2;
-                if (bias_row && key < p.bias_cols) s2 = __builtin_fmaf(bias_row[key], kLog2e, s2);
-                if (live & (1u << (16 * kb + e))) avg[kb][e] += __builtin_amdgcn_exp2f(s2 - lse);
+                avg[kb][e] += __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][e], p.scale_log2, pre[kb][e]) - lse);
             }
         __syncthreads();   // all reads of this head's K tile are done before the next head overwrites it
     }
