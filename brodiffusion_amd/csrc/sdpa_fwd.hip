@@ -956,14 +956,19 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         if constexpr (DG::SWZ) cc ^= swz(row);     // the chunk this slot must receive
         drow[m] = row;
         dcol[m] = static_cast<unsigned>(cc) * 16u;
+        if constexpr (DENSE) {
+            // whole tiles of one segment only: the lane's byte offset inside a tile never changes
+            const bool is_k = DG::NDMA % 8 == 0 ? m < DG::MAXI / 2 : i < DG::NDMA;
+            dcol[m] += static_cast<unsigned>(row) * (static_cast<unsigned>(is_k ? p.k_rs : p.v_rs) * 2u);
+        }
     }
     // One DMA instruction. Written as inline assembly on purpose: for the compiler's builtin every later LDS read may
     // alias the DMA's LDS write, so it waits for the load to land (vmcnt(0)) before the next ds_read. The tiles
     // written here are never read before the explicit wait + barrier at the end of the following step.
     const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)smem));
     auto dma = [&](const TileCursor& c, int m, int j, int lds_off) {
-        const int row = min(drow[m], min(c.rows_left, kBN) - 1);
-        const unsigned voff = static_cast<unsigned>(row) * c.rsb + dcol[m];
+        unsigned voff = dcol[m];
+        if constexpr (!DENSE) voff += static_cast<unsigned>(min(drow[m], min(c.rows_left, kBN) - 1)) * c.rsb;
         const unsigned dst = lds_base + lds_off + j * 1024;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory");
     };
@@ -1056,8 +1061,13 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         // LDS access ahead of it for a long time: right before its softmax.
         auto issue_dma = [&]() {
             issued = dma_tiles(load_k, KD, load_v, VD);
-            if (load_k) kc.next();
-            if (load_v) vc.next();
+            if constexpr (DENSE) {
+                if (load_k) kc.ptr += kBN * kc.rsb;
+                if (load_v) vc.ptr += kBN * vc.rsb;
+            } else {
+                if (load_k) kc.next();
+                if (load_v) vc.next();
+            }
         };
         // group 1 turns the scores of its previous step into P first, so that its MFMA stream meets group 0's softmax
         if (grp == 1) {
