@@ -1,0 +1,37 @@
+"""The dense instances of the 256-row kernels (no mask, no prefix, key count a multiple of 64) on query counts that are
+not a multiple of the tile: the rows past the end repeat the last query row inside the kernel and must not be stored.
+Sampled rows against the CPU checker, the rest against the general instance of the same kernel (reached by passing a
+valid length equal to the key count)."""
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import assert_close, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype,d,H,B,Lq,Lk", [
+    ("bf16", 128, 16, 2, 3999, 4096),     # LDS-DMA kernel
+    ("bf16", 72, 16, 2, 4001, 1024),      # LDS-DMA kernel, head_dim 72
+    ("fp16", 40, 8, 4, 2050, 2048),       # register-staged kernel
+    ("bf16", 64, 16, 2, 3841, 640),
+])
+def test_dense_instance_ragged_queries(oracle, dtype, d, H, B, Lq, Lk):
+    q = randn(601, (B, Lq, H * d), dtype)
+    k = randn(602, (B, Lk, H * d), dtype)
+    v = randn(603, (B, Lk, H * d), dtype)
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    guard = torch.full((B, Lq + 300, H * d), 7.0, device="cuda", dtype=dq.dtype)   # rows behind the output stay untouched
+    out = guard[:, :Lq]
+    bd.sdpa_forward(dq, dk, dv, H, out=out, split_scratch=False)
+    assert (guard[:, Lq:] == 7.0).all()
+    full = torch.tensor([Lk] * B, dtype=torch.int32, device="cuda")
+    general = bd.sdpa_forward(dq, dk, dv, H, kv_valid_len=full, split_scratch=False)
+    unit = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    assert (out.float() - general.float()).abs().max().item() <= unit * max(1.0, general.float().abs().max().item())
+    rows = [0, 255, 256, Lq - 257, Lq - 2, Lq - 1]
+    for b in (0, B - 1):
+        ref = oracle.sdpa(q[b][rows], k[b], v[b], H)
+        assert_close(ref, to_np(out[b][rows]), dtype, f"batch {b}")
