@@ -11,7 +11,7 @@ timed region. Prints ONE JSON line.
               events on the launch stream over the timed region
   cpu_baseline the CPU checker (a port of the reference's FP32/FP64 host attention loop) timed on this
               host's cores on a bounded sample of the same workload
-  configs     ms per call and TFLOP/s (GB/s for linear attention) of every BASELINE config, measured
+  configs     ms per call and TFLOP/s (GB/s for linear attention) of every benchmark configuration, measured
               outside the timed region
 """
 import argparse
@@ -69,7 +69,7 @@ def event_ms(torch, fn, iters, warm=0.05):
 
 
 def all_configs(torch, bd):
-    """Every BASELINE config: ms per call (min and mean over 20 calls), TFLOP/s or GB/s, fraction of peak."""
+    """Every benchmark configuration: ms per call (min and mean over 20 calls), TFLOP/s or GB/s, fraction of peak."""
     g = torch.Generator(device="cuda").manual_seed(1234)
 
     def rnd(*shape, dt=torch.bfloat16):
