@@ -35,3 +35,33 @@ def test_dense_instance_ragged_queries(oracle, dtype, d, H, B, Lq, Lk):
     for b in (0, B - 1):
         ref = oracle.sdpa(q[b][rows], k[b], v[b], H)
         assert_close(ref, to_np(out[b][rows]), dtype, f"batch {b}")
+
+
+@pytest.mark.parametrize("dtype,d,H,Hkv,B,Lq,Lk,axes", [
+    ("bf16", 128, 16, 4, 2, 2304, 2304, (16, 56, 56)),    # LDS-DMA kernel, grouped-query heads, RoPE on Q (on load) and K (scratch)
+    ("fp16", 64, 16, 8, 2, 2304, 2304, (16, 24, 24)),     # register-staged kernel
+])
+def test_dense_instance_gqa_and_rope(oracle, dtype, d, H, Hkv, B, Lq, Lk, axes):
+    """The dense instances with everything that is allowed next to them: fewer key / value heads than query heads and
+    RoPE fused into the Q load, K rotated into a scratch. Sampled rows against the checker."""
+    txt, hp, wp = 256, 32, 64
+    assert txt + hp * wp == Lq == Lk
+    q = randn(611, (B, Lq, H * d), dtype)
+    k = randn(612, (B, Lk, Hkv * d), dtype)
+    v = randn(613, (B, Lk, Hkv * d), dtype)
+    cos, sin = oracle.build_axial_rope_tables(txt, hp, wp, d, axes)
+    dcos, dsin = torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    kr = torch.empty_like(dk)
+    out = bd.sdpa_forward(dq, dk, dv, H, num_kv_heads=Hkv, rope_q=(dcos, dsin), rope_k=(dcos, dsin), rope_k_scratch=kr,
+                          split_scratch=False)
+    rows = [0, 300, Lq - 1]
+    group = H // Hkv
+    for b in (0, B - 1):
+        qr = oracle.rope_apply(q[b][rows], cos[rows], sin[rows], H, d, round_to_dtype=dtype)
+        krr = oracle.rope_apply(k[b], cos, sin, Hkv, d, round_to_dtype=dtype)
+        # widen K / V to one head per query head for the checker
+        kw = np.repeat(krr.reshape(Lk, Hkv, d), group, axis=1).reshape(Lk, H * d)
+        vw = np.repeat(v[b].reshape(Lk, Hkv, d), group, axis=1).reshape(Lk, H * d)
+        ref = oracle.sdpa(qr, kw, vw, H)
+        assert_close(ref, to_np(out[b][rows]), dtype, f"batch {b}")
