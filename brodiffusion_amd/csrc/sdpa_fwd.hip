@@ -813,7 +813,7 @@ __device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2)
 // SPLIT: the launch follows p.split — a work group either processes one whole query tile or one piece of the last
 // round, i.e. one or more (tile, key range) parts in sequence, each leaving a partial result in its scratch slot
 // (merged by sdpa_combine_kernel). Only for unmasked calls without prefix.
-// DENSE: no mask of any kind, no prefix and a key count that is a multiple of 64: every tile is whole and visible to
+// DENSE: no mask of any kind and key counts (cached prefix, if any, and fresh) that are multiples of 64: every tile is whole and visible to
 // every row, so the masked form of the softmax and the per-step bookkeeping (which tile, its limit, whether this
 // wavefront sees it whole) drop out of the kernel, and with them their registers: measured 6 % faster at head_dim 128
 // and 8 % at 72 than the general form on the same dense call.
@@ -892,14 +892,15 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
 
-    int lo = 0, hi = p.Lk;   // DENSE: rows past the end of Q repeat its last row and are never stored
+    const int n_keys = p.Lk;   // counts the cached prefix rows, which come first
+    int lo = 0, hi = n_keys;   // DENSE: rows past the end of Q repeat its last row and are never stored
     if constexpr (!DENSE) row_interval(p, b, qrow, qvalid, lo, hi);
     if constexpr (SPLIT) {
         lo = max(lo, kv_begin);
         hi = min(hi, kv_end);
         if (hi <= lo) { lo = 0; hi = 0; }
     }
-    WaveExtent we{0, 0, p.Lk, p.Lk};
+    WaveExtent we{0, 0, n_keys, n_keys};
     if constexpr (!DENSE) {
         we = wave_extent(lo, hi);
         if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
@@ -915,7 +916,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     for (int i = tid; i < DG::SLACK / 16; i += kThreads8)
         *reinterpret_cast<u32x4*>(smem + kDmaStages * DG::TILE + i * 16) = u32x4{0, 0, 0, 0};
     __syncthreads();
-    int g_lo = 0, kv_stop = p.Lk;
+    int g_lo = 0, kv_stop = n_keys;
     if constexpr (!DENSE) {
         g_lo = red[0]; kv_stop = red[8];
 #pragma unroll
@@ -1041,7 +1042,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
-                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, false, false, 0, 0, p.Lk, lh);
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, false, false, 0, 0, n_keys, lh);
                     return;
                 }
             }
@@ -1061,7 +1062,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         // LDS access ahead of it for a long time: right before its softmax.
         auto issue_dma = [&]() {
             issued = dma_tiles(load_k, KD, load_v, VD);
-            if constexpr (DENSE) {
+            if (DENSE && p.Lp == 0) {
                 if (load_k) kc.ptr += kBN * kc.rsb;
                 if (load_v) vc.ptr += kBN * vc.rsb;
             } else {
@@ -1330,7 +1331,9 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
             if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
             else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
                 if constexpr (dma_kernel_available<D>()) {
-                    const bool dense = p.mask_mode == MI_MASK_NONE && p.kv_valid_len == nullptr && p.Lp == 0 && p.Lk % kBN == 0;
+                    // whole key tiles only; a cached prefix may come first if it is whole tiles too and laid out like K / V
+                    const bool dense = p.mask_mode == MI_MASK_NONE && p.kv_valid_len == nullptr && p.Lk % kBN == 0 &&
+                                       (p.Lp == 0 || (p.Lp % kBN == 0 && p.kp_rs == p.k_rs && p.vp_rs == p.v_rs));
                     if (dense) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false, true>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                     else hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                 }

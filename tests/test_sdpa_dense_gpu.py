@@ -65,3 +65,24 @@ def test_dense_instance_gqa_and_rope(oracle, dtype, d, H, Hkv, B, Lq, Lk, axes):
         vw = np.repeat(v[b].reshape(Lk, Hkv, d), group, axis=1).reshape(Lk, H * d)
         ref = oracle.sdpa(qr, kw, vw, H)
         assert_close(ref, to_np(out[b][rows]), dtype, f"batch {b}")
+
+
+def test_dense_instance_with_cached_prefix(oracle):
+    """The cached step of the Qwen-Image transformer (src/dit/qwenimage21_forward.cpp:599-649): unmasked, queries are
+    the target rows, keys are [cached prefix ; fresh]. With whole tiles on both segments it runs on the dense instance;
+    it must agree with the call on the concatenated keys and with the checker."""
+    dtype, H, d, Lq, Lp = "bf16", 24, 128, 3072, 512
+    q = randn(621, (Lq, H * d), dtype)
+    k = randn(622, (Lq, H * d), dtype); v = randn(623, (Lq, H * d), dtype)
+    kp = randn(624, (Lp, H * d), dtype); vp = randn(625, (Lp, H * d), dtype)
+    dq, dk, dv, dkp, dvp = (to_dev(a, dtype) for a in (q, k, v, kp, vp))
+    out = bd.sdpa_forward(dq, dk, dv, H, k_prefix=dkp, v_prefix=dvp, split_scratch=False)
+    cat = bd.sdpa_forward(dq, torch.cat([dkp, dk]), torch.cat([dvp, dv]), H, split_scratch=False)
+    assert (out.float() - cat.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, cat.float().abs().max().item())
+    rows = [0, 511, 2000, Lq - 1]
+    ref = oracle.sdpa(q[rows], np.concatenate([kp, k]), np.concatenate([vp, v]), H)
+    assert_close(ref, to_np(out[rows]), dtype, "cached prefix, dense instance")
+    # a prefix that is not whole tiles takes the general instance and must give the same rows
+    out2 = bd.sdpa_forward(dq, dk, dv, H, k_prefix=dkp[:500], v_prefix=dvp[:500], split_scratch=False)
+    ref2 = oracle.sdpa(q[rows], np.concatenate([kp[:500], k]), np.concatenate([vp[:500], v]), H)
+    assert_close(ref2, to_np(out2[rows]), dtype, "cached prefix of 500 rows")
