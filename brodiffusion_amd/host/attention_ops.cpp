@@ -372,6 +372,24 @@ void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const
     linear_impl(op, Wo, nullptr, nullptr, w->a, out);
 }
 
+void mha_forward(const Tensor& X, const Tensor& Wq, const Tensor& Wk, const Tensor& Wv, const Tensor& Wo, const Tensor* bq,
+                 const Tensor* bk, const Tensor* bv, const Tensor* bo, const float* d_mask, int num_heads, Tensor& qh,
+                 Tensor& kh, Tensor& vh, Tensor& attn, Tensor& yc, Tensor& out) {
+    const char* op = "mha_forward";
+    (void)attn;
+    need_gpu(op, X);
+    if (num_heads <= 0 || Wq.rows % num_heads != 0) fail(std::string(op) + ": num_heads must divide the projection width");
+    if (Wk.rows != Wq.rows || Wv.rows != Wq.rows || Wo.cols != Wq.rows) fail(std::string(op) + ": Wq, Wk, Wv must project to one width, which Wo takes");
+    linear_impl(op, Wq, nullptr, bq, X, qh);
+    linear_impl(op, Wk, nullptr, bk, X, kh);
+    linear_impl(op, Wv, nullptr, bv, X, vh);
+    mi_sdpa_args a;
+    init_args(a, op, qh, kh, vh, num_heads, num_heads, yc);
+    a.key_mask = d_mask;
+    run_sdpa(op, a);
+    linear_impl(op, Wo, nullptr, bo, yc, out);
+}
+
 }  // namespace bt
 
 void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y) {

@@ -86,6 +86,15 @@ void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const
                                        const Tensor& Wo, const float* d_mask, const Tensor* logit_bias, int num_heads,
                                        Tensor& out, Tensor& AttnAvg);
 
+// Multi-head self attention with the projections around it, as PixArt's self attention calls it on the reference's
+// FP32 path (src/dit/pixart.cpp:325-328): qh = X Wq^T + bq, kh, vh likewise, yc = attention(qh, kh, vh) with the
+// optional key mask, out = yc Wo^T + bo (biases nullable). Here for FP16 / BF16 device tensors, the same four GEMMs
+// and one attention launch as flash_attention_qkvo_forward, with the intermediates in the caller's tensors. The scores
+// are never materialised: `attn` is left as it is.
+void mha_forward(const Tensor& X, const Tensor& Wq, const Tensor& Wk, const Tensor& Wv, const Tensor& Wo, const Tensor* bq,
+                 const Tensor* bk, const Tensor* bv, const Tensor* bo, const float* d_mask, int num_heads, Tensor& qh,
+                 Tensor& kh, Tensor& vh, Tensor& attn, Tensor& yc, Tensor& out);
+
 }  // namespace bt
 
 // The fused helpers of the SD1.5 transformer block, names and argument order of include/brodiffusion/fused_transformer.h:

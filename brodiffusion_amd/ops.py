@@ -774,6 +774,34 @@ def cross_attention_forward_with_attn(X, Ctx, Wq, Wk, Wv, Wo, d_mask, logit_bias
     return out, attn_avg
 
 
+def mha_forward(X, Wq, Wk, Wv, Wo, bq, bk, bv, bo, d_mask, num_heads: int, qh: Optional[torch.Tensor] = None,
+                kh: Optional[torch.Tensor] = None, vh: Optional[torch.Tensor] = None, attn=None,
+                yc: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None):
+    """bt::mha_forward as PixArt's self attention calls it on the reference's FP32 path (src/dit/pixart.cpp:325-328):
+    qh = X Wq^T + bq, kh, vh likewise, yc = attention(qh, kh, vh) with the optional key mask (float32 (L,), 1 = valid),
+    out = yc Wo^T + bo; biases may be None. For float16 / bfloat16 device tensors: four GEMMs and one attention launch,
+    intermediates in the caller's tensors when given. The scores are never materialised, so `attn` is ignored.
+    Returns (out, qh, kh, vh, yc)."""
+    op = "mha_forward"
+    _dev(op, X, Wq, Wk, Wv, Wo, bq, bk, bv, bo, d_mask, qh, kh, vh, yc, out)
+    if X.dim() != 2:
+        _fail(op, "X must be 2-D (rows, channels)")
+    L, inner = X.shape[0], Wq.shape[0]
+    if num_heads <= 0 or inner % num_heads != 0:
+        _fail(op, "num_heads must divide the projection width")
+    if Wk.shape[0] != inner or Wv.shape[0] != inner or Wo.shape[1] != inner:
+        _fail(op, "Wq, Wk, Wv must project to one width, which Wo takes")
+    if d_mask is not None and (d_mask.dtype != torch.float32 or d_mask.numel() != L):
+        _fail(op, "d_mask must be float32 (L,)")
+    qh = linear_batched(Wq, bq, X, qh, op=op)
+    kh = linear_batched(Wk, bk, X, kh, op=op)
+    vh = linear_batched(Wv, bv, X, vh, op=op)
+    mask = None if d_mask is None else d_mask.reshape(L).contiguous()
+    yc = sdpa_forward(qh, kh, vh, num_heads, out=yc, key_mask=mask, op=op)
+    out = linear_batched(Wo, bo, yc, out, op=op)
+    return out, qh, kh, vh, yc
+
+
 def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num_kv_heads: int, d_mask,
                          out: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
     """Bidirectional grouped-query attention with optional RoPE and key-padding mask

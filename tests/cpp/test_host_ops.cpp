@@ -367,6 +367,29 @@ static void gpu_checks() {
         const Err e = compare(ref, download_bf16(out));
         std::printf("qkvo cross attention  rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
+        {   // mha_forward (src/dit/pixart.cpp:325-328): self attention with biased projections, intermediates visible
+            const std::vector<float> bq = randn_bf16(7121, C), bk = randn_bf16(7122, C), bv = randn_bf16(7123, C);
+            std::vector<float> km(Lx, 1.f);
+            km[5] = 0.f; km[Lx - 1] = 0.f;
+            Tensor Bq = upload_bf16(bq, 1, C), Bk = upload_bf16(bk, 1, C), Bv = upload_bf16(bv, 1, C),
+                   M = Tensor::from_host(km.data(), 1, Lx, Dtype::FP32), Wks = upload_bf16(wq, C, C), qh, kh, vh, attn, yc, mo;
+            bt::mha_forward(X, Wq, Wks, Wo, Wo, &Bq, &Bk, &Bv, &Bo, static_cast<const float*>(M.data), Hh, qh, kh, vh, attn, yc, mo);
+            const std::vector<float> mq = lin(x, wq, bq.data(), Lx, C, C, true), mk = lin(x, wq, bk.data(), Lx, C, C, true),
+                                     mvv = lin(x, wo, bv.data(), Lx, C, C, true);
+            CHECK(within_bf16(compare(mq, download_bf16(qh))));
+            CHECK(within_bf16(compare(mk, download_bf16(kh))));
+            CHECK(within_bf16(compare(mvv, download_bf16(vh))));
+            std::vector<float> ma(mq.size());
+            orc_sdpa(mq.data(), mk.data(), mvv.data(), Lx, Lx, Hh, C / Hh, -1.0, km.data(), nullptr, nullptr, nullptr, nullptr, 0, 0, nullptr, 0, ma.data(), nullptr, 0);
+            orc_round_bf16(ma.data(), ma.size());
+            CHECK(within_bf16(compare(ma, download_bf16(yc))));
+            const Err em = compare(lin(ma, wo, bo.data(), Lx, C, C, false), download_bf16(mo));
+            std::printf("mha_forward           rel_l2=%.3e max_abs=%.3e\n", em.rel_l2, em.max_abs);
+            CHECK(within_bf16(em));
+            CHECK(attn.data == nullptr);   // scores are never materialised
+            CHECK(throws_with([&] { bt::mha_forward(X, Wq, Wks, Wo, Wo, nullptr, nullptr, nullptr, nullptr, nullptr, 7, qh, kh, vh, attn, yc, mo); },
+                              "num_heads must divide"));
+        }
         // K/V cache filled once, then the cached form: same kernels, same bits
         Tensor Kc, Vc, out2, own_scratch;
         bt::flash_attention_project_kv(Ctx, Wk, nullptr, Wv, nullptr, Kc, Vc);

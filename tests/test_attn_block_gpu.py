@@ -125,6 +125,42 @@ def test_qkvo_self_attention(oracle, dtype, B, L, C, H, biases):
     assert torch.equal(parts, out)
 
 
+@pytest.mark.parametrize("dtype,L,C,H,with_mask", [("fp16", 1024, 1152, 16, False), ("bf16", 300, 144, 2, True)])
+def test_mha_forward(oracle, dtype, L, C, H, with_mask):
+    """bt::mha_forward as PixArt's self attention calls it (src/dit/pixart.cpp:325-328: 16 heads of 72, biases on all
+    four projections): every intermediate against the checker, and the whole against flash_attention_qkvo_forward."""
+    x = randn(7300 + L, (L, C), dtype)
+    ws = block_weights(7400 + C, C, C, C, dtype, True)
+    d = dev(ws, dtype)
+    mask = None
+    if with_mask:
+        mask = np.ones(L, np.float32)
+        mask[L - 11:] = 0
+        mask[2] = 0
+    dmask = None if mask is None else torch.from_numpy(mask).cuda()
+    out, qh, kh, vh, yc = bd.mha_forward(to_dev(x, dtype), d["wq"], d["wk"], d["wv"], d["wo"], d["bq"], d["bk"], d["bv"], d["bo"],
+                                         dmask, H)
+    q = oracle.round_to(oracle.linear(x, ws["wq"], ws["bq"]), dtype)
+    k = oracle.round_to(oracle.linear(x, ws["wk"], ws["bk"]), dtype)
+    v = oracle.round_to(oracle.linear(x, ws["wv"], ws["bv"]), dtype)
+    assert_close(q, to_np(qh), dtype, "mha qh")
+    assert_close(k, to_np(kh), dtype, "mha kh")
+    assert_close(v, to_np(vh), dtype, "mha vh")
+    a = oracle.round_to(oracle.sdpa(q, k, v, H, key_mask=mask), dtype)
+    assert_close(a, to_np(yc), dtype, "mha yc")
+    print("mha_forward", dtype, L, C, assert_close(oracle.linear(a, ws["wo"], ws["bo"]), to_np(out), dtype, "mha out"))
+    fused = bd.flash_attention_qkvo_forward(to_dev(x, dtype), None, d["wq"], d["bq"], d["wk"], d["bk"], d["wv"], d["bv"],
+                                            d["wo"], d["bo"], dmask, H, False)
+    assert torch.equal(fused, out)
+    # caller-owned intermediates are written in place
+    own = [torch.empty(L, C, dtype=TORCH_DT[dtype], device="cuda") for _ in range(5)]
+    res = bd.mha_forward(to_dev(x, dtype), d["wq"], d["wk"], d["wv"], d["wo"], d["bq"], d["bk"], d["bv"], d["bo"], dmask, H,
+                         qh=own[0], kh=own[1], vh=own[2], yc=own[3], out=own[4])
+    assert res[0].data_ptr() == own[4].data_ptr() and torch.equal(own[4], out) and torch.equal(own[3], yc)
+    with pytest.raises(RuntimeError, match="num_heads must divide"):
+        bd.mha_forward(to_dev(x, dtype), d["wq"], d["wk"], d["wv"], d["wo"], None, None, None, None, None, 7)
+
+
 @pytest.mark.parametrize("dtype,B,L,C,H", [("fp16", 2, 4096, 320, 8), ("bf16", 1, 1024, 640, 8), ("fp16", 1, 64, 1280, 8)])
 def test_qkvo_cross_attention_and_kv_cache(oracle, dtype, B, L, C, H):
     Lc, Cc = 77, 768
