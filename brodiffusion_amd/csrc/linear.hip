@@ -52,8 +52,7 @@ template <int ROWS, bool GATED = false>
 __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
                                           int k0, int K, int tid) {
     const int kc = k0 + (tid & 7) * 8;
-    const bool k_ok = kc < K;
-    const long col = k_ok ? kc : 0;
+    const long col = kc < K ? kc : 0;   // chunks past the end of the contraction are blanked when they are stored
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
         int row;
@@ -61,42 +60,44 @@ __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* bas
         else row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);  // rows past the end repeat the last one; never stored
         r[i] = *reinterpret_cast<const u32x4*>(base + (static_cast<long>(row) * ld + col) * 2);
     }
-    if (!k_ok) {
-#pragma unroll
-        for (int i = 0; i < ROWS / 32; ++i) r[i] = u32x4{0u, 0u, 0u, 0u};
-    }
 }
 // INT8 weight tile: the same 8 contraction elements per thread and row are 8 bytes in memory; they are widened to T
 // (exactly: |w| <= 128) on their way to LDS, the per-row scale is applied to the accumulator in the epilogue.
-template <typename T, int ROWS>
-__device__ __forceinline__ void load_tile_int8(u32x4 (&r)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
+template <int ROWS>
+__device__ __forceinline__ void load_tile_int8(u32x2 (&raw)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
                                                int k0, int K, int tid) {
-    typedef T t8 __attribute__((ext_vector_type(8)));
-    typedef signed char c8 __attribute__((ext_vector_type(8)));
     const int kc = k0 + (tid & 7) * 8;
-    const bool k_ok = kc < K;
-    const long col = k_ok ? kc : 0;
-    u32x2 raw[ROWS / 32];
+    const long col = kc < K ? kc : 0;
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
         const int row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);
         raw[i] = *reinterpret_cast<const u32x2*>(base + static_cast<long>(row) * ld + col);
     }
+}
+
+// Registers -> LDS. Nothing touches the loaded registers before this point, so the wait for the loads sits here,
+// behind the MFMAs of the tile that is in LDS, and not where the loads are issued (blanking the chunks past the end
+// of the contraction, or widening the weight bytes, right after the load made every step wait out the full memory
+// latency before its first MFMA). k_ok: the thread's 8 contraction elements lie inside K.
+template <int ROWS>
+__device__ __forceinline__ void store_tile(const u32x4 (&r)[ROWS / 32], char* lds, int tid, bool k_ok) {
+#pragma unroll
+    for (int i = 0; i < ROWS / 32; ++i)
+        *reinterpret_cast<u32x4*>(lds + ((tid >> 3) + 32 * i) * kRowBytes + (tid & 7) * 16) = k_ok ? r[i] : u32x4{0u, 0u, 0u, 0u};
+}
+template <typename T, int ROWS>
+__device__ __forceinline__ void store_tile_int8(const u32x2 (&raw)[ROWS / 32], char* lds, int tid, bool k_ok) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    typedef signed char c8 __attribute__((ext_vector_type(8)));
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
         const c8 q = __builtin_bit_cast(c8, raw[i]);
         t8 w;
 #pragma unroll
         for (int e = 0; e < 8; ++e) w[e] = static_cast<T>(static_cast<float>(q[e]));
-        r[i] = k_ok ? __builtin_bit_cast(u32x4, w) : u32x4{0u, 0u, 0u, 0u};
+        *reinterpret_cast<u32x4*>(lds + ((tid >> 3) + 32 * i) * kRowBytes + (tid & 7) * 16) =
+            k_ok ? __builtin_bit_cast(u32x4, w) : u32x4{0u, 0u, 0u, 0u};
     }
-}
-
-template <int ROWS>
-__device__ __forceinline__ void store_tile(const u32x4 (&r)[ROWS / 32], char* lds, int tid) {
-#pragma unroll
-    for (int i = 0; i < ROWS / 32; ++i)
-        *reinterpret_cast<u32x4*>(lds + ((tid >> 3) + 32 * i) * kRowBytes + (tid & 7) * 16) = r[i];
 }
 
 // GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
@@ -134,12 +135,26 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    u32x4 xr[BM / 32], wr[BN / 32];
-    load_tile<BM>(xr, xg, p.ldx, m0, p.M, 0, p.K, tid);
-    if constexpr (W8) load_tile_int8<T, BN>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
-    else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, 0, p.K, tid);
-    store_tile<BM>(xr, lds, tid);
-    store_tile<BN>(wr, lds + X_BYTES, tid);
+    // While tile t is multiplied out of LDS, tile t + 1 is on its way into registers; it goes to the other LDS buffer at
+    // the end of the step. (The loads stay under `if (more)`: issued unconditionally, the compiler sinks them behind
+    // the MFMAs, next to the store, and the step waits out the memory latency again. A second register set, two tiles
+    // ahead, and 256 x 256 tiles with 8 wavefronts measured no faster.)
+    u32x4 xr[BM / 32];
+    u32x4 wr[W8 ? 1 : BN / 32];
+    u32x2 wr8[W8 ? BN / 32 : 1];
+    auto load_tiles = [&](int k0) {
+        load_tile<BM>(xr, xg, p.ldx, m0, p.M, k0, p.K, tid);
+        if constexpr (W8) load_tile_int8<BN>(wr8, wg, p.ldw, n0, p.N, k0, p.K, tid);
+        else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, k0, p.K, tid);
+    };
+    auto store_tiles = [&](char* dst, int k0) {
+        const bool k_ok = k0 + (tid & 7) * 8 < p.K;
+        store_tile<BM>(xr, dst, tid, k_ok);
+        if constexpr (W8) store_tile_int8<T, BN>(wr8, dst + X_BYTES, tid, k_ok);
+        else store_tile<BN>(wr, dst + X_BYTES, tid, k_ok);
+    };
+    load_tiles(0);
+    store_tiles(lds, 0);
     __syncthreads();
 
     const int n_steps = (p.K + kBK - 1) / kBK;
@@ -147,11 +162,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
         const char* cur = lds + (t & 1) * (X_BYTES + W_BYTES);
         char* nxt = lds + ((t + 1) & 1) * (X_BYTES + W_BYTES);
         const bool more = t + 1 < n_steps;
-        if (more) {
-            load_tile<BM>(xr, xg, p.ldx, m0, p.M, (t + 1) * kBK, p.K, tid);
-            if constexpr (W8) load_tile_int8<T, BN>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
-            else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, (t + 1) * kBK, p.K, tid);
-        }
+        if (more) load_tiles((t + 1) * kBK);
         const char* xs = cur + (wm * TM * 32 + lq) * kRowBytes + lh * 16;
         const char* ws = cur + X_BYTES + (wn * TN * 32 + lq) * kRowBytes + lh * 16;
 #pragma unroll
@@ -166,10 +177,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
 #pragma unroll
                 for (int b = 0; b < TM; ++b) acc[a][b] = M::run(wf[a], xf[b], acc[a][b]);
         }
-        if (more) {
-            store_tile<BM>(xr, nxt, tid);
-            store_tile<BN>(wr, nxt + X_BYTES, tid);
-        }
+        if (more) store_tiles(nxt, (t + 1) * kBK);
         __syncthreads();
     }
 
