@@ -210,7 +210,7 @@ struct NoMid { __device__ __forceinline__ void operator()() const {} };
 template <typename T, int D, bool DO_PV, bool DO_QK, typename Mid = NoMid>
 __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsigned char* Ks, const typename Mma<T>::v8 (&pf)[4],
                                             const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid(), const f32x16* s_init = nullptr) {
+                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid()) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
     constexpr int NPV = DO_PV ? 4 * G::VB : 0;
@@ -252,9 +252,8 @@ __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsig
             const int k = i - NPV;
             const int kb = k / G::KC, c = k % G::KC;
             if (c == 0) {
-                // the score accumulator starts from zero, or from the caller's vector (minus the row's softmax reference)
                 const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                sacc[kb] = Mma<T>::run(a, qf[c], s_init ? *s_init : zero);
+                sacc[kb] = Mma<T>::run(a, qf[c], zero);
             } else {
                 sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
             }
@@ -370,24 +369,25 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
         for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
 }
 
-// Softmax step for scores that leave the matrix pipe in exponent units and relative to the row's reference: Q carries
-// scale * log2(e), and the first K Q^T MFMA of a key block starts from an accumulator filled with -ref (`neg_ref`, the
-// same value in all 16 slots), so P = exp2(S) needs no further arithmetic and the usual tile maximum is not computed at
-// all. Per 64-key tile and lane that is 32 v_exp, 32 adds and 16 packs instead of ~150 VALU instructions.
+// Softmax step of the 256-row kernels: the exponent of a term is formed by ONE fused multiply-add on the raw FP32 score,
+// x = s * (scale * log2 e) - ref, against a per-row reference that is not the running maximum, so the usual tile maximum
+// is not computed at all: per 64-key tile and lane 32 v_fma, 32 v_exp, 32 adds and 16 packs. Q, K and the scores are
+// untouched by the scale (it multiplies the FP32 accumulator, never a 16-bit operand).
 //   * The reference of a row is the maximum of its first tile with a visible key (then its largest term is 1, so the
 //     denominator stays >= 1), and is raised to a later tile's maximum only when that tile's terms get large (lane sum
 //     above 2^10, or overflow). Any reference gives the same softmax; these two rules keep every term within FP32 / T range.
 //   * Both cases, and rows that have not seen a key yet, take the slow path below (wave-uniform branch): row maximum,
-//     shift of l, O and the scores, new exponentials. Lanes l and l^32 share a row and decide from row-wide values only.
+//     shift of l, O and the reference, new exponentials. Lanes l and l^32 share a row and decide from row-wide values only.
 struct RelSoftmaxState {
     float l = 0.f;          // this lane's share of the denominator
+    float neg_ref = 0.f;    // minus the row's reference, in exponent (base-2) units
     bool started = false;   // the row has a reference (it has seen a visible key)
 };
 constexpr float kRelSumMax = 1024.f;
 
 template <typename T, int D>
 __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                                 RelSoftmaxState& st, f32x16& neg_ref, bool masked, bool dead_row, int j0, int lo,
+                                                 RelSoftmaxState& st, float cl2, bool masked, bool dead_row, int j0, int lo,
                                                  int hi, int lh) {
     if (masked) {
         const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;   // keys outside [lo, hi) become -inf
@@ -401,13 +401,14 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
     }
     auto exponentiate = [&]() -> float {
         float s0 = 0.f, s1 = 0.f;
+        const float nr = st.neg_ref;
         // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
 #pragma unroll
         for (int c4 = 0; c4 < 4; ++c4)
 #pragma unroll
             for (int t = 0; t < 8; t += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t]);
-                const float p1 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t + 1]);
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c4 >> 1][8 * (c4 & 1) + t], cl2, nr));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c4 >> 1][8 * (c4 & 1) + t + 1], cl2, nr));
                 pf[c4][t] = static_cast<T>(p0);
                 pf[c4][t + 1] = static_cast<T>(p1);
                 s0 += p0;
@@ -423,8 +424,10 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
         for (int e = 1; e < 16; ++e) mloc = fmaxf(mloc, fmaxf(sacc[0][e], sacc[1][e]));
         mloc = exchange_max(mloc);
         const bool visible = mloc > kNegInf;
-        // a started row only ever moves its reference up (its terms then stay <= 1)
-        const float shift = !visible ? 0.f : (st.started ? fmaxf(mloc, 0.f) : mloc);
+        // the tile's largest exponent against the present reference; a started row only ever moves its reference up
+        // (its terms then stay <= 1)
+        const float top_x = __builtin_fmaf(mloc, cl2, st.neg_ref);
+        const float shift = !visible ? 0.f : (st.started ? fmaxf(top_x, 0.f) : top_x);
         const float alpha = st.started ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // nothing accumulated before the first key
         st.started = st.started || visible;
         st.l *= alpha;
@@ -432,12 +435,7 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
         for (int vb = 0; vb < HeadGeo<D>::VB; ++vb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[vb][e] *= alpha;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            sacc[0][e] -= shift;
-            sacc[1][e] -= shift;
-            neg_ref[e] -= shift;
-        }
+        st.neg_ref -= shift;
         ls = exponentiate();
     }
     st.l += ls;

@@ -642,7 +642,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
     }
     V8 qf[G::KC];
-    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid, p.scale_log2);   // Q carries scale * log2(e)
+    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid);
     __syncthreads();
     read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
     __syncthreads();
@@ -669,9 +669,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
     RelSoftmaxState st;
     const bool dead_row = hi <= lo;
-    f32x16 neg_ref;   // minus the row's softmax reference in all 16 slots: accumulator start of every score block
-#pragma unroll
-    for (int e = 0; e < 16; ++e) neg_ref[e] = 0.f;
+    const float cl2 = p.scale_log2;
 
     TileMover<T, D, kThreads8, ROPE_K> mv{p, plan,
                                           reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D),
@@ -724,7 +722,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
-                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, false, false, 0, 0, p.Lk, lh);
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, false, false, 0, 0, p.Lk, lh);
                     return;
                 }
             }
@@ -732,7 +730,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -750,7 +748,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
             // movement rides along in the stream (measured faster than in front of the softmax: the stores
             // and loads issue in the shadow of the matrix pipe).
             mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
-                                          [&]() { advance_tiles(t + 2, t + 1); }, &neg_ref);
+                                          [&]() { advance_tiles(t + 2, t + 1); });
             if (grp == 0) {
                 MI_SCHED_BARRIER
                 softmax_of(t + 1);
@@ -906,7 +904,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
     }
     V8 qf[G::KC];
-    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid, p.scale_log2);   // Q carries scale * log2(e)
+    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid);
     __syncthreads();
     read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
     __syncthreads();
@@ -934,9 +932,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
     RelSoftmaxState st;
     const bool dead_row = hi <= lo;
-    f32x16 neg_ref;   // minus the row's softmax reference in all 16 slots: accumulator start of every score block
-#pragma unroll
-    for (int e = 0; e < 16; ++e) neg_ref[e] = 0.f;
+    const float cl2 = p.scale_log2;
 
     // ── DMA duty of this wavefront: instructions i = wave, wave + 8, ... of the list [K 0..NDMA-1, V 0..NDMA-1];
     //    instruction j of an operand fills LDS bytes [1024 j, 1024 j + 1024) of the tile = chunks 64 j + lane ──
@@ -971,7 +967,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         unsigned voff = dcol[m];
         if constexpr (!DENSE) voff += static_cast<unsigned>(min(drow[m], min(c.rows_left, kBN) - 1)) * c.rsb;
         const unsigned dst = lds_base + lds_off + j * 1024;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory", "m0");
     };
     // this wavefront's share of the loads of one K tile (if do_k) and one V tile (if do_v); returns how many it issued
     auto dma_tiles = [&](bool do_k, int k_off, bool do_v, int v_off) -> int {
@@ -1042,7 +1038,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
-                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, false, false, 0, 0, n_keys, lh);
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, false, false, 0, 0, n_keys, lh);
                     return;
                 }
             }
@@ -1050,7 +1046,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, neg_ref, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -1108,7 +1104,8 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                     const int k = i - NPV;
                     const int kb = k / G::KC, c = k % G::KC;
                     if (c == 0) {
-                        sacc[kb] = Mma<T>::run(a, qf[c], neg_ref);
+                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        sacc[kb] = Mma<T>::run(a, qf[c], zero);
                     } else {
                         sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
                     }
@@ -1170,7 +1167,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             write_output<T, D, kThreads8>(smem, reinterpret_cast<T*>(part), D, 0, min(BM, p.Lq - q0), BM, tid);
             if (lh == 0) {
                 float* stat = reinterpret_cast<float*>(part + static_cast<long>(BM) * D * 2);
-                stat[wave * 32 + lq] = -neg_ref[0];
+                stat[wave * 32 + lq] = -st.neg_ref;
                 stat[BM + wave * 32 + lq] = l_tot;
             }
         }
@@ -1244,6 +1241,8 @@ bool plan_split(SdpaDev& p, int n_cu) {
     p.split = SplitGeo{};
     if constexpr (!dma_kernel_available<D>()) return false;
     if (p.mask_mode != MI_MASK_NONE || p.kv_valid_len || p.key_mask || p.Lp > 0 || p.cos_k || p.cu_q) return false;
+    // the logit bias and the softmax denominators exist in the 128-row kernel only
+    if (p.bias != nullptr || p.lse != nullptr) return false;
     if (n_cu < 8 || n_cu % 8 != 0 || sdpa_kernel_choice() == 1 || sdpa_kernel_choice() == 3) return false;
     const long tiles = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int T = (p.Lk + kBN - 1) / kBN;

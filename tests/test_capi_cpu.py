@@ -96,6 +96,26 @@ def test_argument_validation_without_launch(capi):
     assert lib.mi_linear_attn_scratch_bytes(2, 20, 112) % lib.mi_linear_attn_workspace_bytes(2, 20, 112) == 0
 
 
+def test_split_scratch_is_not_offered_to_calls_the_split_kernel_cannot_serve(capi):
+    """The key-axis split of the last round exists in one kernel form only, which neither adds a logit bias nor writes
+    the softmax denominators: a call that asks for either must be told 0 bytes, so that no host layer lends a scratch
+    and sends it down that route. (No GPU: the planner assumes 256 compute units.)"""
+    lib = capi.lib()
+    a = capi.MiSdpaArgs()
+    a.struct_size = C.sizeof(capi.MiSdpaArgs)
+    a.dtype, a.batch, a.num_heads, a.head_dim, a.q_len, a.kv_len = capi.MI_DTYPE_BF16, 1, 24, 128, 2816, 2816
+    a.q = a.k = a.v = a.o = 0x1000                  # never dereferenced: only the launch geometry is planned
+    plain = lib.mi_sdpa_split_scratch_bytes(C.byref(a))
+    assert plain > 0
+    a.lse_out = 0x2000
+    assert lib.mi_sdpa_split_scratch_bytes(C.byref(a)) == 0
+    a.lse_out = None
+    a.logit_bias, a.bias_q0, a.bias_cols = 0x3000, 512, 512
+    assert lib.mi_sdpa_split_scratch_bytes(C.byref(a)) == 0
+    a.logit_bias = None
+    assert lib.mi_sdpa_split_scratch_bytes(C.byref(a)) == plain
+
+
 def test_python_mirror_refuses_cpu_tensors():
     import torch
     import brodiffusion_amd as bd

@@ -1,0 +1,158 @@
+"""Softmax attention on peaked and growing logits, against the CPU checker, through the C ABI.
+
+Seeded N(0,1) inputs give scores of unit spread: every key of a row then lies within a few units of the row maximum and
+the exponentials never leave a narrow range. Real activations are not like that (the reference notes PixArt's un-normed
+cross-attention query reaching +-300 and FP16 scores overflowing, src/dit/pixart.cpp:359-365), so these cases drive the
+softmax of every kernel form through what unit-spread inputs never reach:
+  * queries scaled by 4, 8, 16 (nearly one-hot rows, where a small error in a score moves weight between the top keys);
+  * a score ramp along the key axis, every 64-key tile more than 2^10 above the previous one (a running reference that
+    was fixed by the first tile must be raised again and again);
+  * rows whose first key tiles are masked and whose first visible tile is already large;
+  * one dominant key (closed form: the output is that key's V row);
+  * +-300 queries against a few hundred keys with a valid length (the PixArt cross-attention shape).
+The bound is the one of every other parity test (helpers.TOL); the checker follows src/dit/common.cpp:269-293.
+
+V is N(0,1) / 4 here. A nearly one-hot row returns single V rows, so with unit-variance V the outputs reach magnitude 4,
+where the 16-bit output format itself rounds by up to 1.6e-2 (bf16, half a unit in the last place): the absolute bound of
+2e-2 would then measure the storage format. At a quarter of that the outputs stay near 1, like the outputs of the
+unit-spread cases the bound was stated for; the relative bound does not depend on the scale of V at all.
+"""
+import numpy as np
+import pytest
+import torch
+
+import brodiffusion_amd as bd
+from helpers import assert_close, randn, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+KERNELS = {"auto": 0, "rows128": 1, "rows256": 2, "rows256_regs": 3}
+
+
+@pytest.fixture(autouse=True, params=list(KERNELS))
+def kernel_choice(request):
+    bd.set_sdpa_kernel_choice(KERNELS[request.param])
+    yield request.param
+    bd.set_sdpa_kernel_choice(0)
+
+
+def _values(seed, shape, dtype):
+    return randn(seed, shape, dtype) * np.float32(0.25)      # a power of two: still representable
+
+
+def _run(q, k, v, H, dtype, **kw):
+    return to_np(bd.sdpa_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, **kw))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("d", [40, 72, 128])
+@pytest.mark.parametrize("qmul", [4.0, 8.0, 16.0])
+def test_scaled_queries_dense(oracle, d, dtype, qmul):
+    """Whole key tiles, no mask: the dense kernel instances."""
+    H, Lq, Lk = 2, 300, 640
+    q = randn(100 + d, (Lq, H * d), dtype) * np.float32(qmul)      # a power of two: still representable
+    k = randn(200 + d, (Lk, H * d), dtype); v = _values(300 + d, (Lk, H * d), dtype)
+    assert_close(oracle.sdpa(q, k, v, H), _run(q, k, v, H, dtype), dtype, f"d={d} q x{qmul}")
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72), ("fp16", 64)])
+@pytest.mark.parametrize("qmul", [4.0, 16.0])
+def test_scaled_queries_masked(oracle, d, dtype, qmul):
+    """Causal with a window and a ragged key count: the masked softmax of the general instances; rows deep in the sequence
+    have their first tiles masked, so their reference is set by a later tile."""
+    H, Lq, Lk, window = 2, 280, 470, 150
+    q = randn(110 + d, (Lq, H * d), dtype) * np.float32(qmul)
+    k = randn(210 + d, (Lk, H * d), dtype); v = _values(310 + d, (Lk, H * d), dtype)
+    lo, hi = oracle.rows_causal(Lq, Lk, window=window)
+    out = _run(q, k, v, H, dtype, mask=bd.SdpaMask.causal(Lk - Lq, window))
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), out, dtype, f"d={d} q x{qmul} windowed")
+    vl = torch.tensor([333], dtype=torch.int32, device="cuda")
+    out = _run(q, k, v, H, dtype, kv_valid_len=vl)
+    assert_close(oracle.sdpa(q, k[:333], v[:333], H), out, dtype, f"d={d} q x{qmul} valid_len")
+
+
+def _ramp_inputs(d, dtype, Lq, Lk, H, step, descending=False):
+    """Column 0 of every head: 8 in Q, step * (tile index) in K, so the scores of key tile t sit 8 * step * t * scale above
+    (or, descending, below) those of tile 0, on top of the unit-spread part from the other columns."""
+    q = randn(120 + d, (Lq, H * d), dtype); k = randn(220 + d, (Lk, H * d), dtype); v = _values(320 + d, (Lk, H * d), dtype)
+    tiles = np.arange(Lk) // 64
+    if descending:
+        tiles = tiles.max() - tiles
+    for h in range(H):
+        q[:, h * d] = 8.0
+        k[:, h * d] = (step * tiles).astype(np.float32)     # multiples of `step` below 128 * step: representable
+    return q, k, v
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 128), ("bf16", 72), ("fp16", 40), ("bf16", 64)])
+@pytest.mark.parametrize("descending", [False, True])
+def test_score_ramp_over_key_tiles(oracle, d, dtype, descending):
+    H, Lq, Lk = 2, 270, 768
+    step = 16.0 if d >= 64 else 8.0
+    # tile-to-tile rise in base-2 exponent units: 8 * step / sqrt(d) * log2(e) > 10
+    assert 8 * step / np.sqrt(d) * 1.4427 > 10
+    q, k, v = _ramp_inputs(d, dtype, Lq, Lk, H, step, descending)
+    assert_close(oracle.sdpa(q, k, v, H), _run(q, k, v, H, dtype), dtype, f"d={d} ramp")
+    # the same through the masked instances (ragged valid length cuts the last tile)
+    vl = torch.tensor([Lk - 29], dtype=torch.int32, device="cuda")
+    assert_close(oracle.sdpa(q, k[:Lk - 29], v[:Lk - 29], H), _run(q, k, v, H, dtype, kv_valid_len=vl), dtype, f"d={d} ramp, valid_len")
+    lo, hi = oracle.rows_causal(Lq, Lk)
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), _run(q, k, v, H, dtype, mask=bd.SdpaMask.causal(Lk - Lq)), dtype,
+                 f"d={d} ramp, causal")
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 72), ("bf16", 40)])
+def test_first_visible_tile_is_huge(oracle, d, dtype):
+    """Windowed causal rows: the later rows see nothing of the first key tiles (their window starts past key 192), and
+    the tile many of them start in (keys 192-255, K scaled by 4) carries scores far above everything that follows."""
+    H, Lq, Lk, window = 2, 256, 512, 200
+    q = randn(130 + d, (Lq, H * d), dtype) * np.float32(8.0)
+    k = randn(230 + d, (Lk, H * d), dtype); v = _values(330 + d, (Lk, H * d), dtype)
+    k[192:256] *= np.float32(4.0)
+    lo, hi = oracle.rows_causal(Lq, Lk, window=window)
+    out = _run(q, k, v, H, dtype, mask=bd.SdpaMask.causal(Lk - Lq, window))
+    assert_close(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), out, dtype, f"d={d}")
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72)])
+@pytest.mark.parametrize("jdom", [5, 200, 447])
+def test_one_dominant_key(oracle, d, dtype, jdom):
+    """Every query is 4 * K[jdom]: that key's score exceeds all others by about 4 * d * scale = 4 sqrt(d), and the output is
+    V[jdom] to rounding (closed form), whichever tile the key sits in."""
+    H, Lq, Lk = 2, 260, 448
+    k = randn(240 + d, (Lk, H * d), dtype); v = _values(340 + d, (Lk, H * d), dtype)
+    q = np.tile(k[jdom] * np.float32(4.0), (Lq, 1))
+    out = _run(q, k, v, H, dtype)
+    assert_close(oracle.sdpa(q, k, v, H), out, dtype, f"d={d} key {jdom}")
+    assert np.abs(out - v[jdom]).max() <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+def test_pixart_cross_unnormed_queries(oracle, kernel_choice, dtype):
+    """PixArt cross attention with an un-normed query (src/dit/pixart.cpp:359-365): values up to +-300 against 300 text keys
+    with a valid length, 16 heads of 72; large enough for the short-key kernel when the kernel is chosen by size."""
+    B, H, d, Lq, Lk = 2, 16, 72, 2048, 300
+    q = randn(150, (B, Lq, H * d), dtype) * np.float32(64.0)
+    assert np.abs(q).max() > 250
+    k = randn(250, (B, Lk, H * d), dtype); v = _values(350, (B, Lk, H * d), dtype)
+    valid = [77, 221]
+    vl = torch.tensor(valid, dtype=torch.int32, device="cuda")
+    out = _run(q, k, v, H, dtype, kv_valid_len=vl)
+    rows = np.arange(0, Lq, 7, dtype=np.int32)
+    for b in range(B):
+        ref = oracle.sdpa(q[b], k[b, :valid[b]], v[b, :valid[b]], H, rows=rows)
+        assert_close(ref[rows], out[b][rows], dtype, f"batch {b}")
+
+
+def test_split_launch_scaled_queries(oracle, kernel_choice):
+    """A shape whose last round of work groups is cut along the key axis (24 heads of 128, 2816 rows on 256 compute units):
+    partial results of a tile are merged by their references and denominators, which peaked rows stress."""
+    if kernel_choice not in ("auto", "rows256"):
+        pytest.skip("the split belongs to the DMA kernel")
+    dtype, H, d, L = "bf16", 24, 128, 2816
+    q = randn(160, (L, H * d), dtype) * np.float32(8.0)
+    k = randn(260, (L, H * d), dtype); v = _values(360, (L, H * d), dtype)
+    out = _run(q, k, v, H, dtype)
+    rows = np.arange(3, L, 41, dtype=np.int32)
+    ref = oracle.sdpa(q, k, v, H, rows=rows)
+    assert_close(ref[rows], out[rows], dtype, "split")

@@ -48,6 +48,41 @@ def test_traced_matches_checker(oracle, dtype, H, d, txt, hp, wp, axes, with_bia
         assert np.abs(to_np(avg0)[:txt] - got[:txt]).max() <= 1e-6          # text rows carry no bias
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_traced_at_a_shape_whose_plain_call_splits_its_last_round(oracle, with_bias):
+    """Flux at 768 px (512 text + 48 x 48 image rows, 24 heads of 128): a plain attention call of this shape cuts its last
+    round of work groups along the key axis when a scratch is lent. The traced call asks for the softmax denominators
+    (and a bias), which only the 128-row kernel provides, so it must not take that route: sampled rows of the output and
+    of the map against the checker, and no split scratch is asked for."""
+    import ctypes as C
+    from brodiffusion_amd import _capi as capi
+    dtype, H, d, txt, hp, wp = "bf16", 24, 128, 512, 48, 48
+    L = txt + hp * wp
+    q, k, v = (randn(9700 + i, (L, H * d), dtype) for i in range(3))
+    cos, sin, dcos, dsin = tables(oracle, txt, hp, wp, d, (16, 56, 56))
+    bias = (randn(9710, (L - txt, txt), "fp32") * 1.5).astype(np.float32) if with_bias else None
+    dbias = None if bias is None else torch.from_numpy(bias).cuda()
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    out, avg = bd.joint_attention_traced(dq, dk, dv, dcos, dsin, d, H, txt_len=txt, image_text_bias=dbias)
+    rows = np.concatenate([np.arange(0, txt, 37), np.arange(txt + 5, L, 53)]).astype(np.int32)
+    qr = oracle.rope_apply(q, cos, sin, H, d, round_to_dtype=dtype)
+    kr = oracle.rope_apply(k, cos, sin, H, d, round_to_dtype=dtype)
+    ref_o, ref_avg = oracle.sdpa(qr, kr, v, H, bias=bias, bias_q0=txt, rows=rows, return_attn_avg=True)
+    assert_close(ref_o[rows], to_np(out)[rows], dtype, "traced output")
+    got = to_np(avg)
+    assert np.abs(got[rows] - ref_avg[rows]).max() <= 2e-5
+    assert np.abs(got.sum(axis=1) - 1.0).max() <= 1e-4
+    # the plain call of this shape does split; with a request for the denominators it must not
+    a = capi.MiSdpaArgs()
+    a.struct_size = C.sizeof(capi.MiSdpaArgs)
+    a.dtype, a.batch, a.num_heads, a.head_dim, a.q_len, a.kv_len = capi.MI_DTYPE_BF16, 1, H, d, L, L
+    a.q, a.k, a.v, a.o = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), out.data_ptr()
+    assert capi.lib().mi_sdpa_split_scratch_bytes(C.byref(a)) > 0
+    lse = torch.empty(H * L, dtype=torch.float32, device="cuda")
+    a.lse_out = lse.data_ptr()
+    assert capi.lib().mi_sdpa_split_scratch_bytes(C.byref(a)) == 0
+
+
 def test_traced_equals_fused_path_without_bias(oracle):
     """With no bias the traced output is the ordinary joint attention (same kernels up to the 128-row form)."""
     dtype, H, d, txt, hp, wp = "bf16", 8, 128, 32, 16, 16
