@@ -6,8 +6,8 @@
 //   state kernel: one work group reduces a chunk of tokens. K (ReLU applied on the way in) and V
 //                 tiles of 64 tokens sit row-major in LDS; both MFMA operands need the token axis
 //                 contiguous per lane, which ds_read_b64_tr_b16 (LDS transpose read) delivers.
-//                 z comes from the same K fragments against an all-ones A operand. Partial (S, z)
-//                 are added to the FP32 workspace with atomics.
+//                 z comes from the same K fragments against an all-ones A operand. No atomics anywhere:
+//                 results are bit-reproducible.
 //   apply kernel: S is staged in LDS as 16-bit A operand, relu(Q) rows are B operands straight from
 //                 global memory; the denominator is an exact FP32 dot of z with the lane's own Q
 //                 values plus one exchange between lanes l and l^32.
@@ -100,8 +100,8 @@ __device__ __forceinline__ bool lin_block(const LinDev& p, int& bh, int& chunk) 
 // 128-token tile in flight per group on top of the one being multiplied. Loads are branch-free (rows past the end of
 // the chunk are fetched from its last row and K is blanked at the LDS store, which removes their contribution to S
 // and z) and all issued before the first is used. z comes from the same K fragments against an all-ones A operand.
-// At the end the wavefronts add their blocks into an FP32 image of (S, z) in LDS (several wavefronts share a block
-// when S has fewer than 16 of them), which then goes out in full rows with plain stores: to the state itself when the
+// At the end the wavefronts put their blocks into FP32 images of (S, z) in LDS (one image per wavefront of those that
+// share a block when S has fewer than 16 of them, added in a fixed order), which then go out in full rows with plain stores: to the state itself when the
 // group covers the whole (batch, head), else to the group's slot among the partial states that a small reduction
 // kernel adds up afterwards (atomic adds from several groups to one address are executed at the memory side on this
 // multi-die GPU and were measured to cost far more than the whole pass).
@@ -118,7 +118,7 @@ template <int D> struct StateGeo {
     static constexpr int NLD = (NCH + kStateThreads - 1) / kStateThreads;
     static constexpr int TILE_BYTES = kStateTile * G::T_STRIDE;
     static constexpr int S_FLOATS = G::DP * G::DP + G::DP;
-    static constexpr int LDS_BYTES = 2 * TILE_BYTES > S_FLOATS * 4 ? 2 * TILE_BYTES : S_FLOATS * 4;
+    static constexpr int LDS_BYTES = 2 * TILE_BYTES > NTS * S_FLOATS * 4 ? 2 * TILE_BYTES : NTS * S_FLOATS * 4;
 };
 
 template <typename T, int D>
@@ -217,24 +217,22 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
         __syncthreads();
     }
 
-    // blocks -> FP32 image of (S, z) in LDS (rows of DP floats, then z), reusing the tile space
+    // blocks -> FP32 images of (S, z) in LDS (rows of DP floats, then z), reusing the tile space. Wavefronts that share a
+    // block (each took a share of every tile's tokens) write one image each; the images are added in a fixed order on the
+    // way out, so the result does not depend on which wavefront finishes first. Every element of an image is written:
+    // the NBLK blocks cover S, the blocks of the first block row cover z.
     float* const Sl = reinterpret_cast<float*>(lds);
-    for (int i = tid; i < SG::S_FLOATS; i += kStateThreads) Sl[i] = 0.f;
-    __syncthreads();
     if (active) {
+        float* const img = Sl + ts * SG::S_FLOATS;
         const int j = 32 * cb + lq;
 #pragma unroll
         for (int bb = 0; bb < 4; ++bb)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int i = 32 * rb + 8 * bb + 4 * lh + e;
-                if constexpr (SG::NTS > 1) atomicAdd(Sl + i * G::DP + j, acc[4 * bb + e]);
-                else Sl[i * G::DP + j] = acc[4 * bb + e];
+                img[i * G::DP + j] = acc[4 * bb + e];
             }
-        if (does_z && lh == 0) {
-            if constexpr (SG::NTS > 1) atomicAdd(Sl + G::DP * G::DP + j, zacc[0]);
-            else Sl[G::DP * G::DP + j] = zacc[0];
-        }
+        if (does_z && lh == 0) img[G::DP * G::DP + j] = zacc[0];
     }
     __syncthreads();
     // this group's (S, z): straight into the state when it covers the whole (batch, head), else into its partial slot
@@ -242,7 +240,10 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
                             : p.ws + static_cast<long>(bh) * G::WS_FLOATS;
     for (int idx = tid; idx < (D + 1) * (D / 4); idx += kStateThreads) {
         const int i = idx / (D / 4), j = (idx - i * (D / 4)) * 4;     // i == D: the z row, kept behind the DP rows of S
-        f32x4 v = *reinterpret_cast<const f32x4*>(Sl + (i < D ? i : G::DP) * G::DP + j);
+        const float* const src = Sl + (i < D ? i : G::DP) * G::DP + j;
+        f32x4 v = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+        for (int t = 1; t < SG::NTS; ++t) v += *reinterpret_cast<const f32x4*>(src + t * SG::S_FLOATS);
         if (p.add_to_state) v += *reinterpret_cast<const f32x4*>(S + i * D + j);   // the only group of this (batch, head)
         *reinterpret_cast<f32x4*>(S + i * D + j) = v;
     }
