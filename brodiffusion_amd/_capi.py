@@ -17,12 +17,13 @@ MI_MASK_NONE = 0
 MI_MASK_CAUSAL = 1
 MI_MASK_BLOCK_CAUSAL = 2
 MI_MAX_SEGMENTS = 32
+MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 
 EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
     "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_attention_map_avg", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
-    "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported",
+    "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported", "mi_linear_attn_relu_forward_static_scratch",
     "mi_linear_forward", "mi_linear_geglu_forward", "mi_add_inplace", "mi_add_row_bias", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
     "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv",
 ]
@@ -184,6 +185,7 @@ def lib() -> C.CDLL:
         L.mi_linear_attn_scratch_bytes.restype = C.c_size_t
         L.mi_linear_attn_relu_forward.argtypes = [C.POINTER(MiLinearAttnArgs)]
         L.mi_linear_attn_supported.argtypes = [C.c_int32, C.c_int32]
+        L.mi_linear_attn_relu_forward_static_scratch.argtypes = [C.POINTER(MiLinearAttnArgs)]
         L.mi_linear_forward.argtypes = [C.POINTER(MiLinearArgs)]
         L.mi_linear_geglu_forward.argtypes = [C.POINTER(MiLinearArgs)]
         L.mi_add_inplace.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]

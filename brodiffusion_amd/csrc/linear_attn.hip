@@ -13,10 +13,35 @@
 //                 values plus one exchange between lanes l and l^32.
 #include <algorithm>
 
+#include <atomic>
+
 #include "internal.h"
+
+// Partial states of mi_linear_attn_relu_forward_static_scratch: device memory that belongs to the library, one copy per
+// GPU, present from the moment the code object is loaded until the process ends. Host code never uses this name as an
+// address (on the host it is only a handle for hipGetSymbolAddress): kernels and copies get static_scratch_ptr().
+static __device__ __align__(256) unsigned char scratch[MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES];
 
 namespace mi {
 namespace {
+
+// Device address of `scratch` on the current GPU, looked up once per device (each GPU holds its own copy at its own
+// address). Two threads that meet here for the first time both look up the same address.
+constexpr int kMaxDevices = 64;
+std::atomic<unsigned char*> g_static_scratch[kMaxDevices];
+int static_scratch_ptr(unsigned char** out) {
+    int dev = -1;
+    MI_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail("mi_linear_attn_relu_forward_static_scratch: device %d outside 0..%d", dev, kMaxDevices - 1);
+    unsigned char* ptr = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        MI_HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+        if (ptr == nullptr) return fail("mi_linear_attn_relu_forward_static_scratch: hipGetSymbolAddress returned null");
+        g_static_scratch[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return 0;
+}
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -475,6 +500,51 @@ bool lin_supported(int dtype, int d) {
 }  // namespace
 }  // namespace mi
 
+namespace mi {
+namespace {
+// Shared body of the two entry points: `part` / `part_bytes` is the memory for the partial states of the token chunks
+// (the caller's scratch, the library's static scratch, or none).
+int linear_attn_forward(const mi_linear_attn_args* a, const char* op, void* part, size_t part_bytes) {
+    if (a->batch <= 0 || a->num_heads <= 0 || a->n_tokens < 0) return fail("%s: bad shape", op);
+    if (a->n_tokens == 0) return 0;
+    if (!a->q || !a->k || !a->v || !a->o) return fail("%s: null tensor", op);
+    const size_t need = mi_linear_attn_workspace_bytes(a->batch, a->num_heads, a->head_dim);
+    if (!a->workspace || a->workspace_bytes < need)
+        return fail("%s: workspace needs %zu bytes (got %zu)", op, need, a->workspace ? a->workspace_bytes : 0);
+    // the scratch decides how far the tokens of a head may be split over work groups (one partial state per chunk)
+    int max_split = 0;
+    if (part) {
+        if (reinterpret_cast<uintptr_t>(part) & 15u) return fail("%s: scratch must be 16-byte aligned", op);
+        max_split = static_cast<int>(std::min<size_t>(part_bytes / need, kMaxStateSplit));
+    }
+    const long D = static_cast<long>(a->num_heads) * a->head_dim;
+    LinDev p;
+    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
+    p.B = a->batch; p.H = a->num_heads; p.N = a->n_tokens;
+    auto rs = [D](int64_t s) { return s ? static_cast<long>(s) : D; };
+    p.q_rs = rs(a->q_row_stride); p.k_rs = rs(a->k_row_stride); p.v_rs = rs(a->v_row_stride); p.o_rs = rs(a->o_row_stride);
+    p.q_bs = a->q_batch_stride ? a->q_batch_stride : p.q_rs * a->n_tokens;
+    p.k_bs = a->k_batch_stride ? a->k_batch_stride : p.k_rs * a->n_tokens;
+    p.v_bs = a->v_batch_stride ? a->v_batch_stride : p.v_rs * a->n_tokens;
+    p.o_bs = a->o_batch_stride ? a->o_batch_stride : p.o_rs * a->n_tokens;
+    const long strides[] = {p.q_rs, p.k_rs, p.v_rs, p.o_rs, p.q_bs, p.k_bs, p.v_bs, p.o_bs};
+    for (long s : strides)
+        if (s % 8 != 0) return fail("%s: strides must be multiples of 8 elements", op);
+    if (p.q_rs < D || p.k_rs < D || p.v_rs < D || p.o_rs < D) return fail("%s: row stride smaller than heads*head_dim", op);
+    const uintptr_t al = reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
+                         reinterpret_cast<uintptr_t>(a->o) | reinterpret_cast<uintptr_t>(a->workspace);
+    if (al & 15u) return fail("%s: pointers must be 16-byte aligned", op);
+    p.eps = a->eps;
+    p.ws = static_cast<float*>(a->workspace);
+    p.part = max_split > 0 ? static_cast<float*>(part) : nullptr; p.n_part = 0; p.add_to_state = 0;
+    p.tokens_per_group = 0;
+    hipStream_t st = resolve_stream(a->stream);
+    const int n_cu = device_cu_count();
+    return launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, max_split, n_cu, st);
+}
+}  // namespace
+}  // namespace mi
+
 extern "C" {
 
 int mi_linear_attn_supported(int32_t dtype, int32_t head_dim) { return mi::lin_supported(dtype, head_dim) ? 1 : 0; }
@@ -490,48 +560,31 @@ size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t he
 
 int mi_linear_attn_relu_forward(const mi_linear_attn_args* a) {
     using mi::fail;
+    const char* op = "mi_linear_attn_relu_forward";
     mi::clear_error();
-    if (!a) return fail("mi_linear_attn_relu_forward: null args");
-    if (a->struct_size != sizeof(mi_linear_attn_args)) return fail("mi_linear_attn_relu_forward: struct_size mismatch");
-    if (!mi::lin_supported(a->dtype, a->head_dim))
-        return fail("mi_linear_attn_relu_forward: no kernel for dtype %d head_dim %d", a->dtype, a->head_dim);
-    if (a->batch <= 0 || a->num_heads <= 0 || a->n_tokens < 0) return fail("mi_linear_attn_relu_forward: bad shape");
-    if (a->n_tokens == 0) return 0;
-    if (!a->q || !a->k || !a->v || !a->o) return fail("mi_linear_attn_relu_forward: null tensor");
+    if (!a) return fail("%s: null args", op);
+    if (a->struct_size != sizeof(mi_linear_attn_args)) return fail("%s: struct_size mismatch", op);
+    if (!mi::lin_supported(a->dtype, a->head_dim)) return fail("%s: no kernel for dtype %d head_dim %d", op, a->dtype, a->head_dim);
+    return mi::linear_attn_forward(a, op, a->scratch, a->scratch ? a->scratch_bytes : 0);
+}
+
+int mi_linear_attn_relu_forward_static_scratch(const mi_linear_attn_args* a) {
+    using mi::fail;
+    const char* op = "mi_linear_attn_relu_forward_static_scratch";
+    mi::clear_error();
+    if (!a) return fail("%s: null args", op);
+    if (a->struct_size != sizeof(mi_linear_attn_args)) return fail("%s: struct_size mismatch", op);
+    if (!mi::lin_supported(a->dtype, a->head_dim)) return fail("%s: no kernel for dtype %d head_dim %d", op, a->dtype, a->head_dim);
+    if (a->scratch || a->scratch_bytes) return fail("%s: takes no scratch (the partial states live in the library's own static device array)", op);
+    // one partial state per (batch, head) must fit; larger problems belong to the entry point that takes a caller scratch
     const size_t need = mi_linear_attn_workspace_bytes(a->batch, a->num_heads, a->head_dim);
-    if (!a->workspace || a->workspace_bytes < need)
-        return fail("mi_linear_attn_relu_forward: workspace needs %zu bytes (got %zu)", need, a->workspace ? a->workspace_bytes : 0);
-    // the scratch decides how far the tokens of a head may be split over work groups (one partial state per chunk)
-    int max_split = 0;
-    if (a->scratch) {
-        if (reinterpret_cast<uintptr_t>(a->scratch) & 15u) return fail("mi_linear_attn_relu_forward: scratch must be 16-byte aligned");
-        max_split = static_cast<int>(std::min<size_t>(a->scratch_bytes / need, mi::kMaxStateSplit));
-    }
-    const long D = static_cast<long>(a->num_heads) * a->head_dim;
-    mi::LinDev p;
-    p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
-    p.B = a->batch; p.H = a->num_heads; p.N = a->n_tokens;
-    auto rs = [D](int64_t s) { return s ? static_cast<long>(s) : D; };
-    p.q_rs = rs(a->q_row_stride); p.k_rs = rs(a->k_row_stride); p.v_rs = rs(a->v_row_stride); p.o_rs = rs(a->o_row_stride);
-    p.q_bs = a->q_batch_stride ? a->q_batch_stride : p.q_rs * a->n_tokens;
-    p.k_bs = a->k_batch_stride ? a->k_batch_stride : p.k_rs * a->n_tokens;
-    p.v_bs = a->v_batch_stride ? a->v_batch_stride : p.v_rs * a->n_tokens;
-    p.o_bs = a->o_batch_stride ? a->o_batch_stride : p.o_rs * a->n_tokens;
-    const long strides[] = {p.q_rs, p.k_rs, p.v_rs, p.o_rs, p.q_bs, p.k_bs, p.v_bs, p.o_bs};
-    for (long s : strides)
-        if (s % 8 != 0) return fail("mi_linear_attn_relu_forward: strides must be multiples of 8 elements");
-    if (p.q_rs < D || p.k_rs < D || p.v_rs < D || p.o_rs < D)
-        return fail("mi_linear_attn_relu_forward: row stride smaller than heads*head_dim");
-    const uintptr_t al = reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
-                         reinterpret_cast<uintptr_t>(a->o) | reinterpret_cast<uintptr_t>(a->workspace);
-    if (al & 15u) return fail("mi_linear_attn_relu_forward: pointers must be 16-byte aligned");
-    p.eps = a->eps;
-    p.ws = static_cast<float*>(a->workspace);
-    p.part = max_split > 0 ? static_cast<float*>(a->scratch) : nullptr; p.n_part = 0; p.add_to_state = 0;
-    p.tokens_per_group = 0;
-    hipStream_t st = mi::resolve_stream(a->stream);
-    const int n_cu = mi::device_cu_count();
-    return mi::launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, max_split, n_cu, st);
+    if (a->batch > 0 && a->num_heads > 0 && need > static_cast<size_t>(MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES))
+        return fail("%s: the state of batch %d x heads %d x head_dim %d takes %zu bytes, the static scratch holds %zu: use "
+                    "mi_linear_attn_relu_forward with a caller scratch", op, a->batch, a->num_heads, a->head_dim, need,
+                    static_cast<size_t>(MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES));
+    unsigned char* ptr = nullptr;
+    if (mi::static_scratch_ptr(&ptr) != 0) return -1;
+    return mi::linear_attn_forward(a, op, ptr, static_cast<size_t>(MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES));
 }
 
 }  // extern "C"

@@ -816,15 +816,8 @@ def gqa_attention_masked(Q, K, V, cos, sin, head_dim: int, num_q_heads: int, num
                         rope_q=rope, rope_k=rope, rope_k_scratch=Kr if rope is not None else None, op=op)
 
 
-def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
-                                  workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False,
-                                  scratch: Optional[torch.Tensor] = None):
-    """Sana's ReLU linear attention core (src/dit/sana.cpp:470-586) on token-major (N, heads*head_dim)
-    or (batch, N, heads*head_dim) operands. `workspace` (float32, batch*heads*(d*d+d)) receives the
-    (S, z) state; pass it to capture the state or, with accumulate_state, to inject one. `scratch` (float32) holds
-    partial states of token chunks; None allocates one, False runs without (one work group per batch item and head)."""
-    op = "linear_attention_relu_forward"
-    _dev(op, Q, K, V, out, workspace, scratch if scratch is not False else None)
+def _linear_attn_args(op: str, Q, K, V, num_heads: int, out, eps: float, workspace, accumulate_state: bool):
+    """Validated mi_linear_attn_args for token-major operands; `out` and `workspace` must be given."""
     dt = _dtype_code(op, Q)
     if K.dtype != Q.dtype or V.dtype != Q.dtype:
         _fail(op, "Q, K, V must share one dtype")
@@ -836,16 +829,10 @@ def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.T
     if num_heads <= 0 or D % num_heads != 0:
         _fail(op, "D must equal head_dim * num_heads")
     hd = D // num_heads
-    if out is None:
-        out = torch.empty_like(Q)
     if out.shape != Q.shape or out.dtype != Q.dtype:
         _fail(op, "out must have Q's shape and dtype")
     _, _, _, o_rs, o_bs = _as3(op, out, "out")
     need = capi.lib().mi_linear_attn_workspace_bytes(B, num_heads, hd)
-    if workspace is None:
-        if accumulate_state:
-            _fail(op, "accumulate_state needs a caller workspace holding a state")
-        workspace = torch.empty(need // 4, dtype=torch.float32, device=Q.device)
     if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() * 4 < need:
         _fail(op, f"workspace must be contiguous float32 with at least {need // 4} elements")
     a = capi.MiLinearAttnArgs()
@@ -858,17 +845,53 @@ def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.T
     a.eps = eps
     a.accumulate_state = int(accumulate_state)
     a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * 4
+    a.stream = _stream()
+    return a
+
+
+def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
+                                  workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False,
+                                  scratch: Optional[torch.Tensor] = None):
+    """Sana's ReLU linear attention core (src/dit/sana.cpp:470-586) on token-major (N, heads*head_dim)
+    or (batch, N, heads*head_dim) operands. `workspace` (float32, batch*heads*(d*d+d)) receives the
+    (S, z) state; pass it to capture the state or, with accumulate_state, to inject one. `scratch` (float32) holds
+    partial states of token chunks; None allocates one, False runs without (one work group per batch item and head)."""
+    op = "linear_attention_relu_forward"
+    _dev(op, Q, K, V, out, workspace, scratch if scratch is not False else None)
+    if out is None:
+        out = torch.empty_like(Q)
+    if workspace is None:
+        if accumulate_state:
+            _fail(op, "accumulate_state needs a caller workspace holding a state")
+        if num_heads <= 0 or Q.shape[-1] % num_heads != 0:
+            _fail(op, "D must equal head_dim * num_heads")
+        B = Q.shape[0] if Q.dim() == 3 else 1
+        need = capi.lib().mi_linear_attn_workspace_bytes(B, num_heads, Q.shape[-1] // num_heads)
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=Q.device)
+    a = _linear_attn_args(op, Q, K, V, num_heads, out, eps, workspace, accumulate_state)
     if scratch is False:
         scratch = torch.empty(0, dtype=torch.float32, device=Q.device)      # explicitly none: one work group per (batch, head)
     if scratch is None:
         # partial states of the token chunks (lets the state pass use the whole GPU); comes from torch's caching allocator
-        scratch = torch.empty(capi.lib().mi_linear_attn_scratch_bytes(B, num_heads, hd) // 4, dtype=torch.float32, device=Q.device)
+        scratch = torch.empty(capi.lib().mi_linear_attn_scratch_bytes(a.batch, num_heads, a.head_dim) // 4, dtype=torch.float32,
+                              device=Q.device)
     if scratch.dtype != torch.float32 or not scratch.is_contiguous():
         _fail(op, "scratch must be contiguous float32")
     if scratch.numel() > 0:
         a.scratch, a.scratch_bytes = scratch.data_ptr(), scratch.numel() * 4
-    a.stream = _stream()
     capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
+    return out
+
+
+def linear_attention_relu_forward_static_scratch(Q, K, V, num_heads: int, out: torch.Tensor, workspace: torch.Tensor,
+                                                 eps: float = 1e-15, accumulate_state: bool = False):
+    """linear_attention_relu_forward for callers that must not allocate: `out` and `workspace` are the caller's, the
+    partial states live in the library's static device array (mi_linear_attn_relu_forward_static_scratch). Nothing is
+    allocated here or below; calls on one GPU must not overlap in time."""
+    op = "linear_attention_relu_forward_static_scratch"
+    _dev(op, Q, K, V, out, workspace)
+    a = _linear_attn_args(op, Q, K, V, num_heads, out, eps, workspace, accumulate_state)
+    capi.check(capi.lib().mi_linear_attn_relu_forward_static_scratch(C.byref(a)), op)
     return out
 
 

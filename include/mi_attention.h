@@ -310,6 +310,18 @@ MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, i
 MI_API size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API int mi_linear_attn_relu_forward(const mi_linear_attn_args* args);
 MI_API int mi_linear_attn_supported(int32_t dtype, int32_t head_dim);
+/* The same operator for callers that cannot allocate device memory and have no scratch to lend (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the partial states of the token chunks live in a
+ * static device array inside the library, MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES per GPU for the life of the process.
+ * No counterpart in the reference. Same args; `scratch` / `scratch_bytes` must be NULL / 0; q, k, v, o and `workspace`
+ * (the state, in and out) are still the caller's. Same kernels and, whenever 8 partial states fit the array, bit-identical
+ * results to mi_linear_attn_relu_forward with a full-size scratch. A problem whose state, batch * heads * (head_dim^2 +
+ * head_dim) floats, exceeds the array is refused with an error. Calls no hipMalloc / hipFree; its first call on a GPU looks
+ * up the array's device address (hipGetSymbolAddress) and should happen outside a capture. All calls on one GPU share the
+ * array: calls that overlap in time on one GPU (two streams, two threads) race; nothing in it needs clearing between
+ * calls (every partial state that is read was written by the same call). */
+enum { MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024 };
+MI_API int mi_linear_attn_relu_forward_static_scratch(const mi_linear_attn_args* args);
 
 /* ── linear layer ──────────────────────────────────────────────────────────
  * Y = X W^T + bias: X (rows, in_features), W (out_features, in_features) — the layout of a
