@@ -9,6 +9,9 @@
 // The score tile is computed transposed (rows = keys, columns = queries), so a lane holds scores of
 // ONE query and the accumulator layout of P^T is directly the B operand of O^T += V^T P^T.
 #pragma once
+#include <type_traits>
+#include <utility>
+
 #include "internal.h"
 
 namespace mi {
@@ -207,25 +210,42 @@ constexpr int kAhead = 4;
 // the shadow of the matrix pipe.
 struct NoMid { __device__ __forceinline__ void operator()() const {} };
 
-template <typename T, int D, bool DO_PV, bool DO_QK, typename Mid = NoMid>
+// TO_EXPONENT (needs both products): the stream scores first and then, in the shadow of the PV MFMAs (which do not
+// touch the scores), turns every raw score s into the softmax exponent x = s * cl2 + neg_ref with one FP32 fused
+// multiply-add, a few per MFMA slot, first block first (its MFMAs retired long ago). The scale therefore never touches a
+// 16-bit operand, and the VALU work costs no time of its own while the matrix pipe is the busier unit.
+template <int NPV, int J>
+__device__ __forceinline__ void scores_to_exponents(f32x16 (&sacc)[2], float cl2, float neg_ref) {
+    constexpr int E0 = 32 * J / NPV, E1 = 32 * (J + 1) / NPV;
+#pragma unroll
+    for (int e = E0; e < E1; ++e) sacc[e >> 4][e & 15] = __builtin_fmaf(sacc[e >> 4][e & 15], cl2, neg_ref);
+}
+
+template <typename T, int D, bool DO_PV, bool DO_QK, typename Mid = NoMid, bool TO_EXPONENT = false>
 __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsigned char* Ks, const typename Mma<T>::v8 (&pf)[4],
                                             const typename Mma<T>::v8 (&qf)[HeadGeo<D>::KC], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid()) {
+                                            f32x16 (&sacc)[2], int lane, Mid mid = Mid(), float cl2 = 1.f, float neg_ref = 0.f) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
+    static_assert(!TO_EXPONENT || (DO_PV && DO_QK), "the exponent pass rides under the PV product of a stream that also scores");
     constexpr int NPV = DO_PV ? 4 * G::VB : 0;
     constexpr int NQK = DO_QK ? 2 * G::KC : 0;
     constexpr int N = NPV + NQK;
     if constexpr (N == 0) return;
+    // position i of the stream: PV first by default, QK first when the exponents are formed under the PV part
+    constexpr int PV0 = TO_EXPONENT ? NQK : 0;     // first PV position
+    constexpr int QK0 = TO_EXPONENT ? 0 : NPV;     // first QK position
     const int lq = lane & 31;
     const int lh = lane >> 5;
     const int trow = (lane & 15) >> 2;
     const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
     const unsigned char* const vlane = Vs + (4 * lh + trow) * G::V_STRIDE + tcol * 2;
     const unsigned char* const klane = Ks + lq * G::K_STRIDE + 8 * lh * 2;
+    auto is_pv = [](int i) { return i >= PV0 && i < PV0 + NPV; };
     auto fetch = [&](int i) -> V8 {
-        if (i < NPV) {
-            const int c4 = i / G::VB, vb = i % G::VB;
+        if (is_pv(i)) {
+            const int j = i - PV0;
+            const int c4 = j / G::VB, vb = j % G::VB;
             const unsigned char* vptr = vlane + 16 * c4 * G::V_STRIDE + 32 * vb * 2;
             const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
             const s16x4 v_hi =
@@ -233,7 +253,7 @@ __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsig
             const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
             return __builtin_bit_cast(V8, a);
         } else {
-            const int k = i - NPV;
+            const int k = i - QK0;
             const int kb = k / G::KC, c = k % G::KC;
             const u32x4 a = *reinterpret_cast<const u32x4*>(klane + 32 * kb * G::K_STRIDE + 16 * c * 2);
             return __builtin_bit_cast(V8, a);
@@ -242,29 +262,33 @@ __device__ __forceinline__ void mfma_stream(const unsigned char* Vs, const unsig
     V8 ring[kAhead];
 #pragma unroll
     for (int i = 0; i < kAhead && i < N; ++i) ring[i] = fetch(i);
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const V8 a = ring[i % kAhead];
-        if (i < NPV) {
-            const int c4 = i / G::VB, vb = i % G::VB;
-            oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
-        } else {
-            const int k = i - NPV;
-            const int kb = k / G::KC, c = k % G::KC;
-            if (c == 0) {
-                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                sacc[kb] = Mma<T>::run(a, qf[c], zero);
+    [&]<int... I>(std::integer_sequence<int, I...>) {
+        ([&] {
+            constexpr int i = I;
+            const V8 a = ring[i % kAhead];
+            if constexpr (i >= PV0 && i < PV0 + NPV) {
+                constexpr int j = i - PV0;
+                constexpr int c4 = j / G::VB, vb = j % G::VB;
+                oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
             } else {
-                sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
+                constexpr int k = i - QK0;
+                constexpr int kb = k / G::KC, c = k % G::KC;
+                if constexpr (c == 0) {
+                    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                    sacc[kb] = Mma<T>::run(a, qf[c], zero);
+                } else {
+                    sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
+                }
             }
-        }
-        if (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
-        MI_SCHED_BARRIER
-        if (i == (N > 8 ? 5 : 0)) {
-            mid();
+            if constexpr (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
+            if constexpr (TO_EXPONENT && i >= PV0 && i < PV0 + NPV) scores_to_exponents<NPV, i - PV0>(sacc, cl2, neg_ref);
             MI_SCHED_BARRIER
-        }
-    }
+            if constexpr (i == (N > 8 ? 5 : 0)) {
+                mid();
+                MI_SCHED_BARRIER
+            }
+        }(), ...);
+    }(std::make_integer_sequence<int, N>{});
 }
 
 // score, or -inf when `x` is outside [0, top] (x = key - lo, top = hi - 1 - lo) or `extra` is negative: the sign of
@@ -369,15 +393,26 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
         for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(sacc[c4 >> 1][8 * (c4 & 1) + t]);
 }
 
-// Softmax step of the 256-row kernels: the exponent of a term is formed by ONE fused multiply-add on the raw FP32 score,
-// x = s * (scale * log2 e) - ref, against a per-row reference that is not the running maximum, so the usual tile maximum
-// is not computed at all: per 64-key tile and lane 32 v_fma, 32 v_exp, 32 adds and 16 packs. Q, K and the scores are
-// untouched by the scale (it multiplies the FP32 accumulator, never a 16-bit operand).
+// Softmax step of the 256-row kernels. The scores arrive as exponents relative to the row's reference,
+// x = s * (scale * log2 e) - ref (one FP32 fused multiply-add per raw score, done by the MFMA stream in the shadow of the
+// PV product: Q, K and the raw scores never see the scale), so P = exp2(x) needs no further arithmetic and the usual tile
+// maximum is not computed at all: per 64-key tile and lane 32 v_exp, 32 adds and 16 packs.
 //   * The reference of a row is the maximum of its first tile with a visible key (then its largest term is 1, so the
 //     denominator stays >= 1), and is raised to a later tile's maximum only when that tile's terms get large (lane sum
 //     above 2^10, or overflow). Any reference gives the same softmax; these two rules keep every term within FP32 / T range.
 //   * Both cases, and rows that have not seen a key yet, take the slow path below (wave-uniform branch): row maximum,
-//     shift of l, O and the reference, new exponentials. Lanes l and l^32 share a row and decide from row-wide values only.
+//     shift of l, O, the exponents and the reference, new exponentials. Lanes l and l^32 share a row and decide from
+//     row-wide values only.
+// acc + v[2i] + v[2i+1], products with 1 exact, FP32 accumulation (v_dot2c_f32_bf16 / v_dot2c_f32_f16).
+template <typename T>
+__device__ __forceinline__ float pair_sum(const typename Mma<T>::v8& v, int i, float acc) {
+    typedef T t2 __attribute__((ext_vector_type(2)));
+    const t2 pr = {v[2 * i], v[2 * i + 1]};
+    const t2 one = {static_cast<T>(1.f), static_cast<T>(1.f)};
+    if constexpr (std::is_same_v<T, __bf16>) return __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false);
+    else return __builtin_amdgcn_fdot2(pr, one, acc, false);
+}
+
 struct RelSoftmaxState {
     float l = 0.f;          // this lane's share of the denominator
     float neg_ref = 0.f;    // minus the row's reference, in exponent (base-2) units
@@ -387,8 +422,7 @@ constexpr float kRelSumMax = 1024.f;
 
 template <typename T, int D>
 __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                                 RelSoftmaxState& st, float cl2, bool masked, bool dead_row, int j0, int lo,
-                                                 int hi, int lh) {
+                                                 RelSoftmaxState& st, bool masked, bool dead_row, int j0, int lo, int hi, int lh) {
     if (masked) {
         const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;   // keys outside [lo, hi) become -inf
 #pragma unroll
@@ -399,21 +433,35 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
                 sacc[kb][e] = blank_outside(score, d0 + 32 * kb + 8 * (e >> 2) + (e & 3), top);
             }
     }
+    // Row sum of the tile. Up to head_dim 96 the key step is bound by its VALU instructions, and the sum is taken from the
+    // packed 16-bit P (one v_dot2c per pair against (1, 1), FP32 accumulation: half the instructions, and the denominator
+    // sums exactly the values the PV product uses; measured 4 % faster at head_dim 40 and 72). From 112 on the matrix
+    // pipe is the busier unit and the same change measured 6 % slower, so there the FP32 exponentials are added.
+    constexpr bool PAIR_SUM = HeadGeo<D>::VB < 4;
     auto exponentiate = [&]() -> float {
         float s0 = 0.f, s1 = 0.f;
-        const float nr = st.neg_ref;
         // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
 #pragma unroll
-        for (int c4 = 0; c4 < 4; ++c4)
+        for (int c4 = 0; c4 < 4; ++c4) {
+            if constexpr (PAIR_SUM) {
 #pragma unroll
-            for (int t = 0; t < 8; t += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c4 >> 1][8 * (c4 & 1) + t], cl2, nr));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[c4 >> 1][8 * (c4 & 1) + t + 1], cl2, nr));
-                pf[c4][t] = static_cast<T>(p0);
-                pf[c4][t + 1] = static_cast<T>(p1);
-                s0 += p0;
-                s1 += p1;
+                for (int t = 0; t < 8; ++t) pf[c4][t] = static_cast<T>(__builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t]));
+                s0 = pair_sum<T>(pf[c4], 0, s0);
+                s1 = pair_sum<T>(pf[c4], 1, s1);
+                s0 = pair_sum<T>(pf[c4], 2, s0);
+                s1 = pair_sum<T>(pf[c4], 3, s1);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 8; t += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t]);
+                    const float p1 = __builtin_amdgcn_exp2f(sacc[c4 >> 1][8 * (c4 & 1) + t + 1]);
+                    pf[c4][t] = static_cast<T>(p0);
+                    pf[c4][t + 1] = static_cast<T>(p1);
+                    s0 += p0;
+                    s1 += p1;
+                }
             }
+        }
         return s0 + s1;
     };
     float ls = exponentiate();
@@ -424,10 +472,8 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
         for (int e = 1; e < 16; ++e) mloc = fmaxf(mloc, fmaxf(sacc[0][e], sacc[1][e]));
         mloc = exchange_max(mloc);
         const bool visible = mloc > kNegInf;
-        // the tile's largest exponent against the present reference; a started row only ever moves its reference up
-        // (its terms then stay <= 1)
-        const float top_x = __builtin_fmaf(mloc, cl2, st.neg_ref);
-        const float shift = !visible ? 0.f : (st.started ? fmaxf(top_x, 0.f) : top_x);
+        // a started row only ever moves its reference up (its terms then stay <= 1)
+        const float shift = !visible ? 0.f : (st.started ? fmaxf(mloc, 0.f) : mloc);
         const float alpha = st.started ? __builtin_amdgcn_exp2f(-shift) : 1.f;   // nothing accumulated before the first key
         st.started = st.started || visible;
         st.l *= alpha;
@@ -435,6 +481,11 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
         for (int vb = 0; vb < HeadGeo<D>::VB; ++vb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[vb][e] *= alpha;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            sacc[0][e] -= shift;
+            sacc[1][e] -= shift;
+        }
         st.neg_ref -= shift;
         ls = exponentiate();
     }

@@ -722,7 +722,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
-                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, false, false, 0, 0, p.Lk, lh);
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, false, false, 0, 0, p.Lk, lh);
                     return;
                 }
             }
@@ -730,7 +730,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -747,8 +747,9 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
             // after the last tile the extra scores are never read. This wavefront's share of the tile
             // movement rides along in the stream (measured faster than in front of the softmax: the stores
             // and loads issue in the shadow of the matrix pipe).
-            mfma_stream<T, D, true, true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf, oacc, sacc, lane,
-                                          [&]() { advance_tiles(t + 2, t + 1); });
+            auto mover = [&]() { advance_tiles(t + 2, t + 1); };
+            mfma_stream<T, D, true, true, decltype(mover), true>(Vbuf + (t & 1) * G::V_BYTES, Kbuf + ((t + 1) & 1) * G::K_BYTES, pf, qf,
+                                                                 oacc, sacc, lane, mover, cl2, st.neg_ref);
             if (grp == 0) {
                 MI_SCHED_BARRIER
                 softmax_of(t + 1);
@@ -967,7 +968,9 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         unsigned voff = dcol[m];
         if constexpr (!DENSE) voff += static_cast<unsigned>(min(drow[m], min(c.rows_left, kBN) - 1)) * c.rsb;
         const unsigned dst = lds_base + lds_off + j * 1024;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(voff), "s"(c.ptr) : "memory", "m0");
+        // (the LDS base travels in m0 as a declared input: the compiler writes the register itself and knows it is taken;
+        //  the s_nop is the wait state an LDS-DMA instruction needs behind a write of m0)
+        asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(c.ptr), "{m0}"(dst) : "memory");
     };
     // this wavefront's share of the loads of one K tile (if do_k) and one V tile (if do_v); returns how many it issued
     auto dma_tiles = [&](bool do_k, int k_off, bool do_v, int v_off) -> int {
@@ -1038,7 +1041,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
-                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, false, false, 0, 0, n_keys, lh);
+                    softmax_tile_rel<T, D>(sacc, pf, oacc, st, false, false, 0, 0, n_keys, lh);
                     return;
                 }
             }
@@ -1046,7 +1049,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, cl2, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                softmax_tile_rel<T, D>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -1074,10 +1077,13 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             MI_SCHED_BARRIER
         }
         {
-            constexpr int NPV = 4 * G::VB, N = NPV + 2 * G::KC;
+            // the stream scores first (S_{t+1} = K_{t+1} Q^T), then O += V_t^T P_t; under the PV MFMAs, which do not touch
+            // the scores, each raw score becomes the softmax exponent x = s * cl2 - ref (see mfma_stream)
+            constexpr int NQK = 2 * G::KC, NPV = 4 * G::VB, N = NQK + NPV;
             auto fetch = [&](int i) -> V8 {
-                if (i < NPV) {
-                    const int c4 = i / G::VB, vb = i % G::VB;
+                if (i >= NQK) {
+                    const int j = i - NQK;
+                    const int c4 = j / G::VB, vb = j % G::VB;
                     const s16x4 v_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                         (__attribute__((address_space(3))) s16x4*)(smem + VS + 16 * c4 * DG::ROWB + vaddr[vb][0]));
                     const s16x4 v_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -1085,8 +1091,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                     const s16x8 a = __builtin_shufflevector(v_lo, v_hi, 0, 1, 2, 3, 4, 5, 6, 7);
                     return __builtin_bit_cast(V8, a);
                 } else {
-                    const int k = i - NPV;
-                    const int kb = k / G::KC, c = k % G::KC;
+                    const int kb = i / G::KC, c = i % G::KC;
                     const u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * DG::ROWB + kaddr[c]);
                     return __builtin_bit_cast(V8, a);
                 }
@@ -1094,25 +1099,29 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             V8 ring[kAhead];
 #pragma unroll
             for (int i = 0; i < kAhead; ++i) ring[i] = fetch(i);
-#pragma unroll
-            for (int i = 0; i < N; ++i) {
-                const V8 a = ring[i % kAhead];
-                if (i < NPV) {
-                    const int c4 = i / G::VB, vb = i % G::VB;
-                    oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
-                } else {
-                    const int k = i - NPV;
-                    const int kb = k / G::KC, c = k % G::KC;
-                    if (c == 0) {
-                        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                        sacc[kb] = Mma<T>::run(a, qf[c], zero);
+            const float neg_ref = st.neg_ref;
+            [&]<int... I>(std::integer_sequence<int, I...>) {
+                ([&] {
+                    constexpr int i = I;
+                    const V8 a = ring[i % kAhead];
+                    if constexpr (i >= NQK) {
+                        constexpr int j = i - NQK;
+                        constexpr int c4 = j / G::VB, vb = j % G::VB;
+                        oacc[vb] = Mma<T>::run(a, pf[c4], oacc[vb]);
                     } else {
-                        sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
+                        constexpr int kb = i / G::KC, c = i % G::KC;
+                        if constexpr (c == 0) {
+                            const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                            sacc[kb] = Mma<T>::run(a, qf[c], zero);
+                        } else {
+                            sacc[kb] = Mma<T>::run(a, qf[c], sacc[kb]);
+                        }
                     }
-                }
-                if (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
-                MI_SCHED_BARRIER
-            }
+                    if constexpr (i + kAhead < N) ring[i % kAhead] = fetch(i + kAhead);
+                    if constexpr (i >= NQK) scores_to_exponents<NPV, i - NQK>(sacc, cl2, neg_ref);
+                    MI_SCHED_BARRIER
+                }(), ...);
+            }(std::make_integer_sequence<int, N>{});
         }
         if (grp == 0) {
             MI_SCHED_BARRIER
