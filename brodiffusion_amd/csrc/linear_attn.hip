@@ -4,13 +4,16 @@
 // The op is HBM-bound: Q, K, V are read once and O written once (4 streams of (N, H*d) 16-bit
 // values); the d x d contractions are small and run on MFMA so they hide under the memory time.
 //   state kernel: one work group reduces a chunk of tokens. K (ReLU applied on the way in) and V
-//                 tiles of 64 tokens sit row-major in LDS; both MFMA operands need the token axis
-//                 contiguous per lane, which ds_read_b64_tr_b16 (LDS transpose read) delivers.
-//                 z comes from the same K fragments against an all-ones A operand. No atomics anywhere:
-//                 results are bit-reproducible.
-//   apply kernel: S is staged in LDS as 16-bit A operand, relu(Q) rows are B operands straight from
-//                 global memory; the denominator is an exact FP32 dot of z with the lane's own Q
-//                 values plus one exchange between lanes l and l^32.
+//                 tiles of 128 tokens sit row-major in LDS; both MFMA operands need the token axis
+//                 contiguous per lane, which ds_read_b64_tr_b16 (LDS transpose read) delivers. A
+//                 wavefront owns a 64 x 64 piece of S, so every fragment it reads feeds two MFMAs.
+//                 z falls out of the same product as an extra row of S (a column of ones in V's
+//                 zero pad), or comes from the K fragments against an all-ones operand where the
+//                 head dimension leaves no pad. No atomics anywhere: results are bit-reproducible.
+//   reduce kernel: adds the partial states of the token chunks into the state, in a fixed order.
+//   apply kernel: S is staged in LDS as 16-bit A operand, relu(Q) rows are B operands; the denominator
+//                 is an exact FP32 dot of z with the lane's own Q values plus one exchange between
+//                 lanes l and l^32.
 #include <algorithm>
 
 #include <atomic>
@@ -96,13 +99,20 @@ template <int D> struct LGeo {
     static constexpr int WS_FLOATS = D * D + D;
 };
 
+// ReLU of 8 packed 16-bit floats. Both formats keep the sign in the top bit, so as signed 16-bit integers every negative
+// value (and -0) is below zero and every positive one keeps its bits: a packed integer max with 0 is the ReLU.
+typedef short s16x2 __attribute__((ext_vector_type(2)));
 template <typename T>
 __device__ __forceinline__ u32x4 relu8(u32x4 raw) {
-    typedef T t8 __attribute__((ext_vector_type(8)));
-    t8 x = __builtin_bit_cast(t8, raw);
+    u32x4 out;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[i] = x[i] > static_cast<T>(0.f) ? x[i] : static_cast<T>(0.f);
-    return __builtin_bit_cast(u32x4, x);
+    for (int i = 0; i < 4; ++i) {
+        const unsigned w = raw[i];
+        const s16x2 x = __builtin_bit_cast(s16x2, w);
+        const s16x2 r = __builtin_elementwise_max(x, s16x2{0, 0});
+        out[i] = __builtin_bit_cast(unsigned, r);
+    }
+    return out;
 }
 
 
@@ -119,31 +129,41 @@ __device__ __forceinline__ bool lin_block(const LinDev& p, int& bh, int& chunk) 
     return true;
 }
 
-// ── state: (S, z) += over this group's token chunk ──
-// The pass is a stream of K and V rows with little arithmetic, so what matters is bytes in flight: a work group has
-// 16 wavefronts, each owning at most one 32x32 block of S (16 accumulator registers), which leaves registers for a
-// 128-token tile in flight per group on top of the one being multiplied. Loads are branch-free (rows past the end of
-// the chunk are fetched from its last row and K is blanked at the LDS store, which removes their contribution to S
-// and z) and all issued before the first is used. z comes from the same K fragments against an all-ones A operand.
-// At the end the wavefronts put their blocks into FP32 images of (S, z) in LDS (one image per wavefront of those that
-// share a block when S has fewer than 16 of them, added in a fixed order), which then go out in full rows with plain stores: to the state itself when the
-// group covers the whole (batch, head), else to the group's slot among the partial states that a small reduction
-// kernel adds up afterwards (atomic adds from several groups to one address are executed at the memory side on this
-// multi-die GPU and were measured to cost far more than the whole pass).
-constexpr int kStateThreads = 1024;
+// ── state: (S, z) of this group's token chunk ──
+// The pass streams K and V rows with little arithmetic; what limits it besides HBM is the LDS read path, because both
+// MFMA operands come out of LDS through transpose reads. So a wavefront owns a rectangle of 32x32 blocks of S (2 x 2 where
+// S has 16 blocks: 4 MFMAs per 4 fragments read instead of 1 per 2), and the wavefronts that are left over split the 16-token
+// steps of every tile among themselves. Loads are branch-free (rows past the end of the chunk are fetched from its last
+// row and K is blanked at the LDS store, which removes their contribution to S and z) and all issued before the first is
+// used; the next tile's rows are in flight in registers while the current one is multiplied.
+// z = sum of relu(K) rows: where the padded head dimension leaves room (d = 72, 112) column d of the V tile in LDS holds
+// ones, so row d of S is z and costs nothing; otherwise the wavefronts of the first block row multiply the K fragments
+// with an all-ones operand as well.
+// At the end the wavefronts put their blocks into FP32 images of (S, z) in LDS (one image per token share, added in a
+// fixed order), which then go out in full rows with plain stores: to the state itself when the group covers the whole
+// (batch, head), else to the group's slot among the partial states that a small reduction kernel adds up (atomic adds from several
+// groups to one address are executed at the memory side on this multi-die GPU and were measured to cost far more than
+// the whole pass).
+constexpr int kStateThreads = 512;
+constexpr int kStateWaves = kStateThreads / 64;
 constexpr int kMaxStateSplit = 8;   // most token chunks per (batch, head) whose partial states the workspace can hold
 constexpr int kStateTile = 128;
 
 template <int D> struct StateGeo {
     using G = LGeo<D>;
-    static constexpr int NBLK = G::NB * G::NB;                                   // 32x32 blocks of S
-    static constexpr int NTS = NBLK >= 16 ? 1 : (16 / NBLK > 8 ? 8 : 16 / NBLK); // wavefronts sharing a block (token split)
+    static constexpr int RBW = G::NB == 3 ? 3 : (G::NB >= 2 ? 2 : 1);            // block rows of a wavefront's rectangle
+    static constexpr int CBW = G::NB == 3 ? 1 : (G::NB >= 2 ? 2 : 1);            // block columns
+    static constexpr int NOWN = (G::NB / RBW) * (G::NB / CBW);                   // rectangles that tile S
+    static constexpr int NTS = kStateWaves / NOWN;                               // wavefronts sharing a rectangle (token split)
     static constexpr int KSTEPS = (kStateTile / 16) / NTS;                       // 16-token steps per wavefront and tile
+    static constexpr bool Z_IN_PAD = G::DP > D;                                  // z as row D of S
+    static constexpr int Z_ROW = Z_IN_PAD ? D : G::DP;                           // row of the FP32 image that holds z
     static constexpr int NCH = kStateTile * G::CPR;
     static constexpr int NLD = (NCH + kStateThreads - 1) / kStateThreads;
     static constexpr int TILE_BYTES = kStateTile * G::T_STRIDE;
     static constexpr int S_FLOATS = G::DP * G::DP + G::DP;
     static constexpr int LDS_BYTES = 2 * TILE_BYTES > NTS * S_FLOATS * 4 ? 2 * TILE_BYTES : NTS * S_FLOATS * 4;
+    static_assert((kStateTile / 16) % NTS == 0 && NTS >= 1, "token steps must divide among the sharing wavefronts");
 };
 
 template <typename T, int D>
@@ -165,32 +185,47 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
     const T* const k_base = static_cast<const T*>(p.k) + b * p.k_bs + h * D;
     const T* const v_base = static_cast<const T*>(p.v) + b * p.v_bs + h * D;
 
-    // wave -> (block of S, share of the k-steps of a tile)
-    const int blk = wave % SG::NBLK;
-    const int ts = wave / SG::NBLK;
-    const int rb = blk / G::NB, cb = blk % G::NB;
+    // wave -> (rectangle of S, share of the k-steps of a tile)
+    const int own = wave % SG::NOWN;
+    const int ts = wave / SG::NOWN;
+    const int rb0 = (own / (G::NB / SG::CBW)) * SG::RBW, cb0 = (own % (G::NB / SG::CBW)) * SG::CBW;
     const bool active = ts < SG::NTS;
-    const bool does_z = active && rb == 0;
+    const bool does_z = !SG::Z_IN_PAD && active && rb0 == 0;
 
-    if constexpr (G::DP > D) {  // pad columns stay zero for the whole kernel
+    if constexpr (G::DP > D) {  // pad columns stay as written here for the whole kernel: zero, and ones in column D of V
         constexpr int PC = (G::DP - D) / 8;
+        typedef T t8 __attribute__((ext_vector_type(8)));
+        t8 one_first;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) one_first[e] = static_cast<T>(e == 0 ? 1.f : 0.f);
         for (int i = tid; i < kStateTile * PC; i += kStateThreads) {
             const int off = (i / PC) * G::T_STRIDE + D * 2 + (i % PC) * 16;
             *reinterpret_cast<u32x4*>(Ks + off) = u32x4{0, 0, 0, 0};
-            *reinterpret_cast<u32x4*>(Vs + off) = u32x4{0, 0, 0, 0};
+            *reinterpret_cast<u32x4*>(Vs + off) = (i % PC) == 0 ? __builtin_bit_cast(u32x4, one_first) : u32x4{0, 0, 0, 0};
         }
     }
 
-    f32x16 acc, zacc;
+    f32x16 acc[SG::RBW][SG::CBW], zacc[SG::CBW];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) { acc[e] = 0.f; zacc[e] = 0.f; }
+    for (int e = 0; e < 16; ++e) {
+#pragma unroll
+        for (int j = 0; j < SG::CBW; ++j) {
+            zacc[j][e] = 0.f;
+#pragma unroll
+            for (int i = 0; i < SG::RBW; ++i) acc[i][j][e] = 0.f;
+        }
+    }
     V8 ones;
 #pragma unroll
     for (int t = 0; t < 8; ++t) ones[t] = static_cast<T>(1.f);
 
-    u32x4 kreg[SG::NLD], vreg[SG::NLD];
+    // Two register sets, so that the loads of two tiles are in flight while a third is multiplied: with one set a group
+    // waits out most of the memory latency once per tile. All loads are unconditional (rows past the end of the chunk
+    // repeat its last row), which keeps the order "older set, newer set" the same on every path and lets the wait in
+    // front of an LDS store cover the older set only.
+    u32x4 kregA[SG::NLD], vregA[SG::NLD], kregB[SG::NLD], vregB[SG::NLD];
     const int last = n_end - 1;
-    auto issue_loads = [&](int n0) {
+    auto issue_loads = [&](u32x4 (&kreg)[SG::NLD], u32x4 (&vreg)[SG::NLD], int n0) {
 #pragma unroll
         for (int i = 0; i < SG::NLD; ++i) {
             const int idx = min(tid + kStateThreads * i, SG::NCH - 1);
@@ -200,7 +235,7 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
             vreg[i] = *reinterpret_cast<const u32x4*>(v_base + n * p.v_rs + cc * 8);
         }
     };
-    auto store_tile = [&](int n0) {
+    auto store_tile = [&](const u32x4 (&kreg)[SG::NLD], const u32x4 (&vreg)[SG::NLD], int n0) {
 #pragma unroll
         for (int i = 0; i < SG::NLD; ++i) {
             const int idx = tid + kStateThreads * i;
@@ -213,63 +248,94 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
             }
         }
     };
+    auto frag = [&](const unsigned char* ptr) -> V8 {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr + 8 * G::T_STRIDE));
+        return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
 
     const int trow = (lane & 15) >> 2;
     const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-    issue_loads(n_begin);
-    for (int n0 = n_begin; n0 < n_end; n0 += kStateTile) {
-        store_tile(n0);
-        __syncthreads();
-        if (n0 + kStateTile < n_end) issue_loads(n0 + kStateTile);
+    auto multiply_tile = [&]() {
         if (active) {
 #pragma unroll
             for (int s = 0; s < SG::KSTEPS; ++s) {
                 const int trow0 = 16 * (ts * SG::KSTEPS + s) + 4 * lh + trow;
-                const unsigned char* vptr = Vs + trow0 * G::T_STRIDE + (32 * rb + tcol) * 2;
-                const unsigned char* kptr = Ks + trow0 * G::T_STRIDE + (32 * cb + tcol) * 2;
-                const s16x4 a_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(vptr));
-                const s16x4 a_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(vptr + 8 * G::T_STRIDE));
-                const s16x4 b_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(kptr));
-                const s16x4 b_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(kptr + 8 * G::T_STRIDE));
-                const V8 a = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                const V8 bk = __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-                acc = Mma<T>::run(a, bk, acc);
-                if (does_z) zacc = Mma<T>::run(ones, bk, zacc);
+                V8 a[SG::RBW], bk[SG::CBW];
+#pragma unroll
+                for (int i = 0; i < SG::RBW; ++i) a[i] = frag(Vs + trow0 * G::T_STRIDE + (32 * (rb0 + i) + tcol) * 2);
+#pragma unroll
+                for (int j = 0; j < SG::CBW; ++j) bk[j] = frag(Ks + trow0 * G::T_STRIDE + (32 * (cb0 + j) + tcol) * 2);
+#pragma unroll
+                for (int j = 0; j < SG::CBW; ++j) {
+#pragma unroll
+                    for (int i = 0; i < SG::RBW; ++i) acc[i][j] = Mma<T>::run(a[i], bk[j], acc[i][j]);
+                    if (does_z) zacc[j] = Mma<T>::run(ones, bk[j], zacc[j]);
+                }
             }
         }
+    };
+    // The loop takes two tiles per turn and has one way out, at the bottom: a second exit between the halves would give
+    // the compiler a path on which set A is the newer one, and its waits at the top would drain both sets.
+    const int n_tiles = (n_end - n_begin + kStateTile - 1) / kStateTile;
+    int n0 = n_begin;
+    issue_loads(kregA, vregA, n0);
+    issue_loads(kregB, vregB, n0 + kStateTile);
+    for (int pairs = n_tiles >> 1; pairs > 0; --pairs) {
+        store_tile(kregA, vregA, n0);
+        __syncthreads();
+        issue_loads(kregA, vregA, n0 + 2 * kStateTile);
+        multiply_tile();
+        __syncthreads();
+        store_tile(kregB, vregB, n0 + kStateTile);
+        __syncthreads();
+        issue_loads(kregB, vregB, n0 + 3 * kStateTile);
+        multiply_tile();
+        __syncthreads();
+        n0 += 2 * kStateTile;
+    }
+    if (n_tiles & 1) {
+        store_tile(kregA, vregA, n0);
+        __syncthreads();
+        multiply_tile();
         __syncthreads();
     }
 
-    // blocks -> FP32 images of (S, z) in LDS (rows of DP floats, then z), reusing the tile space. Wavefronts that share a
-    // block (each took a share of every tile's tokens) write one image each; the images are added in a fixed order on the
-    // way out, so the result does not depend on which wavefront finishes first. Every element of an image is written:
-    // the NBLK blocks cover S, the blocks of the first block row cover z.
+    // blocks -> FP32 images of (S, z) in LDS (rows of DP floats, then one more row for z where it is not a row of S),
+    // reusing the tile space. Wavefronts that share a rectangle (each took a share of every tile's tokens) write one
+    // image each; the images are added in a fixed order on the way out, so the result does not depend on which wavefront
+    // finishes first. Every element that is read back is written: the rectangles tile S, those of the first block row
+    // cover the separate z row.
     float* const Sl = reinterpret_cast<float*>(lds);
     if (active) {
         float* const img = Sl + ts * SG::S_FLOATS;
-        const int j = 32 * cb + lq;
 #pragma unroll
-        for (int bb = 0; bb < 4; ++bb)
+        for (int jb = 0; jb < SG::CBW; ++jb) {
+            const int j = 32 * (cb0 + jb) + lq;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int i = 32 * rb + 8 * bb + 4 * lh + e;
-                img[i * G::DP + j] = acc[4 * bb + e];
-            }
-        if (does_z && lh == 0) img[G::DP * G::DP + j] = zacc[0];
+            for (int ib = 0; ib < SG::RBW; ++ib)
+#pragma unroll
+                for (int bb = 0; bb < 4; ++bb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int i = 32 * (rb0 + ib) + 8 * bb + 4 * lh + e;
+                        img[i * G::DP + j] = acc[ib][jb][4 * bb + e];
+                    }
+            if (does_z && lh == 0) img[G::DP * G::DP + j] = zacc[jb][0];
+        }
     }
     __syncthreads();
     // this group's (S, z): straight into the state when it covers the whole (batch, head), else into its partial slot
     float* const S = p.part ? p.part + (static_cast<long>(bh) * p.n_part + chunk) * G::WS_FLOATS
                             : p.ws + static_cast<long>(bh) * G::WS_FLOATS;
+    const float* const old_state = p.add_to_state ? S : nullptr;      // the only group of this (batch, head)
     for (int idx = tid; idx < (D + 1) * (D / 4); idx += kStateThreads) {
-        const int i = idx / (D / 4), j = (idx - i * (D / 4)) * 4;     // i == D: the z row, kept behind the DP rows of S
-        const float* const src = Sl + (i < D ? i : G::DP) * G::DP + j;
+        const int i = idx / (D / 4), j = (idx - i * (D / 4)) * 4;     // i == D: the z row
+        const float* const src = Sl + (i < D ? i : SG::Z_ROW) * G::DP + j;
         f32x4 v = *reinterpret_cast<const f32x4*>(src);
 #pragma unroll
         for (int t = 1; t < SG::NTS; ++t) v += *reinterpret_cast<const f32x4*>(src + t * SG::S_FLOATS);
-        if (p.add_to_state) v += *reinterpret_cast<const f32x4*>(S + i * D + j);   // the only group of this (batch, head)
+        if (old_state) v += *reinterpret_cast<const f32x4*>(old_state + i * D + j);
         *reinterpret_cast<f32x4*>(S + i * D + j) = v;
     }
 }
