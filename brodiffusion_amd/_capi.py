@@ -54,7 +54,7 @@ class MiSdpaArgs(C.Structure):
         ("seg_q_end", C.c_int32 * MI_MAX_SEGMENTS), ("seg_k_end", C.c_int32 * MI_MAX_SEGMENTS),
         ("seg_causal", C.c_int32 * MI_MAX_SEGMENTS),
         ("rope_cos_q", C.c_void_p), ("rope_sin_q", C.c_void_p), ("rope_cos_k", C.c_void_p), ("rope_sin_k", C.c_void_p),
-        ("rope_k_scratch", C.c_void_p),
+        ("rope_split_half", C.c_int32), ("rope_k_scratch", C.c_void_p),
         ("logit_bias", C.c_void_p), ("bias_q0", C.c_int32), ("bias_cols", C.c_int32), ("bias_row_stride", C.c_int64),
         ("lse_out", C.c_void_p),
         ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
@@ -90,7 +90,8 @@ class MiHeadnormRopeArgs(C.Structure):
         ("x", C.c_void_p), ("out", C.c_void_p), ("gain", C.c_void_p), ("cos", C.c_void_p), ("sin", C.c_void_p),
         ("eps", C.c_float), ("rows", C.c_int32), ("num_heads", C.c_int32), ("head_dim", C.c_int32),
         ("x_row_stride", C.c_int64), ("out_row_stride", C.c_int64),
-        ("out2", C.c_void_p), ("out2_rows", C.c_int32), ("out2_row_stride", C.c_int64), ("stream", C.c_void_p),
+        ("out2", C.c_void_p), ("out2_rows", C.c_int32), ("out2_row_stride", C.c_int64), ("split_half", C.c_int32),
+        ("stream", C.c_void_p),
     ]
 
 

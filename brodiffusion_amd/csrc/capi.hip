@@ -187,6 +187,10 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
     for (const void* t : tabs)
         if (t && !mi::aligned16(t)) return fail("mi_sdpa_forward: rope tables must be 16-byte aligned");
     p.cos_q = a->rope_cos_q; p.sin_q = a->rope_sin_q; p.cos_k = a->rope_cos_k; p.sin_k = a->rope_sin_k;
+    if (a->rope_split_half != 0 && a->rope_split_half != 1) return fail("mi_sdpa_forward: rope_split_half must be 0 or 1");
+    p.rope_split = a->rope_split_half;
+    if (p.rope_split && p.cos_k && a->kv_len > 0 && !a->rope_k_scratch)
+        return fail("mi_sdpa_forward: split-half RoPE on K needs rope_k_scratch (K is rotated tile by tile for adjacent pairs only)");
     p.inv_scale = 1.0f / scale;
     if (a->logit_bias) {
         if (a->batch != 1) return fail("mi_sdpa_forward: logit_bias needs batch 1");
@@ -258,6 +262,7 @@ int mi_sdpa_forward(const mi_sdpa_args* a) {
             r.cos = p.cos_k; r.sin = p.sin_k;
             r.rows = a->kv_len; r.num_heads = Hkv; r.head_dim = a->head_dim;
             r.x_row_stride = p.k_rs; r.out_row_stride = Dkv;
+            r.split_half = a->rope_split_half;
             r.stream = mi::resolve_stream(a->stream);
             if (mi_rope_apply(&r) != 0) return -1;
         }

@@ -72,6 +72,7 @@ struct SdpaDev {
     int seg_causal[MI_MAX_SEGMENTS];
     const float* cos_q; const float* sin_q;
     const float* cos_k; const float* sin_k;
+    int rope_split;               // 0: adjacent pairs, 1: the two halves of a head (Q only: K then arrives rotated)
     int n_q_tiles; int n_blocks;  // logical work items = B*H*n_q_tiles
     // additive logit bias (natural-log units, added to the scaled score) for query rows >= bias_q0 and keys < bias_cols
     const float* bias; int bias_q0, bias_cols; long bias_rs;

@@ -61,7 +61,39 @@ __global__ void __launch_bounds__(256) rope_split_kernel(const T* __restrict__ x
     }
 }
 
-// Per-head RMS normalisation fused with the rotation (adjacent pairs) and an optional second destination for the
+// Split-half pairs where half a head is whole 16-byte chunks (d % 16 == 0): one thread rotates the 8 pairs formed by
+// chunk c of the lower half and chunk c of the upper half. Same arithmetic as rope_split_kernel.
+template <typename T>
+__global__ void __launch_bounds__(256) rope_split_vec_kernel(const T* x, T* out, const float* __restrict__ cs,
+                                                             const float* __restrict__ sn, int rows, int H, int d, long x_rs,
+                                                             long o_rs, int per_head) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    const int half = d / 2;
+    const int upr = H * half / 8;  // units (8 pairs) per row
+    const long total = static_cast<long>(rows) * upr;
+    for (long idx = blockIdx.x * 256L + threadIdx.x; idx < total; idx += gridDim.x * 256L) {
+        const int r = static_cast<int>(idx / upr);
+        const int u = static_cast<int>(idx - static_cast<long>(r) * upr);
+        const int h = u / (half / 8);
+        const int pp = (u - h * (half / 8)) * 8;   // first pair of the unit
+        const long trow = per_head ? static_cast<long>(r) * H + h : r;
+        const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + trow * half + pp), c1 = *reinterpret_cast<const f32x4*>(cs + trow * half + pp + 4);
+        const f32x4 s0 = *reinterpret_cast<const f32x4*>(sn + trow * half + pp), s1 = *reinterpret_cast<const f32x4*>(sn + trow * half + pp + 4);
+        t8 lo = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(x + r * x_rs + h * d + pp));
+        t8 hi = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(x + r * x_rs + h * d + pp + half));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float a = static_cast<float>(lo[e]), b = static_cast<float>(hi[e]);
+            const float c = e < 4 ? c0[e & 3] : c1[e & 3], sv = e < 4 ? s0[e & 3] : s1[e & 3];
+            lo[e] = static_cast<T>(rope_re(a, b, c, sv));
+            hi[e] = static_cast<T>(rope_im(a, b, c, sv));
+        }
+        *reinterpret_cast<u32x4*>(out + r * o_rs + h * d + pp) = __builtin_bit_cast(u32x4, lo);
+        *reinterpret_cast<u32x4*>(out + r * o_rs + h * d + pp + half) = __builtin_bit_cast(u32x4, hi);
+    }
+}
+
+// Per-head RMS normalisation fused with the rotation (adjacent or split-half pairs) and an optional second destination for the
 // leading rows: y = RoPE(x * rsqrt(mean_d(x^2) + eps) * gain), one read of x, one rounding. One thread per 16-byte
 // chunk; the CPR = d/8 threads of a head row are neighbouring lanes of one wavefront (CPR is a power of two <= 16),
 // so the sum of squares is CPR-lane butterfly. Everything is FP32 between the load and the single rounding.
@@ -69,7 +101,7 @@ template <typename T, int CPR>
 __global__ void __launch_bounds__(256) headnorm_rope_kernel(const T* x, T* out, T* out2,
                                                             const T* __restrict__ gain, const float* __restrict__ cs,
                                                             const float* __restrict__ sn, int rows, int H, float eps,
-                                                            long x_rs, long o_rs, long o2_rs, int out2_rows) {
+                                                            long x_rs, long o_rs, long o2_rs, int out2_rows, int split_half) {
     typedef T t8 __attribute__((ext_vector_type(8)));
     constexpr int d = CPR * 8;
     const int cpr = H * CPR;
@@ -91,7 +123,23 @@ __global__ void __launch_bounds__(256) headnorm_rope_kernel(const T* x, T* out, 
 #pragma unroll
         for (int e = 0; e < 8; ++e) f[e] = f[e] * inv * static_cast<float>(g[e]);
         t8 o;
-        if (cs != nullptr) {
+        if (cs != nullptr && split_half) {
+            // the partner of chunk c is chunk c ^ (CPR / 2) of the same head row, held by the lane CPR / 2 away; the lower
+            // half yields the real parts, the upper half the imaginary parts of the 8 pairs the two chunks form
+            const bool upper = dc >= d / 2;
+            const int pp = upper ? dc - d / 2 : dc;
+            const f32x4 c0 = *reinterpret_cast<const f32x4*>(cs + static_cast<long>(r) * (d / 2) + pp);
+            const f32x4 c1 = *reinterpret_cast<const f32x4*>(cs + static_cast<long>(r) * (d / 2) + pp + 4);
+            const f32x4 s0 = *reinterpret_cast<const f32x4*>(sn + static_cast<long>(r) * (d / 2) + pp);
+            const f32x4 s1 = *reinterpret_cast<const f32x4*>(sn + static_cast<long>(r) * (d / 2) + pp + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float other = __shfl_xor(f[e], CPR / 2);
+                const float a = upper ? other : f[e], b = upper ? f[e] : other;
+                const float c = e < 4 ? c0[e & 3] : c1[e & 3], sv = e < 4 ? s0[e & 3] : s1[e & 3];
+                o[e] = static_cast<T>(upper ? rope_im(a, b, c, sv) : rope_re(a, b, c, sv));
+            }
+        } else if (cs != nullptr) {
             const f32x4 cv = *reinterpret_cast<const f32x4*>(cs + static_cast<long>(r) * (d / 2) + dc / 2);
             const f32x4 sv = *reinterpret_cast<const f32x4*>(sn + static_cast<long>(r) * (d / 2) + dc / 2);
 #pragma unroll
@@ -140,7 +188,7 @@ int launch_headnorm(const mi_headnorm_rope_args* a, long x_rs, long o_rs, long o
 #define MI_HEADNORM_CASE(CPR)                                                                                          \
     case CPR * 8:                                                                                                      \
         hipLaunchKernelGGL((headnorm_rope_kernel<T, CPR>), dim3(blocks), dim3(256), 0, st, x, o, o2, g, a->cos, a->sin, \
-                           a->rows, a->num_heads, a->eps, x_rs, o_rs, o2_rs, r2);                                      \
+                           a->rows, a->num_heads, a->eps, x_rs, o_rs, o2_rs, r2, a->split_half);                       \
         break;
     switch (a->head_dim) {
         MI_HEADNORM_CASE(4)
@@ -163,7 +211,14 @@ int launch(const mi_rope_args* a, long x_rs, long o_rs, hipStream_t st) {
     if (blocks < 1) blocks = 1;
     const T* x = static_cast<const T*>(a->x);
     T* o = static_cast<T*>(a->out);
-    if (a->split_half) {
+    const uintptr_t al = reinterpret_cast<uintptr_t>(a->x) | reinterpret_cast<uintptr_t>(a->out) | reinterpret_cast<uintptr_t>(a->cos) |
+                         reinterpret_cast<uintptr_t>(a->sin);
+    if (a->split_half && a->head_dim % 16 == 0 && x_rs % 8 == 0 && o_rs % 8 == 0 && (al & 15u) == 0) {
+        long vb = (static_cast<long>(a->rows) * a->num_heads * (a->head_dim / 16) + 255) / 256;
+        if (vb > 256 * 32) vb = 256 * 32;
+        hipLaunchKernelGGL(rope_split_vec_kernel<T>, dim3(vb), dim3(256), 0, st, x, o, a->cos, a->sin, a->rows, a->num_heads,
+                           a->head_dim, x_rs, o_rs, a->per_head);
+    } else if (a->split_half) {
         hipLaunchKernelGGL(rope_split_kernel<T>, dim3(blocks), dim3(256), 0, st, x, o, a->cos, a->sin, a->rows,
                            a->num_heads, a->head_dim, x_rs, o_rs, a->per_head);
     } else {
@@ -217,6 +272,7 @@ extern "C" int mi_headnorm_rope(const mi_headnorm_rope_args* a) {
     if ((a->cos == nullptr) != (a->sin == nullptr)) return fail("mi_headnorm_rope: cos and sin must be given together");
     if (!(a->eps >= 0.f)) return fail("mi_headnorm_rope: eps must be >= 0");
     if (a->out2_rows < 0 || a->out2_rows > a->rows) return fail("mi_headnorm_rope: out2_rows %d outside 0..rows", a->out2_rows);
+    if (a->split_half != 0 && a->split_half != 1) return fail("mi_headnorm_rope: split_half must be 0 or 1");
     const long D = static_cast<long>(a->num_heads) * a->head_dim;
     const long x_rs = a->x_row_stride ? a->x_row_stride : D;
     const long o_rs = a->out_row_stride ? a->out_row_stride : D;

@@ -160,7 +160,7 @@ __device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p
     constexpr int NCH = ROWS * CPRK;
     constexpr int NI = (NCH + NT - 1) / NT;
     const int last_row = last_row_override >= 0 ? last_row_override : p.Lq - 1;   // (a packed sequence has its own length)
-    const bool rope = p.cos_q != nullptr;
+    const bool rope = p.cos_q != nullptr && !p.rope_split;
     u32x4 raw[NI];
     f32x4 cs[NI], sn[NI];
 #pragma unroll
@@ -183,6 +183,31 @@ __device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p
         else if (q_scale != 1.f) v = scale_chunk<T>(v, q_scale);
         if (q0 + row > last_row || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
         if (idx < NCH) *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
+    }
+    // Split-half pairs (x[p], x[p + D/2]) sit in different 16-byte chunks, so that rotation is a second pass over the
+    // staged rows: one thread takes 4 pairs, i.e. 8 bytes from each half of a row (and the 4 table entries they share),
+    // and writes them back. Same arithmetic and single rounding as the stand-alone pass; rows past the end are zero.
+    if (p.cos_q != nullptr && p.rope_split) {
+        typedef T t4 __attribute__((ext_vector_type(4)));
+        constexpr int UPR = D / 8;             // units of 4 pairs per row
+        __syncthreads();
+        for (int u = tid; u < ROWS * UPR; u += NT) {
+            const int row = u / UPR, g = u - row * UPR;
+            const int qrow = min(q0 + row, last_row);
+            const f32x4 c4 = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + g * 4);
+            const f32x4 s4 = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + g * 4);
+            t4* const lo_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + g * 8);
+            t4* const hi_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + D + g * 8);
+            t4 lo = *lo_p, hi = *hi_p;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float a = static_cast<float>(lo[e]), b = static_cast<float>(hi[e]);
+                lo[e] = static_cast<T>(rope_re(a, b, c4[e], s4[e]) * q_scale);
+                hi[e] = static_cast<T>(rope_im(a, b, c4[e], s4[e]) * q_scale);
+            }
+            *lo_p = lo;
+            *hi_p = hi;
+        }
     }
 }
 

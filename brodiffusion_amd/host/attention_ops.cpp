@@ -110,6 +110,10 @@ void flash_attention_varlen_forward(const Tensor& Q, const Tensor& K, const Tens
     run_sdpa(op, a);
 }
 
+static bool g_rope_split_half = false;
+void set_rope_split_half(bool split_half) { g_rope_split_half = split_half; }
+bool rope_split_half() { return g_rope_split_half; }
+
 static void rope_impl(const char* op, const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads,
                       Tensor& out, bool per_head) {
     need_gpu(op, X); need_gpu(op, cos); need_gpu(op, sin);
@@ -127,6 +131,7 @@ static void rope_impl(const char* op, const Tensor& X, const Tensor& cos, const 
     a.x = X.data; a.out = out.data;
     a.cos = static_cast<const float*>(cos.data); a.sin = static_cast<const float*>(sin.data);
     a.rows = X.rows; a.num_heads = num_heads; a.head_dim = head_dim; a.per_head = per_head ? 1 : 0;
+    a.split_half = g_rope_split_half ? 1 : 0;
     check(op, mi_rope_apply(&a));
 }
 void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out) {
@@ -525,6 +530,7 @@ void headnorm_rope(const Tensor& X, const Tensor& gain, float eps, const Tensor*
     a.cos = cos ? static_cast<const float*>(cos->data) : nullptr;
     a.sin = sin ? static_cast<const float*>(sin->data) : nullptr;
     a.eps = eps;
+    a.split_half = bt::rope_split_half() ? 1 : 0;
     a.rows = X.rows; a.num_heads = num_heads; a.head_dim = head_dim;
     if (cache_out && cache_rows > 0) {
         if (cache_out->data == nullptr || cache_out->rows != cache_rows || cache_out->cols != X.cols || cache_out->dtype != X.dtype)
@@ -545,6 +551,7 @@ void joint_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Te
     set_rope(a, op, &cos, &sin, K.rows, false);
     Kr.resize(K.rows, K.cols, K.dtype, K.device);  // receives RoPE(K), as in the reference
     a.rope_k_scratch = Kr.data;
+    a.rope_split_half = bt::rope_split_half() ? 1 : 0;
     run_sdpa(op, a);
 }
 
@@ -598,6 +605,7 @@ void gqa_attention_masked(const Tensor& Q, const Tensor& K, const Tensor& V, con
     if (cos) {
         Kr.resize(K.rows, K.cols, K.dtype, K.device);
         a.rope_k_scratch = Kr.data;
+        a.rope_split_half = bt::rope_split_half() ? 1 : 0;
     }
     run_sdpa(op, a);
 }

@@ -36,6 +36,12 @@ void flash_attention_gqa_forward(const Tensor& Q, const Tensor& K, const Tensor&
                                  int num_kv_heads, bool causal, Tensor& out);
 void flash_attention_varlen_forward(const Tensor& Q, const Tensor& K, const Tensor& V, const int32_t* cu_q, const int32_t* cu_k,
                                     int n_seqs, int max_q, int max_k, int num_heads, int head_dim, bool causal, Tensor& out);
+// Pair convention of every rotation in this layer (rope_apply, rope_apply_perhead, and the rotations fused into
+// joint_attention, gqa_attention_masked, joint_attention_traced and headnorm_rope): false (default) pairs adjacent
+// elements (x[2p], x[2p+1]), true pairs the two halves of a head (x[p], x[p + head_dim/2]). brotensor's rope_apply has
+// one fixed convention that the reference's sources do not state; a binding sets this once, to whatever brotensor does.
+void set_rope_split_half(bool split_half);
+bool rope_split_half();
 void rope_apply(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
 void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, int head_dim, int num_heads, Tensor& out);
 

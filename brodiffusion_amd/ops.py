@@ -113,7 +113,7 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
                  kv_valid_len: Optional[torch.Tensor] = None, key_mask: Optional[torch.Tensor] = None,
                  rope_q: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                 rope_k_scratch: Optional[torch.Tensor] = None, split_scratch=None,
+                 rope_k_scratch: Optional[torch.Tensor] = None, rope_split_half: bool = False, split_scratch=None,
                  logit_bias: Optional[torch.Tensor] = None, bias_q0: int = 0, lse_out: Optional[torch.Tensor] = None,
                  op: str = "sdpa_forward") -> torch.Tensor:
     """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None).
@@ -197,6 +197,7 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
             a.rope_cos_q, a.rope_sin_q = cs.data_ptr(), sn.data_ptr()
         else:
             a.rope_cos_k, a.rope_sin_k = cs.data_ptr(), sn.data_ptr()
+    a.rope_split_half = int(bool(rope_split_half))
     if rope_k_scratch is not None:
         if rope_k is None:
             _fail(op, "rope_k_scratch given without rope_k tables")
@@ -621,7 +622,7 @@ def scale_rows(X, scale: float = 1.0, row_scale: Optional[torch.Tensor] = None, 
 
 
 def headnorm_rope(X, gain, eps: float, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
-                  cache_out: Optional[torch.Tensor] = None):
+                  cache_out: Optional[torch.Tensor] = None, split_half: bool = False):
     """headnorm + rope_apply of the DiT blocks (src/dit/qwenimage21_forward.cpp:582-585, src/dit/flux.cpp:462-469) in
     one pass: per (row, head) RMS normalisation with `gain` (head_dim), then the rotation (cos = sin = None: the
     normalisation alone). cache_out (rows <= X's rows): its rows also receive the result — the prefix rows of K going
@@ -648,6 +649,7 @@ def headnorm_rope(X, gain, eps: float, cos, sin, head_dim: int, num_heads: int, 
                 _fail(op, "cos/sin must be contiguous float32 (L, head_dim/2)")
         a.cos, a.sin = cos.data_ptr(), sin.data_ptr()
     a.eps = eps
+    a.split_half = int(bool(split_half))
     a.rows, a.num_heads, a.head_dim = X.shape[0], num_heads, head_dim
     a.x_row_stride, a.out_row_stride = X.stride(0), out.stride(0)
     if cache_out is not None:
@@ -661,11 +663,12 @@ def headnorm_rope(X, gain, eps: float, cos, sin, head_dim: int, num_heads: int, 
 
 
 def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optional[torch.Tensor] = None,
-                    Qr: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None):
+                    Qr: Optional[torch.Tensor] = None, Kr: Optional[torch.Tensor] = None, split_half: bool = False):
     """Full-bidirectional joint attention with RoPE on Q and K (include/brodiffusion/dit/common.h:74-88).
     Q is rotated while it is loaded. With a Kr scratch (K's shape and dtype) K is rotated into it by one
     pass and, as in the reference, Kr holds RoPE(K) afterwards; without one K is rotated tile by tile
-    inside the attention kernel (slower). Qr is accepted and left untouched."""
+    inside the attention kernel (slower; adjacent pairs only). Qr is accepted and left untouched. split_half selects the
+    pair convention of the rotation as in rope_apply."""
     op = "joint_attention"
     if Q.dim() != 2 or Q.shape[1] != head_dim * num_heads:
         _fail(op, "D must equal head_dim * num_heads")
@@ -673,7 +676,8 @@ def joint_attention(Q, K, V, cos, sin, head_dim: int, num_heads: int, out: Optio
         _fail(op, "Q/K/V must share shape (L, D)")
     if Kr is not None and (Kr.shape != K.shape or Kr.dtype != K.dtype):
         _fail(op, "Kr must have K's shape and dtype")
-    return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), rope_k_scratch=Kr, op=op)
+    return sdpa_forward(Q, K, V, num_heads, out=out, rope_q=(cos, sin), rope_k=(cos, sin), rope_k_scratch=Kr,
+                        rope_split_half=split_half, op=op)
 
 
 def attention_map_avg(q, k, lse, num_heads: int, *, scale: Optional[float] = None, logit_bias: Optional[torch.Tensor] = None,

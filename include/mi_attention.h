@@ -89,7 +89,7 @@ MI_API int mi_memset_async(void* dst, int value, size_t bytes, void* stream);
  *   - rope_*: RoPE applied to Q as it is loaded and to the rows of `k` (as they are loaded, or by
  *     one pass into rope_k_scratch when the caller lends one), replacing the two bt::rope_apply
  *     passes of dit::joint_attention (src/dit/common.cpp:188-196).
- *     Adjacent-pair convention (x[2p], x[2p+1]); prefix rows are taken as already rotated
+ *     Adjacent pairs (x[2p], x[2p+1]) or, with rope_split_half, the two halves of a head; prefix rows are taken as already rotated
  *     (the reference caches post-RoPE K, qwenimage21_forward.cpp:587-597);
  *   - block-causal segments: the per-segment calls of the prefill form
  *     (qwenimage21_forward.cpp:650-676) in one launch; key tiles no query row of a work
@@ -140,6 +140,11 @@ typedef struct mi_sdpa_args {
     const float* rope_sin_q;
     const float* rope_cos_k;     /* device FP32 (kv_len, head_dim/2) or NULL; rows of `k` only */
     const float* rope_sin_k;
+    int32_t rope_split_half;     /* 0: the rotation pairs adjacent elements (x[2p], x[2p+1]); 1: it pairs the two halves of a head,
+                                    (x[p], x[p + head_dim/2]), as mi_rope_apply's split_half. Applies to Q as it is loaded and to the
+                                    pass that rotates K into rope_k_scratch; with 1 the scratch is required when rope_cos_k is given
+                                    (the tile-by-tile rotation of K exists for adjacent pairs only). Which convention brotensor's
+                                    rope_apply uses cannot be read from the reference: the binding picks it per call site */
     void* rope_k_scratch;        /* device (batch, kv_len, kv_heads*head_dim) of `dtype`, dense, or NULL. With rope_cos_k:
                                     K is rotated into it by one bandwidth-bound pass and attention reads the rotated copy
                                     (fastest form); afterwards it holds RoPE(K) like the Kr scratch of dit::joint_attention
@@ -232,8 +237,8 @@ MI_API int mi_rope_apply(const mi_rope_args* args);
  * out = RoPE(x * rsqrt(mean over head_dim of x^2 + eps) * gain) per (row, head): what the DiT blocks do between the
  * Q/K projections and attention as two passes, bt::rms_norm_forward on the (L*heads, head_dim) view followed by
  * bt::rope_apply (headnorm, src/dit/qwenimage21_forward.cpp:53-63 and :582-585; src/dit/flux.cpp:462-469). One read
- * of x, FP32 in between, a single rounding. gain: (head_dim) of `dtype`. cos / sin: FP32 (rows, head_dim/2), adjacent
- * pairs, or both NULL for the normalisation alone. out2 (optional): rows [0, out2_rows) are written there as well —
+ * of x, FP32 in between, a single rounding. gain: (head_dim) of `dtype`. cos / sin: FP32 (rows, head_dim/2), pairs as
+ * split_half says, or both NULL for the normalisation alone. out2 (optional): rows [0, out2_rows) are written there as well —
  * the prefix rows of K going into the prefix cache while the full K goes to attention
  * (qwenimage21_forward.cpp:587-597). In-place (out == x) is allowed. head_dim 32, 64 or 128. */
 typedef struct mi_headnorm_rope_args {
@@ -250,6 +255,7 @@ typedef struct mi_headnorm_rope_args {
     void* out2;
     int32_t out2_rows;
     int64_t out2_row_stride;
+    int32_t split_half;      /* 0: adjacent pairs (x[2p], x[2p+1]); 1: pairs (x[p], x[p + head_dim/2]) */
     void* stream;
 } mi_headnorm_rope_args;
 MI_API int mi_headnorm_rope(const mi_headnorm_rope_args* args);

@@ -36,13 +36,16 @@ def test_header_symbols_exported(capi):
 
 def test_struct_sizes_match_c(capi, tmp_path):
     src = tmp_path / "sz.c"
-    src.write_text('#include "mi_attention.h"\n#include <stdio.h>\nint main(void){printf("%zu %zu %zu %zu\\n",'
-                   'sizeof(mi_sdpa_args),sizeof(mi_rope_args),sizeof(mi_linear_attn_args),sizeof(mi_device_info_t));return 0;}\n')
+    src.write_text('#include "mi_attention.h"\n#include <stdio.h>\nint main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",'
+                   'sizeof(mi_sdpa_args),sizeof(mi_rope_args),sizeof(mi_linear_attn_args),sizeof(mi_device_info_t),'
+                   'sizeof(mi_headnorm_rope_args),sizeof(mi_scale_rows_args),sizeof(mi_attention_map_args),sizeof(mi_linear_args),'
+                   'sizeof(mi_attn_block_args));return 0;}\n')
     exe = tmp_path / "sz"
     subprocess.run(["gcc", "-std=c99", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     sizes = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
     assert sizes == [C.sizeof(capi.MiSdpaArgs), C.sizeof(capi.MiRopeArgs), C.sizeof(capi.MiLinearAttnArgs),
-                     C.sizeof(capi.MiDeviceInfo)]
+                     C.sizeof(capi.MiDeviceInfo), C.sizeof(capi.MiHeadnormRopeArgs), C.sizeof(capi.MiScaleRowsArgs),
+                     C.sizeof(capi.MiAttentionMapArgs), C.sizeof(capi.MiLinearArgs), C.sizeof(capi.MiAttnBlockArgs)]
 
 
 def test_argument_validation_without_launch(capi):
