@@ -24,7 +24,7 @@ EXPORTS = [
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
     "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_attention_map_avg", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported", "mi_linear_attn_relu_forward_static_scratch",
-    "mi_linear_forward", "mi_linear_geglu_forward", "mi_add_inplace", "mi_add_row_bias", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
+    "mi_linear_forward", "mi_linear_geglu_forward", "mi_add_inplace", "mi_add_row_bias", "mi_rms_norm_forward", "mi_flash_attention_scratch_bytes", "mi_flash_attention_qkvo_forward",
     "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv",
 ]
 
@@ -113,7 +113,7 @@ class MiLinearAttnArgs(C.Structure):
         ("k_row_stride", C.c_int64), ("k_batch_stride", C.c_int64),
         ("v_row_stride", C.c_int64), ("v_batch_stride", C.c_int64),
         ("o_row_stride", C.c_int64), ("o_batch_stride", C.c_int64),
-        ("eps", C.c_float), ("accumulate_state", C.c_int32),
+        ("eps", C.c_float), ("accumulate_state", C.c_int32), ("accumulate_weight", C.c_float),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("stream", C.c_void_p),
     ]
@@ -191,6 +191,8 @@ def lib() -> C.CDLL:
         L.mi_linear_geglu_forward.argtypes = [C.POINTER(MiLinearArgs)]
         L.mi_add_inplace.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p]
         L.mi_add_row_bias.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int32, C.c_void_p]
+        L.mi_rms_norm_forward.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int64, C.c_int64, C.c_float,
+                                          C.c_int32, C.c_void_p]
         L.mi_flash_attention_scratch_bytes.argtypes = [C.c_int32] * 5
         L.mi_flash_attention_scratch_bytes.restype = C.c_size_t
         for name in ("mi_flash_attention_qkvo_forward", "mi_flash_attention_q_with_kv_cached_forward", "mi_flash_attention_project_kv"):

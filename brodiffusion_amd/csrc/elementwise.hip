@@ -50,6 +50,48 @@ __global__ void __launch_bounds__(256) add_row_bias_kernel(T* y, const T* bias, 
     }
 }
 
+// RMS normalisation of whole rows: one work group per row (grid-stride over rows), the row held in registers between
+// the sum of squares and the scaling (up to kRmsChunks 16-byte chunks per thread), FP32 arithmetic, one rounding.
+constexpr int kRmsChunks = 8;   // 256 threads x 8 chunks x 8 elements = rows of up to 16384 columns
+template <typename T>
+__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const T* x, const T* __restrict__ gain, T* out, int rows, int cols,
+                                                            long x_rs, long o_rs, float eps) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    __shared__ float red[4];
+    const int cpr = cols / 8;
+    const int tid = threadIdx.x;
+    for (int r = blockIdx.x; r < rows; r += gridDim.x) {
+        t8 v[kRmsChunks];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < kRmsChunks; ++i) {
+            const int c = tid + 256 * i;
+            if (c < cpr) {
+                v[i] = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(x + static_cast<long>(r) * x_rs + c * 8));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { const float f = static_cast<float>(v[i][e]); ss = __builtin_fmaf(f, f, ss); }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off);
+        __syncthreads();                      // the previous row's readers are done with `red`
+        if ((tid & 63) == 0) red[tid >> 6] = ss;
+        __syncthreads();
+        const float inv = __builtin_amdgcn_rsqf((red[0] + red[1] + red[2] + red[3]) / static_cast<float>(cols) + eps);
+#pragma unroll
+        for (int i = 0; i < kRmsChunks; ++i) {
+            const int c = tid + 256 * i;
+            if (c < cpr) {
+                const t8 g = __builtin_bit_cast(t8, *reinterpret_cast<const u32x4*>(gain + c * 8));
+                t8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = static_cast<T>(static_cast<float>(v[i][e]) * inv * static_cast<float>(g[e]));
+                *reinterpret_cast<u32x4*>(out + static_cast<long>(r) * o_rs + c * 8) = __builtin_bit_cast(u32x4, o);
+            }
+        }
+    }
+}
+
 long grid_for(long work) {
     long blocks = (work + 255) / 256;
     return blocks < 1 ? 1 : (blocks > 256 * 32 ? 256 * 32 : blocks);
@@ -100,6 +142,34 @@ int mi_add_row_bias(void* y, const void* bias, int32_t rows, int32_t cols, int64
         return fail("mi_add_row_bias: dtype %d not supported", dtype);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("mi_add_row_bias launch: %s", hipGetErrorString(e));
+    return 0;
+}
+
+int mi_rms_norm_forward(const void* x, const void* gain, void* out, int32_t rows, int32_t cols, int64_t x_row_stride,
+                        int64_t out_row_stride, float eps, int32_t dtype, void* stream) {
+    mi::clear_error();
+    if (rows < 0 || cols <= 0 || cols % 8 != 0) return fail("mi_rms_norm_forward: cols must be a positive multiple of 8, rows >= 0");
+    if (cols > 256 * 8 * mi::kRmsChunks) return fail("mi_rms_norm_forward: rows of more than %d columns are not supported", 256 * 8 * mi::kRmsChunks);
+    if (rows == 0) return 0;
+    if (!x || !gain || !out) return fail("mi_rms_norm_forward: null tensor");
+    if (!(eps >= 0.f)) return fail("mi_rms_norm_forward: eps must be >= 0");
+    const long x_rs = x_row_stride ? x_row_stride : cols, o_rs = out_row_stride ? out_row_stride : cols;
+    if (x_rs < cols || o_rs < cols || x_rs % 8 != 0 || o_rs % 8 != 0)
+        return fail("mi_rms_norm_forward: row strides must be multiples of 8 elements and at least cols");
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(gain) | reinterpret_cast<uintptr_t>(out)) & 15u)
+        return fail("mi_rms_norm_forward: pointers must be 16-byte aligned");
+    hipStream_t st = mi::resolve_stream(stream);
+    const dim3 grid(static_cast<unsigned>(rows < 256 * 16 ? rows : 256 * 16));
+    if (dtype == MI_DTYPE_BF16)
+        hipLaunchKernelGGL(mi::rms_norm_rows_kernel<__bf16>, grid, dim3(256), 0, st, static_cast<const __bf16*>(x), static_cast<const __bf16*>(gain),
+                           static_cast<__bf16*>(out), rows, cols, x_rs, o_rs, eps);
+    else if (dtype == MI_DTYPE_F16)
+        hipLaunchKernelGGL(mi::rms_norm_rows_kernel<_Float16>, grid, dim3(256), 0, st, static_cast<const _Float16*>(x), static_cast<const _Float16*>(gain),
+                           static_cast<_Float16*>(out), rows, cols, x_rs, o_rs, eps);
+    else
+        return fail("mi_rms_norm_forward: dtype %d not supported", dtype);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail("mi_rms_norm_forward launch: %s", hipGetErrorString(e));
     return 0;
 }
 

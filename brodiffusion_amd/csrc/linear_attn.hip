@@ -81,6 +81,7 @@ struct LinDev {
     float* part;    // partial states of the token chunks: [(b,h)][chunk][D*D + D], or null
     int n_part;     // chunks per (b,h) in `part`
     int add_to_state;   // no partials: this group's (S, z) is added to the state instead of replacing it
+    float old_weight;   // weight of the state that was there before, where the call accumulates
     int tokens_per_group;
     int n_chunks;   // token chunks per (batch, head)
     int n_blocks;   // work groups with work = B * H * n_chunks
@@ -335,17 +336,17 @@ __global__ void __launch_bounds__(kStateThreads) linattn_state_kernel(const LinD
         f32x4 v = *reinterpret_cast<const f32x4*>(src);
 #pragma unroll
         for (int t = 1; t < SG::NTS; ++t) v += *reinterpret_cast<const f32x4*>(src + t * SG::S_FLOATS);
-        if (old_state) v += *reinterpret_cast<const f32x4*>(old_state + i * D + j);
+        if (old_state) v += *reinterpret_cast<const f32x4*>(old_state + i * D + j) * p.old_weight;
         *reinterpret_cast<f32x4*>(S + i * D + j) = v;
     }
 }
 
 // state (+)= sum of the partial states of the token chunks, one element per thread and step.
 __global__ void __launch_bounds__(256) linattn_reduce_kernel(float* ws, const float* part, int n_part, long ws_floats4, long total4,
-                                                             int accumulate) {
+                                                             int accumulate, float old_weight) {
     for (long i = blockIdx.x * 256L + threadIdx.x; i < total4; i += gridDim.x * 256L) {
         const long bh = i / ws_floats4, off = i - bh * ws_floats4;
-        f32x4 v = accumulate ? reinterpret_cast<const f32x4*>(ws)[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 v = accumulate ? reinterpret_cast<const f32x4*>(ws)[i] * old_weight : f32x4{0.f, 0.f, 0.f, 0.f};
         for (int c = 0; c < n_part; ++c) v += reinterpret_cast<const f32x4*>(part)[(bh * n_part + c) * ws_floats4 + off];
         reinterpret_cast<f32x4*>(ws)[i] = v;
     }
@@ -522,7 +523,7 @@ int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st)
             const long ws4 = G::WS_FLOATS / 4, total4 = static_cast<long>(BH) * ws4;   // D is a multiple of 8: whole 16-byte pieces
             const int blocks = static_cast<int>(std::min<long>((total4 + 255) / 256, 2048));
             hipLaunchKernelGGL(linattn_reduce_kernel, dim3(blocks), dim3(256), 0, st, p.ws, p.part, ps.n_part, ws4, total4,
-                               accumulate ? 1 : 0);
+                               accumulate ? 1 : 0, p.old_weight);
         }
     }
     // Apply pass: chunks are multiples of the tile; two resident work groups per CU hide each other's latencies, beyond
@@ -603,6 +604,7 @@ int linear_attn_forward(const mi_linear_attn_args* a, const char* op, void* part
     p.eps = a->eps;
     p.ws = static_cast<float*>(a->workspace);
     p.part = max_split > 0 ? static_cast<float*>(part) : nullptr; p.n_part = 0; p.add_to_state = 0;
+    p.old_weight = a->accumulate_weight != 0.f ? a->accumulate_weight : 1.f;
     p.tokens_per_group = 0;
     hipStream_t st = resolve_stream(a->stream);
     const int n_cu = device_cu_count();

@@ -665,5 +665,61 @@ void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, c
     run_sdpa(op, a);
 }
 
+void rms_norm_rows(const Tensor& X, const Tensor& gain, float eps, Tensor& out) {
+    const char* op = "rms_norm_rows";
+    need_gpu(op, X); need_gpu(op, gain);
+    if (gain.dtype != X.dtype || gain.size() != static_cast<std::size_t>(X.cols)) fail(std::string(op) + ": gain must hold one value of X's dtype per column");
+    if (out.data == nullptr || out.rows != X.rows || out.cols != X.cols || out.dtype != X.dtype) out.resize(X.rows, X.cols, X.dtype, X.device);
+    check(op, mi_rms_norm_forward(X.data, gain.data, out.data, X.rows, X.cols, 0, 0, eps, dtype_code(op, X.dtype), nullptr));
+}
+
+void sana_self_attention(const Tensor& x_mod, const SanaAttnWeights& w, int num_heads, Tensor& out, SanaAttnScratch& sc,
+                         RefMode ref_mode, Tensor* ref_state, float ref_weight, float rms_eps, float attn_eps) {
+    const char* op = "sana_self_attention";
+    need_gpu(op, x_mod);
+    const int N = x_mod.rows, D = x_mod.cols;
+    if (!w.Wq || !w.Wk || !w.Wv || !w.Wo) fail(std::string(op) + ": Wq, Wk, Wv and Wo are required");
+    if (num_heads <= 0 || D % num_heads != 0) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if ((w.nq == nullptr) != (w.nk == nullptr)) fail(std::string(op) + ": the qk_norm gains come as a pair");
+    const int hd = D / num_heads, per_head = hd * hd + hd;
+    if (ref_mode != RefMode::Off && ref_state == nullptr) fail(std::string(op) + ": capture / inject needs ref_state");
+    if (ref_mode == RefMode::Inject &&
+        (ref_state->data == nullptr || ref_state->rows != num_heads || ref_state->cols != per_head || ref_state->dtype != Dtype::FP32))
+        fail(std::string(op) + ": inject needs a (heads, (head_dim + 1) * head_dim) FP32 ref_state");
+    bt::linear_batched(*w.Wq, nullptr, x_mod, sc.q);
+    bt::linear_batched(*w.Wk, nullptr, x_mod, sc.k);
+    bt::linear_batched(*w.Wv, nullptr, x_mod, sc.v);
+    if (w.nq) {
+        rms_norm_rows(sc.q, *w.nq, rms_eps, sc.q);
+        rms_norm_rows(sc.k, *w.nk, rms_eps, sc.k);
+    }
+    // the state this call computes lands in the caller's ref_state when capturing, else in the scratch
+    Tensor& state = ref_mode == RefMode::Capture ? *ref_state : sc.state;
+    if (state.data == nullptr || state.rows != num_heads || state.cols != per_head || state.dtype != Dtype::FP32)
+        state.resize(num_heads, per_head, Dtype::FP32, x_mod.device);
+    if (ref_mode == RefMode::Inject) {
+        // the anchor stays as it is: a copy of it takes this call's (S, z) on top, weighted
+        if (mi_memcpy_d2d_async(state.data, ref_state->data, state.bytes(), nullptr) != 0) fail(std::string(op) + ": " + mi_last_error());
+    }
+    if (sc.attn.data == nullptr || sc.attn.rows != N || sc.attn.cols != D || sc.attn.dtype != x_mod.dtype) sc.attn.resize(N, D, x_mod.dtype, x_mod.device);
+    mi_linear_attn_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, x_mod.dtype);
+    a.q = sc.q.data; a.k = sc.k.data; a.v = sc.v.data; a.o = sc.attn.data;
+    a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.n_tokens = N;
+    a.eps = attn_eps;
+    a.accumulate_state = ref_mode == RefMode::Inject ? 1 : 0;
+    a.accumulate_weight = ref_weight;
+    if (ref_mode == RefMode::Inject && ref_weight == 0.f) a.accumulate_state = 0;    // weight 0: the anchor does not take part
+    a.workspace = state.data; a.workspace_bytes = state.bytes();
+    const std::size_t need = mi_linear_attn_scratch_bytes(1, num_heads, hd);
+    if (sc.partials.data == nullptr || sc.partials.bytes() < need || sc.partials.dtype != Dtype::FP32)
+        sc.partials.resize(1, static_cast<int>(need / 4), Dtype::FP32, x_mod.device);
+    a.scratch = sc.partials.data; a.scratch_bytes = sc.partials.bytes();
+    check(op, mi_linear_attn_relu_forward(&a));
+    bt::linear_batched(*w.Wo, w.bo, sc.attn, out);
+}
+
 }  // namespace dit
 }  // namespace bdamd

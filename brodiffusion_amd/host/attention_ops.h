@@ -179,5 +179,28 @@ void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, c
                             const Tensor* v_prefix, const std::vector<Segment>& segments, int q_offset,
                             int num_heads, const Tensor* cos_q, const Tensor* sin_q, Tensor& out);
 
+// RMS normalisation of whole rows with a per-column gain: bt::rms_norm_forward(X, gain, eps, out) (src/dit/sana.cpp:455).
+void rms_norm_rows(const Tensor& X, const Tensor& gain, float eps, Tensor& out);
+
+// SanaDenoiser::self_attention_ (src/dit/sana.cpp:411-595) as one operator: the three bias-free projections of x_mod, the
+// optional qk_norm (RMS normalisation of q and k across the full inner dimension, :449-461), the ReLU linear-attention
+// core (:470-586) and the biased output projection (:587-594). The reference runs the core channel-major, (D, N), between
+// a transposing projection and a transpose back; here everything from x_mod (N, D) to out (N, D) stays token-major, so
+// neither transpose exists, and the core is one mi_linear_attn_relu_forward call.
+// Weights are (out_features, in_features) as loaded; nq / nk (D) may be null (no qk_norm); bo may be null.
+// Identity seam (:489-506, :543-552): Capture fills `ref_state` with this call's (S, z) — FP32, num_heads blocks of
+// (head_dim + 1, head_dim): head_dim rows of S, then z, which is the layout of the reference's FP32 cache; Inject adds
+// ref_weight * ref_state to this call's (S, z) before the queries read it and leaves ref_state untouched.
+struct SanaAttnWeights {
+    const Tensor* Wq; const Tensor* Wk; const Tensor* Wv;   // (D, D)
+    const Tensor* nq; const Tensor* nk;                     // (D) gains of the qk_norm, or null
+    const Tensor* Wo; const Tensor* bo;                     // (D, D), (D) or null
+};
+struct SanaAttnScratch { Tensor q, k, v, attn, state, partials; };   // caller-owned, sized on first use, reused afterwards
+enum class RefMode { Off, Capture, Inject };
+void sana_self_attention(const Tensor& x_mod, const SanaAttnWeights& w, int num_heads, Tensor& out, SanaAttnScratch& scratch,
+                         RefMode ref_mode = RefMode::Off, Tensor* ref_state = nullptr, float ref_weight = 0.f,
+                         float rms_eps = 1e-5f, float attn_eps = 1e-15f);
+
 }  // namespace dit
 }  // namespace bdamd

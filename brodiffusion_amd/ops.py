@@ -899,6 +899,71 @@ def linear_attention_relu_forward_static_scratch(Q, K, V, num_heads: int, out: t
     return out
 
 
+def rms_norm_rows(X, gain, eps: float, out: Optional[torch.Tensor] = None):
+    """RMS normalisation of whole rows with a per-column gain: bt::rms_norm_forward(X, gain, eps, out) as Sana-Sprint's
+    qk_norm uses it (src/dit/sana.cpp:449-461). X (rows, cols), gain (cols) of X's dtype; in place is allowed."""
+    op = "rms_norm_rows"
+    _dev(op, X, gain, out)
+    dt = _dtype_code(op, X)
+    if X.dim() != 2 or X.stride(1) != 1:
+        _fail(op, "X must be (rows, cols), contiguous along columns")
+    if gain.dtype != X.dtype or gain.numel() != X.shape[1] or not gain.is_contiguous():
+        _fail(op, "gain must hold one value of X's dtype per column")
+    if out is None:
+        out = torch.empty_like(X)
+    if out.shape != X.shape or out.dtype != X.dtype or out.stride(1) != 1:
+        _fail(op, "out must have X's shape and dtype")
+    capi.check(capi.lib().mi_rms_norm_forward(X.data_ptr(), gain.data_ptr(), out.data_ptr(), X.shape[0], X.shape[1], X.stride(0),
+                                              out.stride(0), eps, dt, _stream()), op)
+    return out
+
+
+def sana_self_attention(x_mod, Wq, Wk, Wv, Wo, bo, num_heads: int, *, nq=None, nk=None, rms_eps: float = 1e-5,
+                        attn_eps: float = 1e-15, ref_mode: str = "off", ref_state: Optional[torch.Tensor] = None,
+                        ref_weight: float = 0.0, out: Optional[torch.Tensor] = None):
+    """SanaDenoiser::self_attention_ (src/dit/sana.cpp:411-595) as one operator on token-major tensors: the bias-free q, k, v
+    projections of x_mod (N, D), the optional qk_norm (nq, nk: per-column gains), the ReLU linear-attention core and the
+    output projection (Wo, bo). The reference's channel-major (D, N) layout of the core and the two transposes around it do
+    not exist here. ref_mode "capture" writes this call's (S, z) into ref_state (float32, heads x (head_dim + 1) x head_dim:
+    S rows then z, the reference's FP32 cache layout, :489-497); "inject" adds ref_weight * ref_state to this call's state
+    before the queries read it (:498-505) and leaves ref_state untouched."""
+    op = "sana_self_attention"
+    _dev(op, x_mod, Wq, Wk, Wv, Wo, bo, nq, nk, ref_state, out)
+    if x_mod.dim() != 2:
+        _fail(op, "x_mod must be (N, D)")
+    N, D = x_mod.shape
+    if num_heads <= 0 or D % num_heads != 0:
+        _fail(op, "D must equal head_dim * num_heads")
+    if (nq is None) != (nk is None):
+        _fail(op, "the qk_norm gains come as a pair")
+    if ref_mode not in ("off", "capture", "inject"):
+        _fail(op, "ref_mode must be 'off', 'capture' or 'inject'")
+    hd = D // num_heads
+    n_state = num_heads * (hd * hd + hd)
+    if ref_mode != "off":
+        if ref_state is None or ref_state.dtype != torch.float32 or ref_state.numel() != n_state or not ref_state.is_contiguous():
+            _fail(op, f"{ref_mode} needs a contiguous float32 ref_state of {n_state} values")
+    q = linear_batched(Wq, None, x_mod)
+    k = linear_batched(Wk, None, x_mod)
+    v = linear_batched(Wv, None, x_mod)
+    if nq is not None:
+        rms_norm_rows(q, nq, rms_eps, out=q)
+        rms_norm_rows(k, nk, rms_eps, out=k)
+    if ref_mode == "capture":
+        attn = linear_attention_relu_forward(q, k, v, num_heads, eps=attn_eps, workspace=ref_state.view(-1))
+    elif ref_mode == "inject" and ref_weight != 0.0:
+        attn = torch.empty_like(q)
+        ws = ref_state.view(-1).clone()                   # the anchor stays as it is; the copy takes this call's state on top
+        a = _linear_attn_args(op, q, k, v, num_heads, attn, attn_eps, ws, True)
+        a.accumulate_weight = float(ref_weight)
+        sc = torch.empty(capi.lib().mi_linear_attn_scratch_bytes(1, num_heads, hd) // 4, dtype=torch.float32, device=q.device)
+        a.scratch, a.scratch_bytes = sc.data_ptr(), sc.numel() * 4
+        capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
+    else:
+        attn = linear_attention_relu_forward(q, k, v, num_heads, eps=attn_eps)
+    return linear_batched(Wo, bo, attn, out)
+
+
 def build_axial_rope_tables(txt_len: int, hp: int, wp: int, head_dim: int, axes_dims_rope: Sequence[int],
                             theta: float = 10000.0, device="cuda"):
     """cos / sin tables (txt_len + hp*wp, head_dim/2) FP32 for the joint [text ; image] sequence

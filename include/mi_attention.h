@@ -306,6 +306,9 @@ typedef struct mi_linear_attn_args {
     int64_t o_row_stride, o_batch_stride;
     float eps;
     int32_t accumulate_state;
+    float accumulate_weight; /* with accumulate_state: weight w of the state found in the workspace, new state = this call's
+                                (S, z) + w * old (the inject strength of the identity seam, src/dit/sana.cpp:498-505, :547-551);
+                                0 means 1 */
     void* workspace;
     size_t workspace_bytes;
     void* scratch;          /* device, 16-byte aligned, or NULL */
@@ -364,6 +367,12 @@ MI_API int mi_linear_geglu_forward(const mi_linear_args* args);
  * accesses when the addresses (and, for the bias form, cols and the row stride) allow. */
 MI_API int mi_add_inplace(void* y, const void* x, int64_t n_elements, int32_t dtype, void* stream);
 MI_API int mi_add_row_bias(void* y, const void* bias, int32_t rows, int32_t cols, int64_t y_row_stride, int32_t dtype, void* stream);
+/* out[r][c] = x[r][c] * rsqrt(mean over c of x[r][c]^2 + eps) * gain[c]: RMS normalisation of whole rows, FP32 in between,
+ * one rounding. bt::rms_norm_forward(X, gain, eps, out) as Sana-Sprint applies it to the projected q and k across the full
+ * inner dimension before the head split (qk_norm, src/dit/sana.cpp:449-461). cols a multiple of 8; strides in elements
+ * (0 = dense), multiples of 8; gain (cols) of `dtype`; in place (out == x) is allowed. */
+MI_API int mi_rms_norm_forward(const void* x, const void* gain, void* out, int32_t rows, int32_t cols, int64_t x_row_stride,
+                               int64_t out_row_stride, float eps, int32_t dtype, void* stream);
 
 /* ── attention with its projections ────────────────────────────────────────
  * The three operators the U-Net spatial transformer calls (src/unet_blocks.cpp:255-327,

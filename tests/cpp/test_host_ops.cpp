@@ -493,6 +493,55 @@ static void gpu_checks() {
         bt::flash_attention_forward(Q, K, V, nullptr, H, false, o_plain);
         CHECK(o_gqa.to_host_bytes() == o_plain.to_host_bytes());
     }
+    {   // SanaDenoiser::self_attention_ as one token-major operator: projections, qk_norm, linear attention, out-projection
+        const int Ns = 192, Hs = 6, ds = 32, Ds = Hs * ds;
+        auto weight = [&](uint64_t seed) {
+            std::vector<float> wv = randn_bf16(seed, static_cast<size_t>(Ds) * Ds);
+            for (float& f : wv) f /= std::sqrt(static_cast<float>(Ds));
+            orc_round_bf16(wv.data(), wv.size());
+            return wv;
+        };
+        const std::vector<float> x = randn_bf16(8101, static_cast<size_t>(Ns) * Ds);
+        const std::vector<float> wq = weight(8102), wk = weight(8103), wv = weight(8104), wo = weight(8105);
+        std::vector<float> bo = randn_bf16(8106, Ds), nq = randn_bf16(8107, Ds), nk = randn_bf16(8108, Ds);
+        for (int i = 0; i < Ds; ++i) { nq[i] = 1.f + 0.25f * nq[i]; nk[i] = 1.f + 0.25f * nk[i]; }
+        orc_round_bf16(nq.data(), nq.size()); orc_round_bf16(nk.data(), nk.size());
+        const Tensor X = upload_bf16(x, Ns, Ds), Wq = upload_bf16(wq, Ds, Ds), Wk = upload_bf16(wk, Ds, Ds), Wv = upload_bf16(wv, Ds, Ds),
+                     Wo = upload_bf16(wo, Ds, Ds), Bo = upload_bf16(bo, 1, Ds), Nq = upload_bf16(nq, 1, Ds), Nk = upload_bf16(nk, 1, Ds);
+        const dit::SanaAttnWeights w{&Wq, &Wk, &Wv, &Nq, &Nk, &Wo, &Bo};
+        dit::SanaAttnScratch sc;
+        Tensor out, state;
+        dit::sana_self_attention(X, w, Hs, out, sc, dit::RefMode::Capture, &state);
+        // checker: the same chain, every intermediate rounded to bf16 as a tensor of the compute dtype
+        auto lin = [&](const std::vector<float>& a, const std::vector<float>& wt, const float* b) {
+            std::vector<float> y(static_cast<size_t>(Ns) * Ds);
+            orc_linear(a.data(), wt.data(), b, Ns, Ds, Ds, y.data(), 0);
+            return y;
+        };
+        std::vector<float> q = lin(x, wq, nullptr), k = lin(x, wk, nullptr), v = lin(x, wv, nullptr);
+        orc_round_bf16(q.data(), q.size()); orc_round_bf16(k.data(), k.size()); orc_round_bf16(v.data(), v.size());
+        std::vector<float> qn(q.size()), kn(k.size());
+        orc_rms_norm(q.data(), nq.data(), 1e-5, Ns, Ds, qn.data()); orc_rms_norm(k.data(), nk.data(), 1e-5, Ns, Ds, kn.data());
+        orc_round_bf16(qn.data(), qn.size()); orc_round_bf16(kn.data(), kn.size());
+        std::vector<float> attn(q.size()), S(static_cast<size_t>(Hs) * ds * ds), z(static_cast<size_t>(Hs) * ds);
+        orc_linear_attn_relu(qn.data(), kn.data(), v.data(), Ns, Hs, ds, 1e-15f, attn.data(), S.data(), z.data(), 0);
+        orc_round_bf16(attn.data(), attn.size());
+        const std::vector<float> ref = lin(attn, wo, bo.data());
+        CHECK(within_bf16(compare(ref, download_bf16(out))));
+        CHECK(state.rows == Hs && state.cols == ds * ds + ds && state.dtype == Dtype::FP32);
+        // inject with weight 1 of the call's own state doubles numerator and denominator alike: same output, anchor untouched
+        const std::vector<uint8_t> anchor_before = state.to_host_bytes();
+        Tensor out2;
+        dit::sana_self_attention(X, w, Hs, out2, sc, dit::RefMode::Inject, &state, 1.0f);
+        CHECK(state.to_host_bytes() == anchor_before);
+        CHECK(within_bf16(compare(ref, download_bf16(out2))));
+        CHECK(throws_with([&] { dit::sana_self_attention(X, w, Hs, out2, sc, dit::RefMode::Inject, nullptr, 1.0f); }, "needs ref_state"));
+        Tensor n_out;
+        dit::rms_norm_rows(X, Nq, 1e-5f, n_out);
+        std::vector<float> n_ref(x.size());
+        orc_rms_norm(x.data(), nq.data(), 1e-5, Ns, Ds, n_ref.data());
+        CHECK(compare(n_ref, download_bf16(n_out)).rel_l2 <= 5e-3);
+    }
     {   // GPU-side error path: unsupported head_dim surfaces the C ABI's message
         Tensor out;
         CHECK(throws_with([&] { bt::flash_attention_forward(Q, K, V, nullptr, 8, false, out); }, "no kernel"));
