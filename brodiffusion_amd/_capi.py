@@ -58,6 +58,8 @@ class MiSdpaArgs(C.Structure):
         ("logit_bias", C.c_void_p), ("bias_q0", C.c_int32), ("bias_cols", C.c_int32), ("bias_row_stride", C.c_int64),
         ("lse_out", C.c_void_p),
         ("cu_seqlens_q", C.c_void_p), ("cu_seqlens_k", C.c_void_p),
+        ("prefix_k_scale", C.c_float), ("prefix_v_scale", C.c_float),
+        ("prefix_k_row_scale", C.c_void_p), ("prefix_v_row_scale", C.c_void_p),
         ("split_scratch", C.c_void_p), ("split_scratch_bytes", C.c_size_t),
         ("stream", C.c_void_p),
     ]

@@ -201,6 +201,17 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
         if (reinterpret_cast<uintptr_t>(a->logit_bias) & 3u) return fail("mi_sdpa_forward: logit_bias must be 4-byte aligned");
         if (a->bias_cols == 0 || a->bias_q0 >= a->q_len) p.bias = nullptr;   // nothing to add
     }
+    {
+        const float ks = a->prefix_k_scale != 0.f ? a->prefix_k_scale : 1.f, vs = a->prefix_v_scale != 0.f ? a->prefix_v_scale : 1.f;
+        if (!std::isfinite(ks) || !std::isfinite(vs)) return fail("mi_sdpa_forward: prefix_k_scale / prefix_v_scale must be finite");
+        if ((reinterpret_cast<uintptr_t>(a->prefix_k_row_scale) | reinterpret_cast<uintptr_t>(a->prefix_v_row_scale)) & 3u)
+            return fail("mi_sdpa_forward: prefix row scales must be 4-byte aligned");
+        if (a->prefix_len > 0 && (ks != 1.f || vs != 1.f || a->prefix_k_row_scale || a->prefix_v_row_scale)) {
+            p.prefix_scaled = 1;
+            p.pk_scale = ks; p.pv_scale = vs;
+            p.pk_row = a->prefix_k_row_scale; p.pv_row = a->prefix_v_row_scale;
+        }
+    }
     if ((a->cu_seqlens_q == nullptr) != (a->cu_seqlens_k == nullptr)) return fail("mi_sdpa_forward: cu_seqlens_q and cu_seqlens_k must be given together");
     if (a->cu_seqlens_q) {
         if (a->prefix_len > 0 || a->key_mask || a->kv_valid_len || a->rope_cos_q || a->rope_cos_k || a->logit_bias || a->lse_out)

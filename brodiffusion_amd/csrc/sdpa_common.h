@@ -327,6 +327,26 @@ __device__ __forceinline__ float blank_outside(float score, int x, int top, int 
     return __builtin_bit_cast(float, (bits & ~out) | (0xff800000u & out));
 }
 
+// Factors carried by the rows of the cached prefix (the dial's scalar times the optional per-row weight), handed to the
+// softmax of a prefix tile by value; on == false: the tile has none. Rows of a partly filled last prefix tile that lie
+// past the prefix read its last entry; their scores are blanked anyway.
+struct PrefixScale {
+    bool on = false;
+    const float* k_row = nullptr; const float* v_row = nullptr;
+    float ks = 1.f, vs = 1.f;
+    int Lp = 0;
+    __device__ __forceinline__ float k(int key) const { return k_row ? ks * k_row[min(key, Lp - 1)] : ks; }
+    __device__ __forceinline__ float v(int key) const { return v_row ? vs * v_row[min(key, Lp - 1)] : vs; }
+};
+__device__ __forceinline__ PrefixScale prefix_scale_of(const SdpaDev& p, bool tile_in_prefix) {
+    PrefixScale s;
+    s.on = p.prefix_scaled && tile_in_prefix;
+    s.k_row = p.pk_row; s.v_row = p.pv_row; s.ks = p.pk_scale; s.vs = p.pv_scale; s.Lp = p.Lp;
+    return s;
+}
+// key index of accumulator element e of key block kb for this lane half
+__device__ __forceinline__ int key_of(int j0, int kb, int e, int lh) { return j0 + 32 * kb + 8 * (e >> 2) + 4 * lh + (e & 3); }
+
 // Online-softmax state of one lane (one query row, shared with lane l^32).
 // m is the reference the exponentials are taken against; it is raised only when a tile's maximum
 // exceeds it by more than 2^kLazyLog2, so most tiles skip the rescale of l and O. The result does
@@ -341,11 +361,18 @@ struct SoftmaxState {
 // of the PV product. The mask step only touches the scores, so the two cases share every other
 // instruction and the accumulators are updated at one place only (separate masked / unmasked copies of
 // this function cost the register allocator ~70 registers in copies of O).
-template <typename T, int D>
+template <typename T, int D, bool PSCALE = false>
 __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
                                              SoftmaxState& st, float cl2, float lazy_raw, bool masked, int j0, int lo, int hi,
                                              int lh, const float* mask_tile, const float* bias_row = nullptr, int bias_cols = 0,
-                                             float bias_k = 0.f) {
+                                             float bias_k = 0.f, PrefixScale prefix = PrefixScale()) {
+    // tile of the cached prefix whose rows carry factors (PSCALE instances only): K's factor multiplies the raw scores
+    if (PSCALE && prefix.on) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[kb][e] *= prefix.k(key_of(j0, kb, e, lh));
+    }
     if (masked) {
         // additive logit bias of this lane's query row (null: none) for keys below bias_cols, in raw-score units
         if (bias_row) {
@@ -411,6 +438,13 @@ __device__ __forceinline__ void softmax_tile(f32x16 (&sacc)[2], typename Mma<T>:
         lsum1 += p1;
     }
     st.l += lsum0 + lsum1;
+    // ... and V's factor multiplies the probabilities, after the row sum has been taken
+    if (PSCALE && prefix.on) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[kb][e] *= prefix.v(key_of(j0, kb, e, lh));
+    }
     // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4)
@@ -445,9 +479,20 @@ struct RelSoftmaxState {
 };
 constexpr float kRelSumMax = 1024.f;
 
-template <typename T, int D>
+template <typename T, int D, bool PSCALE = false>
 __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
-                                                 RelSoftmaxState& st, bool masked, bool dead_row, int j0, int lo, int hi, int lh) {
+                                                 RelSoftmaxState& st, bool masked, bool dead_row, int j0, int lo, int hi, int lh,
+                                                 PrefixScale prefix = PrefixScale()) {
+    // Tile of the cached prefix whose rows carry factors (wave-uniform flag; PSCALE instances only, so that the other
+    // instances keep their register budget). The scores arrive as exponents x = s * cl2 - ref; K's factor f belongs on s:
+    // x' = f * (x + ref) - ref.
+    if (PSCALE && prefix.on) {
+        const float nr = st.neg_ref;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) sacc[kb][e] = __builtin_fmaf(prefix.k(key_of(j0, kb, e, lh)), sacc[kb][e] - nr, nr);
+    }
     if (masked) {
         const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;   // keys outside [lo, hi) become -inf
 #pragma unroll
@@ -465,6 +510,19 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
     constexpr bool PAIR_SUM = HeadGeo<D>::VB < 4;
     auto exponentiate = [&]() -> float {
         float s0 = 0.f, s1 = 0.f;
+        if (PSCALE && prefix.on) {
+            // V's factor multiplies the probabilities that go into the PV product; the row sum takes them as they are
+#pragma unroll
+            for (int c4 = 0; c4 < 4; ++c4)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int kb = c4 >> 1, e = 8 * (c4 & 1) + t;
+                    const float pr = __builtin_amdgcn_exp2f(sacc[kb][e]);
+                    pf[c4][t] = static_cast<T>(pr * prefix.v(key_of(j0, kb, e, lh)));
+                    if (t & 1) s1 += pr; else s0 += pr;
+                }
+            return s0 + s1;
+        }
         // P^T as B operand: 16-key chunk c4 is acc[8*(c4%2) .. +7] of block c4/2
 #pragma unroll
         for (int c4 = 0; c4 < 4; ++c4) {

@@ -299,7 +299,9 @@ template <int D> constexpr int lds_bytes_4() {
 // VARLEN: the batch items are sequences of different lengths packed back to back along the row axis
 // (cu_q / cu_k: device arrays of batch + 1 row offsets, the cu_seqlens convention); Lq and Lk of the launch are the
 // longest sequence and only size the grid. Each work group rebuilds the launch view for its own sequence.
-template <typename T, int D, bool ROPE_K, bool VARLEN = false>
+// PSCALE: the rows of the cached prefix carry factors (the prefix-KV dial); a separate instance so that the code for it
+// costs the other instances no registers.
+template <typename T, int D, bool ROPE_K, bool VARLEN = false, bool PSCALE = false>
 __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(const SdpaDev p_in) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
@@ -405,8 +407,9 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
             mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
             const bool biased = p.bias != nullptr && j0 < p.bias_cols;
             const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim)) && (key_mask == nullptr) && !biased;
-            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, Ms,
-                               biased ? bias_row : nullptr, p.bias_cols, p.inv_scale);
+            softmax_tile<T, D, PSCALE>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, lim), lh, Ms,
+                                       biased ? bias_row : nullptr, p.bias_cols, p.inv_scale,
+                                       PSCALE ? prefix_scale_of(p, plan.in_prefix(t)) : PrefixScale());
             mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
         }
         if (t + 1 < n_tiles) {
@@ -816,9 +819,11 @@ __device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2)
 // every row, so the masked form of the softmax and the per-step bookkeeping (which tile, its limit, whether this
 // wavefront sees it whole) drop out of the kernel, and with them their registers: measured 6 % faster at head_dim 128
 // and 8 % at 72 than the general form on the same dense call.
-template <typename T, int D, bool SPLIT, bool DENSE = false>
+// PSCALE: the general form with the prefix-KV dial (factors on the rows of the cached prefix) in its softmax.
+template <typename T, int D, bool SPLIT, bool DENSE = false, bool PSCALE = false>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const SdpaDev p) {
     static_assert(!(SPLIT && DENSE), "the split launch clips key ranges per part");
+    static_assert(!PSCALE || (!SPLIT && !DENSE), "the dial belongs to the general form");
     using G = HeadGeo<D>;
     using DG = DmaGeo<D>;
     using V8 = typename Mma<T>::v8;
@@ -1049,7 +1054,8 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
                 const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                softmax_tile_rel<T, D, PSCALE>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh,
+                                               PSCALE ? prefix_scale_of(p, plan.in_prefix(tt)) : PrefixScale());
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -1312,7 +1318,9 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     const int choice = sdpa_kernel_choice();
     // calls with a key mask stay on the 128-row kernel, which stages the mask tile in LDS
     // ... and so do calls with a logit bias or a request for the softmax denominators
-    const bool pingpong = D <= 128 && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr &&
+    // ... and so do calls with the prefix-KV dial, unless the DMA kernel (which has an instance for it) takes them
+    const bool dial_ok = !p.prefix_scaled || (dma_kernel_available<D>() && !rope_k && choice != 3);
+    const bool pingpong = D <= 128 && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr && dial_ok &&
                           (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
     // short key sequences whose K and V fit in LDS next to a query tile: one work group walks several query tiles
     const int n_kt = (p.Lk + kBN - 1) / kBN;
@@ -1340,9 +1348,10 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
             else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
                 if constexpr (dma_kernel_available<D>()) {
                     // whole key tiles only; a cached prefix may come first if it is whole tiles too and laid out like K / V
-                    const bool dense = p.mask_mode == MI_MASK_NONE && p.kv_valid_len == nullptr && p.Lk % kBN == 0 &&
+                    const bool dense = p.mask_mode == MI_MASK_NONE && p.kv_valid_len == nullptr && p.Lk % kBN == 0 && !p.prefix_scaled &&
                                        (p.Lp == 0 || (p.Lp % kBN == 0 && p.kp_rs == p.k_rs && p.vp_rs == p.v_rs));
                     if (dense) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false, true>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
+                    else if (p.prefix_scaled) hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false, false, true>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                     else hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false>), grid, block, DmaGeo<D>::lds_bytes(), stream, p);
                 }
             }
@@ -1355,7 +1364,11 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
         p.n_q_tiles = (p.Lq + 127) / 128;
         p.n_blocks = p.B * p.H * p.n_q_tiles;
         const dim3 grid(grid_blocks(p)), block(kThreads4);
-        if (rope_k) hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, true>), grid, block, lds_bytes_4<D>(), stream, p);
+        if (p.prefix_scaled) {
+            if (rope_k) return fail("mi_sdpa_forward: the prefix-KV dial with K rotated tile by tile is not supported (lend rope_k_scratch)");
+            hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false, false, true>), grid, block, lds_bytes_4<D>(), stream, p);
+        }
+        else if (rope_k) hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, true>), grid, block, lds_bytes_4<D>(), stream, p);
         else hipLaunchKernelGGL((sdpa_fwd_kernel<T, D, false>), grid, block, lds_bytes_4<D>(), stream, p);
     }
     const hipError_t e = hipGetLastError();

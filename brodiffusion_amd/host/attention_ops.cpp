@@ -633,7 +633,7 @@ void scale_rows(const Tensor& X, float scale, const Tensor* row_scale, Tensor& o
 
 void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix, const Tensor* v_prefix,
                             const std::vector<Segment>& segments, int q_offset, int num_heads, const Tensor* cos_q,
-                            const Tensor* sin_q, Tensor& out) {
+                            const Tensor* sin_q, Tensor& out, const PrefixDial* dial) {
     const char* op = "block_causal_attention";
     if (segments.empty() || segments.size() > static_cast<std::size_t>(MI_MAX_SEGMENTS))
         fail(std::string(op) + ": between 1 and 32 segments");
@@ -646,6 +646,17 @@ void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, c
             k_prefix->dtype != Q.dtype || v_prefix->dtype != Q.dtype)
             fail(std::string(op) + ": prefix K/V must be (prefix_len, D) in Q's dtype");
         a.k_prefix = k_prefix->data; a.v_prefix = v_prefix->data; a.prefix_len = k_prefix->rows;
+    }
+    if (dial && a.prefix_len > 0) {
+        a.prefix_k_scale = dial->k_scale; a.prefix_v_scale = dial->v_scale;
+        for (const Tensor* rows : {dial->k_rows, dial->v_rows}) {
+            if (!rows) continue;
+            need_gpu(op, *rows);
+            if (rows->dtype != Dtype::FP32 || rows->size() != static_cast<std::size_t>(a.prefix_len))
+                fail(std::string(op) + ": the dial's row weights must hold prefix_len FP32 values");
+        }
+        a.prefix_k_row_scale = dial->k_rows ? static_cast<const float*>(dial->k_rows->data) : nullptr;
+        a.prefix_v_row_scale = dial->v_rows ? static_cast<const float*>(dial->v_rows->data) : nullptr;
     }
     a.mask_mode = MI_MASK_BLOCK_CAUSAL;
     a.q_offset = q_offset;

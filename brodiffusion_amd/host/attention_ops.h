@@ -175,9 +175,17 @@ struct Segment {
 // `segments` describe the query rows in order: a Text run is causal, an Image block sees every key
 // up to its own end. Equals the reference's one-call-per-segment decomposition; with a single Image
 // segment covering all keys it is the cached form (qwenimage21_forward.cpp:599-649).
+// `dial` (optional): the prefix-KV dial of the cached step (set_prefix_kv_scale, qwenimage21_forward.cpp:606-645) applied
+// inside the kernel — a factor per side on the rows of the cached prefix, optionally times a per-row FP32 weight
+// ((prefix_len, 1) or (1, prefix_len)); the cache tensors are never written and no scaled copy is made.
+struct PrefixDial {
+    float k_scale = 1.f, v_scale = 1.f;
+    const Tensor* k_rows = nullptr; const Tensor* v_rows = nullptr;
+};
 void block_causal_attention(const Tensor& Q, const Tensor& K, const Tensor& V, const Tensor* k_prefix,
                             const Tensor* v_prefix, const std::vector<Segment>& segments, int q_offset,
-                            int num_heads, const Tensor* cos_q, const Tensor* sin_q, Tensor& out);
+                            int num_heads, const Tensor* cos_q, const Tensor* sin_q, Tensor& out,
+                            const PrefixDial* dial = nullptr);
 
 // RMS normalisation of whole rows with a per-column gain: bt::rms_norm_forward(X, gain, eps, out) (src/dit/sana.cpp:455).
 void rms_norm_rows(const Tensor& X, const Tensor& gain, float eps, Tensor& out);

@@ -115,7 +115,8 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
                  rope_k: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  rope_k_scratch: Optional[torch.Tensor] = None, rope_split_half: bool = False, split_scratch=None,
                  logit_bias: Optional[torch.Tensor] = None, bias_q0: int = 0, lse_out: Optional[torch.Tensor] = None,
-                 op: str = "sdpa_forward") -> torch.Tensor:
+                 prefix_k_scale: float = 1.0, prefix_v_scale: float = 1.0, prefix_k_row_scale: Optional[torch.Tensor] = None,
+                 prefix_v_row_scale: Optional[torch.Tensor] = None, op: str = "sdpa_forward") -> torch.Tensor:
     """General entry: everything mi_sdpa_forward offers. Returns `out` (allocated like q if None).
     split_scratch: None = lend the module's own scratch (grown on demand, one per device, shared by all calls of the
     process: use one stream at a time) when the launch can use one, False = never split, a uint8 tensor = lend that."""
@@ -162,6 +163,14 @@ def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: i
         a.k_prefix, a.v_prefix, a.prefix_len = k_prefix.data_ptr(), v_prefix.data_ptr(), Lp
         a.kp_row_stride, a.kp_batch_stride, a.vp_row_stride, a.vp_batch_stride = kp_rs, kp_bs, vp_rs, vp_bs
     a.scale = float(scale) if scale is not None else 0.0
+    a.prefix_k_scale, a.prefix_v_scale = float(prefix_k_scale), float(prefix_v_scale)
+    for nm, rs in (("prefix_k_row_scale", prefix_k_row_scale), ("prefix_v_row_scale", prefix_v_row_scale)):
+        if rs is None:
+            continue
+        _dev(op, rs)
+        if rs.dtype != torch.float32 or rs.numel() != Lp or not rs.is_contiguous():
+            _fail(op, f"{nm} must be a contiguous float32 tensor of prefix_len ({Lp}) values")
+        setattr(a, nm, rs.data_ptr())
     if mask is not None:
         a.mask_mode, a.q_offset, a.window = mask.mode, mask.q_offset, mask.window
         if mask.mode == capi.MI_MASK_BLOCK_CAUSAL:

@@ -165,6 +165,17 @@ typedef struct mi_sdpa_args {
                                     (q, k, v, cu_q, cu_k, n_seqs, max_q, max_k, num_heads, head_dim, causal, out),
                                     src/dit/krea2.cpp:574. MI_MASK_NONE or MI_MASK_CAUSAL (window 0; each sequence aligns its last
                                     query with its last key); no prefix, key mask, kv_valid_len, RoPE, bias */
+    /* The prefix-KV dial of the Qwen-Image cached step (set_prefix_kv_scale, src/dit/qwenimage21_forward.cpp:606-645): the
+       rows of k_prefix count as multiplied by prefix_k_scale, those of v_prefix by prefix_v_scale (0 = 1), and, if the
+       arrays are given, row j additionally by prefix_k_row_scale[j] / prefix_v_row_scale[j] (device FP32 [prefix_len],
+       shared by the batch). Nothing is copied or written: the K factor multiplies the FP32 scores of the prefix keys,
+       the V factor their probabilities after the row sum is taken, inside the attention kernel (the reference scales a
+       copy of the cached rows and rounds it to the storage type; mi_scale_rows + k_prefix is that dataflow). With
+       scalars of exactly 1 and no arrays the call is the unscaled one bit for bit. */
+    float prefix_k_scale;
+    float prefix_v_scale;
+    const float* prefix_k_row_scale;
+    const float* prefix_v_row_scale;
     void* split_scratch;         /* device, 16-byte aligned, or NULL: lets a launch whose last round of work groups would fill
                                     only part of the GPU cut the query tiles of that round along the key axis into equal
                                     pieces for all compute units (partial results in the scratch, merged by a second small

@@ -233,6 +233,20 @@ static void gpu_checks() {
         std::printf("prefix-KV dial        rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
         CHECK(throws_with([&] { Tensor o2; dit::scale_rows(kp, 1.0f, &Wk, o2); dit::scale_rows(K, 1.0f, &Wk, o2); }, "the row scale holds 21 values"));
+        // the same dial applied inside the kernel (no scaled copy): within tolerance of the checker, the cache untouched, set
+        // twice the same bits, identity = the plain step, and close to the scaled-copy route it replaces
+        dit::PrefixDial dial;
+        dial.k_scale = 0.8f; dial.v_scale = 1.0f; dial.k_rows = &Wk; dial.v_rows = &Wv;
+        Tensor o_in, o_in2, o_id;
+        dit::block_causal_attention(Qt, Kt, Vt, &kp, &vp, seg, prefix, H, nullptr, nullptr, o_in, &dial);
+        dit::block_causal_attention(Qt, Kt, Vt, &kp, &vp, seg, prefix, H, nullptr, nullptr, o_in2, &dial);
+        CHECK(o_in.to_host_bytes() == o_in2.to_host_bytes());
+        CHECK(kp.to_host_bytes() == cache_before);
+        CHECK(within_bf16(compare(ref, download_bf16(o_in))));
+        CHECK(within_bf16(compare(download_bf16(o_w), download_bf16(o_in))));
+        const dit::PrefixDial identity;
+        dit::block_causal_attention(Qt, Kt, Vt, &kp, &vp, seg, prefix, H, nullptr, nullptr, o_id, &identity);
+        CHECK(o_id.to_host_bytes() == plain);
     }
     {   // ReLU linear attention, 70 x 32 (the reference's own head split) on a short sequence
         const int Hl = 70, dl = 32, N = 96, Dl = Hl * dl;
