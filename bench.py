@@ -3,14 +3,17 @@
 
 A step is one call of the hot path on the headline workload: Flux.1 double-stream joint attention,
 B=1, H=24, head_dim=128, 512 text + 4096 image tokens, bf16, RoPE (axes 16/56/56, theta 1e4) applied
-to Q and K inside the attention launch. Inputs are synthetic N(0,1), resident in HBM before the
-timed region. Prints ONE JSON line.
+to Q and K inside the attention launch. Inputs are synthetic N(0,1) from the seeded generator the reference's
+harnesses use (torch_randn_f32 of include/brodiffusion/detail/torch_rng.h = torch's CPU generator; configuration c
+takes seeds 1000 c + 1, + 2, + 3 for Q, K, V), rounded once to the GPU dtype and resident in HBM before the timed
+region. Prints ONE JSON line.
 
   metric      attention TFLOP/s, algorithmic FLOPs = 4 * B * H * Lq * Lk * d (QK^T and PV, nothing else)
   roofline    the flash kernel against MI355X dense bf16 MFMA peak (2.5 PFLOP/s), kernel time from HIP
               events on the launch stream over the timed region
   cpu_baseline the CPU checker (a port of the reference's FP32/FP64 host attention loop) timed on this
-              host's cores on a bounded sample of the same workload
+              host's cores on a bounded sample of the same workload (all threads, and one thread), the GPU
+              result of the timed step compared with it on the sampled rows, and the same for every configuration
   configs     ms per call and TFLOP/s (GB/s for linear attention) of every benchmark configuration, measured
               outside the timed region
 """
@@ -25,9 +28,11 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16 / fp16 MFMA, published
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E, published
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --traffic-probe`: (69300 KiB x 2.00 calibration) fetched + 27648 KiB written.
+# HBM bytes per launch of the headline kernel. Not measured in this run: a constant taken from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs of `bench.py --traffic-probe` (counter values and calibration in the file named below):
+# (FETCH_SIZE KiB x 2.00 calibration) fetched + WRITE_SIZE KiB written.
 TRAFFIC_BYTES_PER_LAUNCH = (69300 * 2 + 27648) * 1024
+TRAFFIC_SOURCE = "profiles/sdpa_fwd_pp_dma_bf16_flux_joint_4608_hbm_traffic.txt"
 
 
 def parse():
@@ -68,7 +73,32 @@ def event_ms(torch, fn, iters, warm=0.05):
     return min(ts), sum(ts) / len(ts)
 
 
-def all_configs(torch, bd):
+def seeded(torch, seed, shape, dtype):
+    """N(0,1) values of torch's CPU generator for `seed` (what torch_randn_f32(seed, n) of the reference's torch_rng.h
+    reproduces), rounded once to `dtype`, on the GPU."""
+    n = 1
+    for e in shape:
+        n *= e
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, generator=g, dtype=torch.float32).reshape(shape).to(dtype).cuda()
+
+
+def config_inputs(torch):
+    """Q, K, V (and what else a call takes) of the benchmark configurations other than the headline one."""
+    f16, b16 = torch.float16, torch.bfloat16
+    c = {}
+    c["cfg1"] = tuple(seeded(torch, 1000 + i, (2, 4096, 320), f16) for i in (1, 2, 3))
+    c["cfg2a"] = tuple(seeded(torch, 2000 + i, (2, 4096, 1152), b16) for i in (1, 2, 3))
+    gen = torch.Generator().manual_seed(2099)
+    valid = [int(20 + torch.randint(0, 281, (1,), generator=gen).item()) for _ in range(2)]
+    c["cfg2b"] = (c["cfg2a"][0], seeded(torch, 2012, (2, 300, 1152), b16), seeded(torch, 2013, (2, 300, 1152), b16), valid)
+    c["cfg4"] = (seeded(torch, 4001, (4096, 3072), b16), seeded(torch, 4002, (4608, 3072), b16), seeded(torch, 4003, (4608, 3072), b16))
+    c["cfg5a"] = tuple(seeded(torch, 5000 + i, (2, 1024, 2240), b16) for i in (1, 2, 3))
+    c["cfg5b"] = tuple(seeded(torch, 5010 + i, (2, 4096, 2240), b16) for i in (1, 2, 3))
+    return c
+
+
+def all_configs(torch, bd, cin, keep):
     """Every benchmark configuration: ms per call (min and mean over 20 calls), TFLOP/s or GB/s, fraction of peak."""
     g = torch.Generator(device="cuda").manual_seed(1234)
 
@@ -83,8 +113,10 @@ def all_configs(torch, bd):
                      "frac_mfma_peak": round(flops / (mn * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, 4), "dtype": dtype,
                      "gflop": round(flops / 1e9, 2)}
 
-    q, k, v = (rnd(2, 4096, 320, dt=torch.float16) for _ in range(3))
-    sdpa_entry("cfg1_sd15_selfattn_d40_fp16", 4 * 2 * 8 * 4096 * 4096 * 40, lambda: bd.flash_attention_forward(q, k, v, None, 8, False), "fp16")
+    q, k, v = cin["cfg1"]
+    o1 = torch.empty_like(q)
+    sdpa_entry("cfg1_sd15_selfattn_d40_fp16", 4 * 2 * 8 * 4096 * 4096 * 40, lambda: bd.flash_attention_forward(q, k, v, None, 8, False, out=o1), "fp16")
+    keep["cfg1"] = o1
     # the same attention inside the U-Net block: Q/K/V projections (one launch), attention, output projection
     x, ctx = rnd(2, 4096, 320, dt=torch.float16), rnd(2, 77, 768, dt=torch.float16)
     wq, wk, wv, wo = (rnd(320, 320, dt=torch.float16) / 320 ** 0.5 for _ in range(4))
@@ -108,27 +140,31 @@ def all_configs(torch, bd):
     wg_, bg_ = rnd(2560, 320, dt=torch.float16) / 320 ** 0.5, rnd(2560, dt=torch.float16)
     yg_ = torch.empty(8192, 1280, dtype=torch.float16, device="cuda")
     sdpa_entry("sd15_unet_block_ff1_geglu_8192x320x2560_fp16", 2 * 8192 * 2560 * 320, lambda: bd.fused_linear_geglu(x2, wg_, bg_, yg_), "fp16")
-    q, k, v = (rnd(2, 4096, 1152) for _ in range(3))
-    sdpa_entry("cfg2a_pixart_selfattn_d72_bf16", 4 * 2 * 16 * 4096 * 4096 * 72, lambda: bd.flash_attention_forward(q, k, v, None, 16, False), "bf16")
-    kc, vc = rnd(2, 300, 1152), rnd(2, 300, 1152)
-    gen = torch.Generator().manual_seed(2099)
-    valid = [int(20 + torch.randint(0, 281, (1,), generator=gen).item()) for _ in range(2)]
+    q, k, v = cin["cfg2a"]
+    o2a = torch.empty_like(q)
+    sdpa_entry("cfg2a_pixart_selfattn_d72_bf16", 4 * 2 * 16 * 4096 * 4096 * 72, lambda: bd.flash_attention_forward(q, k, v, None, 16, False, out=o2a), "bf16")
+    keep["cfg2a"] = o2a
+    _, kc, vc, valid = cin["cfg2b"]
     vl = torch.tensor(valid, dtype=torch.int32, device="cuda")
-    sdpa_entry("cfg2b_pixart_crossattn_d72_bf16", 4 * 16 * 4096 * sum(valid) * 72, lambda: bd.sdpa_forward(q, kc, vc, 16, kv_valid_len=vl), "bf16")
+    o2b = torch.empty_like(q)
+    sdpa_entry("cfg2b_pixart_crossattn_d72_bf16", 4 * 16 * 4096 * sum(valid) * 72, lambda: bd.sdpa_forward(q, kc, vc, 16, kv_valid_len=vl, out=o2b), "bf16")
     out["cfg2b_pixart_crossattn_d72_bf16"]["valid_len"] = valid
+    keep["cfg2b"] = o2b
     q, k, v = (rnd(4608, 3072) for _ in range(3))
     cos, sin = bd.build_axial_rope_tables(512, 64, 64, 128, (16, 56, 56))
     kr3 = torch.empty_like(k)
     sdpa_entry("cfg3_flux_joint_d128_bf16_rope", 4 * 24 * 4608 * 4608 * 128, lambda: bd.joint_attention(q, k, v, cos, sin, 128, 24, Kr=kr3), "bf16")
     out["cfg3_flux_joint_d128_bf16_rope_fused_k"] = None
     sdpa_entry("cfg3_flux_joint_d128_bf16_rope_fused_k", 4 * 24 * 4608 * 4608 * 128, lambda: bd.joint_attention(q, k, v, cos, sin, 128, 24), "bf16")
-    qb, kb, vb = (rnd(4096, 3072) for _ in range(3))
-    kp, vp = rnd(512, 3072), rnd(512, 3072)
+    qb, kall, vall = cin["cfg4"]                       # keys: 512 cached prefix rows (their own buffers), then 4096 fresh rows
+    kp, vp, kb, vb = kall[:512].clone(), vall[:512].clone(), kall[512:].clone(), vall[512:].clone()
     sq = [1024, 2048, 3072, 4096]
     sk = [512 + e for e in sq]
     mask = bd.SdpaMask.block_causal(512, sq, sk, [0] * 4)
+    o4 = torch.empty_like(qb)
     sdpa_entry("cfg4_qwen_blockcausal_prefixkv_d128_bf16", 4 * 24 * sum(1024 * e for e in sk) * 128,
-               lambda: bd.sdpa_forward(qb, kb, vb, 24, k_prefix=kp, v_prefix=vp, mask=mask), "bf16")
+               lambda: bd.sdpa_forward(qb, kb, vb, 24, k_prefix=kp, v_prefix=vp, mask=mask, out=o4), "bf16")
+    keep["cfg4"] = o4
     out["cfg4_qwen_blockcausal_prefixkv_d128_bf16"]["dense_equivalent_gflop"] = round(4 * 24 * 4096 * 4608 * 128 / 1e9, 2)
     xh, gh = rnd(4608, 3072), rnd(128)
     oh = torch.empty_like(xh)
@@ -146,8 +182,8 @@ def all_configs(torch, bd):
     out["hbm_copy_ceiling_147mb"] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(copy_gbs, 1),
                                      "frac_hbm_peak": round(copy_gbs / PEAK_HBM_GBS, 4)}
     del csrc, cdst
-    for name, n in (("cfg5a_sana_linear_n1024_d112_bf16", 1024), ("cfg5b_sana_linear_n4096_d112_bf16", 4096)):
-        ql, kl, vl_ = (rnd(2, n, 2240) for _ in range(3))
+    for name, n, key in (("cfg5a_sana_linear_n1024_d112_bf16", 1024, "cfg5a"), ("cfg5b_sana_linear_n4096_d112_bf16", 4096, "cfg5b")):
+        ql, kl, vl_ = cin[key]
         ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
         sc = torch.empty(8 * ws.numel(), dtype=torch.float32, device="cuda")     # partial states (mi_linear_attn_scratch_bytes)
         o = torch.empty_like(ql)
@@ -157,18 +193,31 @@ def all_configs(torch, bd):
                      "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                      "frac_copy_ceiling": round(nbytes / (mn * 1e-3) / 1e9 / copy_gbs, 4), "dtype": "bf16 in, f32 accumulate",
                      "mbytes": round(nbytes / 1e6, 2)}
+        keep[key] = o
     return out
 
 
-def cpu_baseline():
-    """The CPU checker on a bounded sample of the headline workload: RoPE on all of Q and K, then the
-    exact attention loop for a subset of query rows (all heads, all 4608 keys), sized for ~10-20 s."""
+def cpu_baseline(torch, headline, cin, keep):
+    """The CPU checker (a port of the reference's host attention loop, src/dit/common.cpp:246-305, and of Sana's FP32 core,
+    src/dit/sana.cpp:470-520) timed on this host on bounded samples of the same workloads, and the GPU results of this run
+    compared with it on the sampled rows. Headline: RoPE on all of Q and K, then the exact attention loop for a subset of
+    query rows (all heads, all 4608 keys; all rows where the host finishes them within ~12 s), once on all threads and
+    once on one thread (~3 s). Every other configuration: one batch item on all threads (a few seconds each)."""
     import numpy as np
     import oracle as orc
-    H, d, L = 24, 128, 4608
-    q, k, v = (orc.round_to(orc.torch_randn_f32(3000 + i, L * H * d).reshape(L, H * d), "bf16") for i in (1, 2, 3))
-    cos, sin = orc.build_axial_rope_tables(512, 64, 64, d, (16, 56, 56))
+
+    def host(t):
+        return t.detach().float().cpu().numpy()
+
+    def parity(ref, got, dtype):
+        m = orc.compare(ref, got)
+        rel, mx = (5e-3, 2e-2) if dtype == "bf16" else (1e-3, 5e-3)
+        return {"rel_l2": float(f"{m['rel_l2']:.3e}"), "max_abs": float(f"{m['max_abs']:.3e}"), "within_tolerance": bool(m["rel_l2"] <= rel and m["max_abs"] <= mx)}
+
     threads = orc.max_threads()
+    H, d, L = 24, 128, 4608
+    q, k, v, cos, sin, out = headline
+    q, k, v, cos, sin = host(q), host(k), host(v), host(cos), host(sin)
     probe = np.arange(0, L, L // 32, dtype=np.int32)[:32]
     t0 = time.perf_counter()
     orc.sdpa(q, k, v, H, rows=probe)
@@ -178,12 +227,64 @@ def cpu_baseline():
     t0 = time.perf_counter()
     qr = orc.rope_apply(q, cos, sin, H, d, round_to_dtype="bf16")
     kr = orc.rope_apply(k, cos, sin, H, d, round_to_dtype="bf16")
-    orc.sdpa(qr, kr, v, H, rows=rows)
+    ref = orc.sdpa(qr, kr, v, H, rows=rows)
     dt = time.perf_counter() - t0
     flops = 4.0 * H * len(rows) * L * d
-    return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{len(rows)} of {L} query rows x 24 heads x all 4608 keys, RoPE on all of Q and K included, "
-                      f"{dt:.1f} s on {threads} OpenMP threads; full call extrapolates to {dt * L / len(rows):.0f} s"}
+    res = {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+           "sample": f"{len(rows)} of {L} query rows x 24 heads x all 4608 keys, RoPE on all of Q and K included, "
+                     f"{dt:.1f} s on {threads} OpenMP threads; full call extrapolates to {dt * L / len(rows):.0f} s",
+           "parity_of_timed_step": parity(ref[rows], host(out)[rows], "bf16")}
+    # the faithful single-thread form of the same loop, on fewer rows
+    per_row_1 = dt * threads / len(rows)                    # one thread's time per query row, about
+    rows1 = rows[np.unique(np.linspace(0, len(rows) - 1, max(8, min(len(rows), int(3.0 / max(per_row_1, 1e-6))))).astype(np.int32))]
+    t0 = time.perf_counter()
+    orc.sdpa(qr, kr, v, H, rows=rows1, n_threads=1)
+    dt1 = time.perf_counter() - t0
+    res["single_thread"] = {"value": round(4.0 * H * len(rows1) * L * d / dt1 / 1e12, 5), "unit": "TFLOP/s", "cores": 1,
+                            "sample": f"{len(rows1)} query rows x 24 heads x all keys (RoPE passes not included), {dt1:.1f} s on one thread; "
+                                      f"full call extrapolates to {dt1 * L / len(rows1):.0f} s"}
+    orc.sdpa(q[:8], k[:8], v[:8], H, n_threads=threads)      # back to all threads for what follows
+    if cin is None:
+        return res
+
+    def sdpa_cfg(name, qh, kh, vh, Hc, dtype, gpu_rows, n_rows, **kw):
+        Lq, Lk = qh.shape[0], kh.shape[0]
+        rws = np.unique(np.linspace(0, Lq - 1, n_rows).astype(np.int32))
+        t0 = time.perf_counter()
+        r = orc.sdpa(qh, kh, vh, Hc, rows=rws, **kw)
+        dtc = time.perf_counter() - t0
+        hi = kw.get("row_hi")
+        pairs = float(sum(int(hi[i]) for i in rws)) if hi is not None else float(len(rws)) * Lk
+        all_pairs = float(np.sum(hi)) if hi is not None else float(Lq) * Lk
+        dd = qh.shape[1] // Hc
+        return {"value": round(4.0 * Hc * pairs * dd / dtc / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
+                "sample": f"{len(rws)} of {Lq} query rows of one batch item x {Hc} heads, {dtc:.2f} s; one batch item extrapolates to "
+                          f"{dtc * all_pairs / pairs:.2f} s",
+                "parity": parity(r[rws], gpu_rows[rws], dtype)}
+
+    cfgs = {}
+    q1, k1, v1 = (host(t[0]) for t in cin["cfg1"])
+    cfgs["cfg1_sd15_selfattn_d40_fp16"] = sdpa_cfg("cfg1", q1, k1, v1, 8, "fp16", host(keep["cfg1"][0]), 4096)
+    q2, k2, v2 = (host(t[0]) for t in cin["cfg2a"])
+    cfgs["cfg2a_pixart_selfattn_d72_bf16"] = sdpa_cfg("cfg2a", q2, k2, v2, 16, "bf16", host(keep["cfg2a"][0]), 4096)
+    valid = cin["cfg2b"][3]
+    kc, vc = host(cin["cfg2b"][1][0])[:valid[0]], host(cin["cfg2b"][2][0])[:valid[0]]
+    cfgs["cfg2b_pixart_crossattn_d72_bf16"] = sdpa_cfg("cfg2b", q2, kc, vc, 16, "bf16", host(keep["cfg2b"][0]), 4096)
+    q4, k4, v4 = (host(t) for t in cin["cfg4"])
+    sq = [1024, 2048, 3072, 4096]
+    lo, hi = orc.rows_block_causal(4096, 4608, 512, sq, [512 + e for e in sq], [0] * 4)
+    cfgs["cfg4_qwen_blockcausal_prefixkv_d128_bf16"] = sdpa_cfg("cfg4", q4, k4, v4, 24, "bf16", host(keep["cfg4"]), 4096, row_lo=lo, row_hi=hi)
+    for name, key in (("cfg5a_sana_linear_n1024_d112_bf16", "cfg5a"), ("cfg5b_sana_linear_n4096_d112_bf16", "cfg5b")):
+        ql, kl, vl = (host(t[0]) for t in cin[key])
+        t0 = time.perf_counter()
+        r = orc.linear_attn_relu(ql, kl, vl, 20)
+        dtc = time.perf_counter() - t0
+        nbytes = 4 * ql.size * 2
+        cfgs[name] = {"value": round(nbytes / dtc / 1e9, 3), "unit": "GB/s", "cores": threads,
+                      "sample": f"one of the 2 batch items, whole, {dtc:.2f} s (algorithmic bytes of the bf16 streams, as for the GPU figure)",
+                      "parity": parity(r, host(keep[key][0]), "bf16")}
+    res["configs"] = cfgs
+    return res
 
 
 def main():
@@ -201,8 +302,8 @@ def main():
 
     B, H, d, txt, hp, wp = 1, 24, 128, 512, 64, 64
     L = txt + hp * wp
-    g = torch.Generator(device="cuda").manual_seed(3000)
-    q, k, v = (torch.randn(L, H * d, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(3))
+    g = torch.Generator(device="cuda").manual_seed(3000)     # (probe tensors only)
+    q, k, v = (seeded(torch, 3000 + i, (L, H * d), torch.bfloat16) for i in (1, 2, 3))
     cos, sin = bd.build_axial_rope_tables(txt, hp, wp, d, (16, 56, 56))
     out = torch.empty_like(q)
     kr = torch.empty_like(k)                 # the Kr scratch of the reference's joint_attention signature
@@ -262,14 +363,19 @@ def main():
         "pct_of_mfma_peak": round(100.0 * (flops / (ms_per_step * 1e-3) / 1e12) / PEAK_MFMA_BF16_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_MFMA_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "sdpa_fwd_pp_dma_kernel<__bf16>", "kernel_ms": round(kernel_ms, 4),
+                     "traffic_source": "constant from counter runs, not measured in this run: " + TRAFFIC_SOURCE,
+                     "kernel": "sdpa_fwd_pp_dma_kernel<__bf16, 128, dense>", "kernel_ms": round(kernel_ms, 4),
                      "step_ms_events": round(step_ms_events, 4)},
         "device": bd.device_info(),
     }
+    step()                                    # `out` holds the result of a step: compared with the checker below
+    torch.cuda.synchronize()
+    cin, keep = None, {}
     if not args.no_configs:
-        res["configs"] = all_configs(torch, bd)
+        cin = config_inputs(torch)
+        res["configs"] = all_configs(torch, bd, cin, keep)
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline()
+        res["cpu_baseline"] = cpu_baseline(torch, (q, k, v, cos, sin, out), cin, keep)
     print(json.dumps(res))
 
 
