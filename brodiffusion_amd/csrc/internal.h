@@ -125,5 +125,8 @@ struct LinearBatch { LinearProblem p[kMaxLinearProblems]; };
 // Validates and launches up to kMaxLinearProblems problems as one grid.
 // geglu: problem 0 has W (2 N, K) and bias (2 N), value half first; Y (M, N) = value * gelu_exact(gate).
 int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream_t stream, bool geglu = false);
+// The 256 x 256-tile form with LDS-DMA operand rings (linear_dma.hip): whether it takes a validated launch, and the launch.
+bool linear_dma_takes(const LinearBatch& batch, int n_problems, int n_cu);
+int launch_linear_dma(const LinearBatch& batch, int n_problems, int dtype, hipStream_t stream);
 
 }  // namespace mi
