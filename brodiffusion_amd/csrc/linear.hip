@@ -11,16 +11,10 @@
 // in flight while step t multiplies; one barrier per step. LDS rows are 144 bytes (128 + 16): 16 consecutive rows start
 // on distinct 16-byte bank groups, so the ds_read_b128 fragment reads are conflict free.
 // Up to three problems share one launch (blockIdx.y): the Q, K and V projections of an attention block.
-#include <cstdlib>
-
+// Large problems with 16-bit weights go to the 256 x 256-tile kernel of linear_dma.hip instead (launch_linear decides).
 #include "internal.h"
 
 namespace mi {
-// (a switch for measurements: MI_LINEAR_SMALL_TILES=1 in the environment keeps every launch on the kernels of this file)
-static bool linear_big_tiles_enabled() {
-    static const bool on = [] { const char* e = getenv("MI_LINEAR_SMALL_TILES"); return !(e && e[0] == '1'); }();
-    return on;
-}
 namespace gemm {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -320,7 +314,7 @@ int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream
         if (static_cast<long>((p.M + 63) / 64) * ((p.N + 63) / 64) > 0x7fffffffL) return fail("linear: problem too large for one launch");
     }
     if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_F16) return fail("linear: dtype %d is neither MI_DTYPE_F16 nor MI_DTYPE_BF16", dtype);
-    if (!geglu && linear_big_tiles_enabled() && linear_dma_takes(batch, n_problems, device_cu_count())) return launch_linear_dma(batch, n_problems, dtype, st);
+    if (!geglu && linear_dma_takes(batch, n_problems, device_cu_count())) return launch_linear_dma(batch, n_problems, dtype, st);
     if (dtype == MI_DTYPE_BF16) return gemm::launch_t<__bf16>(batch, n_problems, st, geglu);
     if (dtype == MI_DTYPE_F16) return gemm::launch_t<_Float16>(batch, n_problems, st, geglu);
     return fail("linear: dtype %d is neither MI_DTYPE_F16 nor MI_DTYPE_BF16", dtype);

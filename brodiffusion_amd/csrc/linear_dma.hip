@@ -1,5 +1,5 @@
-// Y = X W^T + b for large problems on gfx950: 256 x 256 output tiles, 8 wavefronts, operand tiles moved global -> LDS
-// by DMA into a four-stage ring.
+// Y = X W^T + b for large problems on gfx950: 256 x 256 output tiles, 8 wavefronts, operand blocks moved global -> LDS
+// by DMA into rings.
 //
 // The work group's 512 threads are 8 wavefronts in a 2 (feature halves) x 4 (token quarters) arrangement; a wavefront owns
 // 128 features x 64 tokens = 4 x 2 accumulator blocks of v_mfma_f32_32x32x16 (128 registers). As in linear.hip the product
