@@ -68,7 +68,9 @@ MI_API int mi_set_stream(void* stream);
 MI_API void* mi_get_stream(void);
 MI_API int mi_stream_synchronize(void* stream);
 
-/* Device memory for host code that owns no HIP of its own (the C++ Tensor type). */
+/* Device memory for host code that owns no HIP of its own (the C++ Tensor type). mi_memset_async is hipMemsetAsync:
+ * do not record it into a HIP graph (memset nodes have replayed wrongly on this hardware); inside a capture clear memory
+ * with a kernel of your own. No operator of this library calls it. */
 MI_API void* mi_malloc(size_t bytes);
 MI_API int mi_free(void* ptr);
 MI_API int mi_memcpy_h2d(void* dst, const void* src, size_t bytes);
