@@ -39,6 +39,9 @@ def test_graph_replays_equal_eager():
     o_ff = torch.empty(2 * 256, 640, dtype=torch.float16, device=dev)
     gain = (1 + 0.1 * rnd(d)).to(torch.bfloat16)
     o_hn = torch.empty_like(k)
+    # a linear layer large enough for the 256 x 256-tile kernel
+    xl, wl, bl = rnd(4608, 1024), rnd(3072, 1024) / 32, rnd(3072)
+    o_big = torch.empty(4608, 3072, dtype=torch.bfloat16, device=dev)
 
     def step():
         bd.joint_attention(q, k, v, cos, sin, d, H, out=o_joint, Kr=kr)
@@ -48,15 +51,16 @@ def test_graph_replays_equal_eager():
         bd.fused_linear_geglu(x.view(512, C), wg, bg, o_ff)
         bd.add_inplace_vec(o_blk, x)
         bd.headnorm_rope(k, gain, 1e-6, cos, sin, d, H, out=o_hn)
+        bd.linear_batched(wl, bl, xl, o_big)
 
-    outs = (o_joint, o_block, o_lin, o_blk, o_ff, o_hn, ws)
+    outs = (o_joint, o_block, o_lin, o_blk, o_ff, o_hn, o_big, ws)
     step()                                            # warm-up outside the capture (first-use set-up of the library)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
     for it in range(4):
-        for t in (q, k, v, lq, lk, lv, x):
+        for t in (q, k, v, lq, lk, lv, x, xl):
             t.copy_(rnd(*t.shape, dt=t.dtype))        # eager work between the replays: new input values
         step()
         torch.cuda.synchronize()
@@ -66,5 +70,5 @@ def test_graph_replays_equal_eager():
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for name, a, b in zip(("joint", "block-causal", "linear attention", "attention block", "geglu", "headnorm", "state"), eager, outs):
+        for name, a, b in zip(("joint", "block-causal", "linear attention", "attention block", "geglu", "headnorm", "large linear", "state"), eager, outs):
             assert torch.equal(a, b), f"replay {it}: {name} differs from the eager call"
