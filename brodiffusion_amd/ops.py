@@ -95,7 +95,8 @@ def _as3(op: str, t: torch.Tensor, name: str):
 
 
 def set_sdpa_kernel_choice(choice: int) -> None:
-    """0 = by problem size, 1 = 128-row tiles, 2 = 256-row ping-pong kernel (see mi_sdpa_set_kernel_choice)."""
+    """0 = by problem size, 1 = 128-row tiles, 2 = 256-row ping-pong kernel, 3 = the same with register-staged tiles
+    (see mi_sdpa_set_kernel_choice)."""
     capi.check(capi.lib().mi_sdpa_set_kernel_choice(choice), "set_sdpa_kernel_choice")
 
 
