@@ -12,6 +12,9 @@
 // on distinct 16-byte bank groups, so the ds_read_b128 fragment reads are conflict free.
 // Up to three problems share one launch (blockIdx.y): the Q, K and V projections of an attention block.
 // Large problems with 16-bit weights go to the 256 x 256-tile kernel of linear_dma.hip instead (launch_linear decides).
+#include <type_traits>
+#include <utility>
+
 #include "internal.h"
 
 namespace mi {
@@ -44,6 +47,7 @@ template <> struct Mma<_Float16> {
 constexpr int kBK = 64;                // contraction elements per step
 constexpr int kRowBytes = kBK * 2 + 16;  // LDS row stride
 constexpr int kThreads = 256;
+constexpr int kRing = 5;               // contraction steps in flight in the ring form (K a multiple of 320)
 
 // One 16-byte chunk column (tid % 8) and 32 rows per pass: ROWS / 32 loads per thread and tile.
 // GATED (the W tile of the GEGLU form): the tile's 32-row groups alternate between the value half and the gate half
@@ -101,19 +105,167 @@ __device__ __forceinline__ void store_tile_int8(const u32x2 (&raw)[ROWS / 32], c
     }
 }
 
-// GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
+// x * Phi(x), the erf form of GELU (gelu_exact_scalar, src/fused_transformer.cu:89-92), branch free: with z = |x| / sqrt 2,
+// erfc(z) = t exp(-z^2 + P(t)), t = 1 / (1 + z / 2) (the Chebyshev fit of Numerical Recipes' erfcc, fractional error below
+// 1.2e-7 for all z >= 0), and 1 + erf(x / sqrt 2) = erfc(z) for x < 0, 2 - erfc(z) otherwise - so the left tail keeps its
+// relative accuracy, which the sum 1 + erf loses to cancellation.
+__device__ __forceinline__ float gelu_erf(float x) {
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.5f, z, 1.f));
+    float q = 0.17087277f;
+    q = __builtin_fmaf(q, t, -0.82215223f);
+    q = __builtin_fmaf(q, t, 1.48851587f);
+    q = __builtin_fmaf(q, t, -1.13520398f);
+    q = __builtin_fmaf(q, t, 0.27886807f);
+    q = __builtin_fmaf(q, t, -0.18628806f);
+    q = __builtin_fmaf(q, t, 0.09678418f);
+    q = __builtin_fmaf(q, t, 0.37409196f);
+    q = __builtin_fmaf(q, t, 1.00002368f);
+    q = __builtin_fmaf(q, t, -1.26551223f);
+    const float e = t * __builtin_amdgcn_exp2f(__builtin_fmaf(-z, z, q) * 1.4426950408889634f);
+    return 0.5f * x * (x < 0.f ? e : 2.f - e);
+}
+
+// What the two kernels below share: the MFMA step and the epilogue of a BM x BN tile held by WM x WN wavefronts. GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
 // value * gelu_exact(gate) (diffusers' GEGLU with the erf form of GELU). A work group's 128 W-tile rows are 64 output
 // features times {value, gate}; each wavefront holds both accumulators of its 32 features, so the product of the two
 // halves never leaves registers and the (M, 2 N) intermediate does not exist.
 // W8: W is INT8 (N, K) with one FP32 scale per row (LinearProblem::w_scale): Y = (X Wq^T) * scale + bias.
-template <typename T, int BM, int BN, bool GEGLU = false, bool W8 = false>
-__global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batch) {
+template <typename T, int BM, int BN, bool GEGLU, bool W8, int WM = 2, int WN = 2>
+struct TileMath {
     using M = Mma<T>;
-    constexpr int TM = BM / 64, TN = BN / 64;  // 32 x 32 blocks per wavefront along tokens / features
+    using V4 = typename M::v4;
+    static constexpr int NT = 64 * WM * WN;                       // threads: WM x WN wavefronts over tokens x features
+    static constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);  // 32 x 32 blocks per wavefront along tokens / features
     static_assert(!GEGLU || TN == 2, "the GEGLU form pairs the two feature blocks of a wavefront");
     static_assert(!(GEGLU && W8), "no INT8-weight GEGLU form");
-    constexpr int BN_OUT = GEGLU ? BN / 2 : BN;   // output features per tile
-    constexpr int X_BYTES = BM * kRowBytes, W_BYTES = BN * kRowBytes;
+    static constexpr int BN_OUT = GEGLU ? BN / 2 : BN;   // output features per tile
+    static constexpr int X_BYTES = BM * kRowBytes, W_BYTES = BN * kRowBytes;
+    static constexpr int kOutRow = BN_OUT * 2 + 16;      // staged output row (bytes)
+    static constexpr int kOutBytes = BM * kOutRow;
+
+    int tid, lq, lh, wm, wn;
+    __device__ __forceinline__ explicit TileMath(int tid_) : tid(tid_) {
+        const int lane = tid & 63, wave = tid >> 6;
+        lq = lane & 31; lh = lane >> 5; wm = wave % WM; wn = wave / WM;
+    }
+    static __device__ __forceinline__ void clear(f32x16 (&acc)[TN][TM]) {
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int b = 0; b < TM; ++b)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+    }
+    // The bias of this lane's features of the tile at feature n0, requested long before the epilogue (there each of these
+    // loads would be a memory latency of its own). Straight-line code: lanes without a bias read the first bytes of W and
+    // blank what they got, so that no wait for these loads is placed before the operand loads that follow.
+    // GEGLU: [0] = value half, [1] = gate half.
+    __device__ __forceinline__ void request_bias(V4 (&braw)[TN][4], const LinearProblem& p, int n0) const {
+        const T* bias = static_cast<const T*>(p.bias);
+#pragma unroll
+        for (int a = 0; a < TN; ++a)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int feat = GEGLU ? n0 + wn * 32 + 8 * g + 4 * lh : n0 + (wn * TN + a) * 32 + 8 * g + 4 * lh;
+                const bool there = bias != nullptr && feat < p.N;
+                const T* src = there ? bias + feat + (GEGLU ? a * p.N : 0) : static_cast<const T*>(p.w);
+                const V4 raw = *reinterpret_cast<const V4*>(src);
+                const V4 zero = {static_cast<T>(0.f), static_cast<T>(0.f), static_cast<T>(0.f), static_cast<T>(0.f)};
+                braw[a][g] = there ? raw : zero;
+            }
+    }
+    // the four k-substeps of 16 of one step for every 32 x 32 block of this wavefront, operands from the LDS tile pair at `cur`
+    __device__ __forceinline__ void multiply(f32x16 (&acc)[TN][TM], const char* cur) const {
+        const char* xs = cur + (wm * TM * 32 + lq) * kRowBytes + lh * 16;
+        const char* ws = cur + X_BYTES + (wn * TN * 32 + lq) * kRowBytes + lh * 16;
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+            typename M::v8 xf[TM], wf[TN];
+#pragma unroll
+            for (int b = 0; b < TM; ++b) xf[b] = *reinterpret_cast<const typename M::v8*>(xs + b * 32 * kRowBytes + kk * 32);
+#pragma unroll
+            for (int a = 0; a < TN; ++a) wf[a] = *reinterpret_cast<const typename M::v8*>(ws + a * 32 * kRowBytes + kk * 32);
+#pragma unroll
+            for (int a = 0; a < TN; ++a)
+#pragma unroll
+                for (int b = 0; b < TM; ++b) acc[a][b] = M::run(wf[a], xf[b], acc[a][b]);
+        }
+    }
+    // acc[a][b][4g + i]: feature n0 + (wn*TN + a)*32 + 8g + 4*lh + i of token m0 + (wm*TM + b)*32 + lq.
+    // The results leave through LDS (`stage`, kOutBytes, not in use by anything else): a lane holds 4 features of one token
+    // per group, and written from there a wavefront's store instruction would touch 32 rows of Y with 16 bytes each.
+    // Staged, consecutive threads write consecutive 16-byte pieces of a row.
+    __device__ __forceinline__ void write_tile(const f32x16 (&acc)[TN][TM], const V4 (&braw)[TN][4], const LinearProblem& p, char* stage,
+                                               int m0, int n0) const {
+        if constexpr (GEGLU) {
+            // acc[0] = value, acc[1] = gate of features n0 + wn*32 + 8g + 4*lh + i
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int feat = wn * 32 + 8 * g + 4 * lh;
+                float bv[4], bg[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { bv[i] = static_cast<float>(braw[0][g][i]); bg[i] = static_cast<float>(braw[1][g][i]); }
+#pragma unroll
+                for (int b = 0; b < TM; ++b) {
+                    V4 o;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float val = acc[0][b][4 * g + i] + bv[i];
+                        const float gate = acc[1][b][4 * g + i] + bg[i];
+                        o[i] = static_cast<T>(val * gelu_erf(gate));
+                    }
+                    *reinterpret_cast<V4*>(stage + ((wm * TM + b) * 32 + lq) * kOutRow + feat * 2) = o;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < TN; ++a) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int feat = (wn * TN + a) * 32 + 8 * g + 4 * lh;
+                    float bv[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) bv[i] = static_cast<float>(braw[a][g][i]);
+                    float sc[4] = {1.f, 1.f, 1.f, 1.f};
+                    if constexpr (W8) {
+                        if (n0 + feat < p.N) {   // N is a multiple of 8, so the 4 features are in or out together
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) sc[i] = p.w_scale[n0 + feat + i];
+                        }
+                    }
+#pragma unroll
+                    for (int b = 0; b < TM; ++b) {
+                        V4 o;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            if constexpr (W8) o[i] = static_cast<T>(__builtin_fmaf(acc[a][b][4 * g + i], sc[i], bv[i]));
+                            else o[i] = static_cast<T>(acc[a][b][4 * g + i] + bv[i]);
+                        }
+                        *reinterpret_cast<V4*>(stage + ((wm * TM + b) * 32 + lq) * kOutRow + feat * 2) = o;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        char* yg = static_cast<char*>(p.y);
+        constexpr int PPR = BN_OUT / 8;   // 16-byte pieces per staged row
+#pragma unroll
+        for (int idx = tid; idx < BM * PPR; idx += NT) {
+            const int row = idx / PPR, piece = idx % PPR;
+            if (m0 + row < p.M && n0 + piece * 8 < p.N)
+                *reinterpret_cast<u32x4*>(yg + (static_cast<long>(m0 + row) * p.ldy + n0 + piece * 8) * 2) =
+                    *reinterpret_cast<const u32x4*>(stage + row * kOutRow + piece * 16);
+        }
+    }
+};
+
+// The streaming form: one work group per output tile, one contraction step prefetched while the previous one is multiplied.
+template <typename T, int BM, int BN, bool GEGLU = false, bool W8 = false>
+__global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batch) {
+    using TM_ = TileMath<T, BM, BN, GEGLU, W8>;
+    constexpr int TM = TM_::TM, TN = TM_::TN, BN_OUT = TM_::BN_OUT, X_BYTES = TM_::X_BYTES, W_BYTES = TM_::W_BYTES;
+    static_assert(TM_::kOutBytes <= 2 * (X_BYTES + W_BYTES), "the staged output fits the operand buffers");
     extern __shared__ __attribute__((aligned(16))) char lds[];  // [2][X tile ; W tile]
 
     const LinearProblem& p = batch.p[blockIdx.y];
@@ -122,19 +274,15 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
     if (static_cast<int>(blockIdx.x) >= tiles_m * tiles_n) return;  // uniform: this problem has fewer tiles than the grid
     const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN_OUT;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int lq = lane & 31, lh = lane >> 5;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int tid = threadIdx.x;
+    const TM_ tm(tid);
     const char* xg = static_cast<const char*>(p.x);
     const char* wg = static_cast<const char*>(p.w);
 
     f32x16 acc[TN][TM];
-#pragma unroll
-    for (int a = 0; a < TN; ++a)
-#pragma unroll
-        for (int b = 0; b < TM; ++b)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+    TM_::clear(acc);
+    typename TM_::V4 braw[TN][4];
+    tm.request_bias(braw, p, n0);
 
     // While tile t is multiplied out of LDS, tile t + 1 is on its way into registers; it goes to the other LDS buffer at
     // the end of the step. (The loads stay under `if (more)`: issued unconditionally, the compiler sinks them behind
@@ -164,86 +312,124 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
         char* nxt = lds + ((t + 1) & 1) * (X_BYTES + W_BYTES);
         const bool more = t + 1 < n_steps;
         if (more) load_tiles((t + 1) * kBK);
-        const char* xs = cur + (wm * TM * 32 + lq) * kRowBytes + lh * 16;
-        const char* ws = cur + X_BYTES + (wn * TN * 32 + lq) * kRowBytes + lh * 16;
-#pragma unroll
-        for (int kk = 0; kk < kBK / 16; ++kk) {
-            typename M::v8 xf[TM], wf[TN];
-#pragma unroll
-            for (int b = 0; b < TM; ++b) xf[b] = *reinterpret_cast<const typename M::v8*>(xs + b * 32 * kRowBytes + kk * 32);
-#pragma unroll
-            for (int a = 0; a < TN; ++a) wf[a] = *reinterpret_cast<const typename M::v8*>(ws + a * 32 * kRowBytes + kk * 32);
-#pragma unroll
-            for (int a = 0; a < TN; ++a)
-#pragma unroll
-                for (int b = 0; b < TM; ++b) acc[a][b] = M::run(wf[a], xf[b], acc[a][b]);
-        }
+        tm.multiply(acc, cur);
         if (more) store_tiles(nxt, (t + 1) * kBK);
         __syncthreads();
     }
+    tm.write_tile(acc, braw, p, lds, m0, n0);
+}
 
-    // acc[a][b][4g + i]: feature n0 + (wn*TN + a)*32 + 8g + 4*lh + i of token m0 + (wm*TM + b)*32 + lq
-    char* yg = static_cast<char*>(p.y);
-    const T* bias = static_cast<const T*>(p.bias);
-    if constexpr (GEGLU) {
-        // acc[0] = value, acc[1] = gate of features n0 + wn*32 + 8g + 4*lh + i
+// The ring form, for contractions that are a multiple of kRing steps (the channel counts of the U-Net: 320, 640, 1280 and
+// their FF multiples). A work group of the streaming form lives a few microseconds, most of them waiting: every step for
+// the one tile it prefetched, at the start for its first, and the tile's few hundred cycles of MFMAs hide none of it.
+// Here a work group stays and walks output tiles (a contiguous run per XCD, so that the tiles sharing X rows meet in one
+// L2), and the operand tiles of kRing consecutive steps are in flight at any time, across tile boundaries: the registers
+// of step t + 1 go to LDS during step t and are at once requested again for step t + 1 + kRing (of this output tile or of
+// the next). All loads are unconditional, straight-line code (past the last tile they re-read the first rows of the
+// operands), so the waits the compiler places count exactly, and nothing ever waits for a store.
+template <typename T, int BM, int BN, bool GEGLU = false, int WM = 2, int WN = 2>
+__global__ __launch_bounds__(64 * WM * WN) void linear_ring_kernel(const LinearBatch batch) {
+    using TM_ = TileMath<T, BM, BN, GEGLU, false, WM, WN>;
+    constexpr int RP = TM_::NT / 8;             // tile rows per pass of the work group (8 threads per 128-byte row piece)
+    constexpr int XL = BM / RP, WL = BN / RP;   // loads per thread, operand and step
+    static_assert(BM % RP == 0 && BN % RP == 0 && RP % 32 == 0, "whole passes; a pass covers whole 32-row groups");
+    constexpr int TM = TM_::TM, TN = TM_::TN, BN_OUT = TM_::BN_OUT, X_BYTES = TM_::X_BYTES, W_BYTES = TM_::W_BYTES;
+    constexpr int R = kRing;
+    extern __shared__ __attribute__((aligned(16))) char lds[];  // [2][X tile ; W tile], then the staged output
+    char* const stage = lds + 2 * (X_BYTES + W_BYTES);
+
+    const LinearProblem& p = batch.p[blockIdx.y];
+    const int tiles_n = (p.N + BN_OUT - 1) / BN_OUT;
+    const int tiles_m = (p.M + BM - 1) / BM;
+    const int n_tiles = tiles_m * tiles_n;
+    // consecutive work-group ids go to the 8 XCDs in turn: every XCD takes a contiguous run of tiles
+    const int run = (n_tiles + 7) >> 3;
+    const int stride = static_cast<int>(gridDim.x) >> 3;
+    const int run_end = min(((static_cast<int>(blockIdx.x) & 7) + 1) * run, n_tiles);
+    int tile = (static_cast<int>(blockIdx.x) & 7) * run + (static_cast<int>(blockIdx.x) >> 3);
+    if (tile >= run_end) return;   // uniform
+
+    const int tid = threadIdx.x;
+    const TM_ tm(tid);
+    const char* xg = static_cast<const char*>(p.x);
+    const char* wg = static_cast<const char*>(p.w);
+    const unsigned x_pitch = static_cast<unsigned>(p.ldx) * 2u, w_pitch = static_cast<unsigned>(p.ldw) * 2u;
+    const unsigned k_bytes = static_cast<unsigned>(p.K) * 2u;
+
+    // ── the load cursor: kRing steps ahead of the multiplication; 32-bit byte offsets from the operand bases ──
+    int c_tile = tile;
+    unsigned c_k = 0;                       // byte offset of the cursor's step in a row (uniform)
+    const unsigned kcol = (tid & 7) * 16u;  // this thread's 16 bytes of a step
+    unsigned xrow[XL], wrow[WL];
+    auto cursor_rows = [&]() {
+        if (c_tile < run_end) {
+            const int m0 = (c_tile / tiles_n) * BM, n0 = (c_tile % tiles_n) * BN_OUT;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int n = n0 + wn * 32 + 8 * g + 4 * lh;
-            if (n >= p.N) continue;
-            float bv[4] = {0.f, 0.f, 0.f, 0.f}, bg[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
-                const typename M::v4 b4 = *reinterpret_cast<const typename M::v4*>(bias + n);
-                const typename M::v4 g4 = *reinterpret_cast<const typename M::v4*>(bias + p.N + n);
+            for (int i = 0; i < XL; ++i) xrow[i] = static_cast<unsigned>(min(m0 + (tid >> 3) + RP * i, p.M - 1)) * x_pitch + kcol;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { bv[i] = static_cast<float>(b4[i]); bg[i] = static_cast<float>(g4[i]); }
+            for (int i = 0; i < WL; ++i) {
+                // (GEGLU: the tile's 32-row groups alternate between the value and the gate half of W, see load_tile)
+                const int r = (tid >> 3) + RP * i, grp = r >> 5;
+                const int row = GEGLU ? min(n0 + 32 * (grp >> 1) + (r & 31), p.N - 1) + (grp & 1) * p.N : min(n0 + r, p.N - 1);
+                wrow[i] = static_cast<unsigned>(row) * w_pitch + kcol;
             }
+        } else {   // past the last tile: the first row of either operand
 #pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                const int m = m0 + (wm * TM + b) * 32 + lq;
-                if (m >= p.M) continue;
-                typename M::v4 o;
+            for (int i = 0; i < XL; ++i) xrow[i] = kcol;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float val = acc[0][b][4 * g + i] + bv[i];
-                    const float gate = acc[1][b][4 * g + i] + bg[i];
-                    o[i] = static_cast<T>(val * (0.5f * gate * (1.0f + erff(gate * 0.70710678118654752f))));
-                }
-                *reinterpret_cast<typename M::v4*>(yg + (static_cast<long>(m) * p.ldy + n) * 2) = o;
-            }
+            for (int i = 0; i < WL; ++i) wrow[i] = kcol;
         }
-        return;
-    }
+    };
+    u32x4 xs_[R][XL], ws_[R][WL];
+    auto request = [&](auto s_tag) {
+        constexpr int s = decltype(s_tag)::value;
 #pragma unroll
-    for (int a = 0; a < TN; ++a) {
+        for (int i = 0; i < XL; ++i) xs_[s][i] = *reinterpret_cast<const u32x4*>(xg + (xrow[i] + c_k));
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int n = n0 + (wn * TN + a) * 32 + 8 * g + 4 * lh;
-            if (n >= p.N) continue;  // N is a multiple of 8, so the 4 features are in or out together
-            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias) {
-                const typename M::v4 b4 = *reinterpret_cast<const typename M::v4*>(bias + n);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) bv[i] = static_cast<float>(b4[i]);
-            }
-            float sc[4] = {1.f, 1.f, 1.f, 1.f};
-            if constexpr (W8) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) sc[i] = p.w_scale[n + i];
-            }
-#pragma unroll
-            for (int b = 0; b < TM; ++b) {
-                const int m = m0 + (wm * TM + b) * 32 + lq;
-                if (m >= p.M) continue;
-                typename M::v4 o;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if constexpr (W8) o[i] = static_cast<T>(__builtin_fmaf(acc[a][b][4 * g + i], sc[i], bv[i]));
-                    else o[i] = static_cast<T>(acc[a][b][4 * g + i] + bv[i]);
-                }
-                *reinterpret_cast<typename M::v4*>(yg + (static_cast<long>(m) * p.ldy + n) * 2) = o;
-            }
+        for (int i = 0; i < WL; ++i) ws_[s][i] = *reinterpret_cast<const u32x4*>(wg + (wrow[i] + c_k));
+        c_k += kBK * 2;
+        if (c_k == k_bytes) {   // uniform: on to the next output tile of this work group
+            c_k = 0;
+            c_tile += stride;
+            cursor_rows();
         }
+    };
+    auto to_lds = [&](auto s_tag, char* dst) {
+        constexpr int s = decltype(s_tag)::value;
+#pragma unroll
+        for (int i = 0; i < XL; ++i) *reinterpret_cast<u32x4*>(dst + ((tid >> 3) + RP * i) * kRowBytes + (tid & 7) * 16) = xs_[s][i];
+#pragma unroll
+        for (int i = 0; i < WL; ++i) *reinterpret_cast<u32x4*>(dst + X_BYTES + ((tid >> 3) + RP * i) * kRowBytes + (tid & 7) * 16) = ws_[s][i];
+    };
+    cursor_rows();
+    [&]<int... S>(std::integer_sequence<int, S...>) { (request(std::integral_constant<int, S>{}), ...); }(std::make_integer_sequence<int, R>{});
+    to_lds(std::integral_constant<int, 0>{}, lds);
+    request(std::integral_constant<int, 0>{});
+    __syncthreads();
+
+    const int groups = p.K / (R * kBK);
+    int par = 0;   // LDS buffer of the step about to be multiplied
+    f32x16 acc[TN][TM];
+    for (; tile < run_end; tile += stride) {
+        const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN_OUT;
+        typename TM_::V4 braw[TN][4];
+        tm.request_bias(braw, p, n0);
+        TM_::clear(acc);
+        int g = 0;
+        do {   // (at least one group: a loop that may not run would make the wait for the bias a wait for every load)
+            [&]<int... S>(std::integer_sequence<int, S...>) {
+                ([&] {
+                    // step S of the group: the registers of the following step go to the other buffer and are requested anew
+                    constexpr int nxt = (S + 1) % R;
+                    to_lds(std::integral_constant<int, nxt>{}, lds + (par ^ 1) * (X_BYTES + W_BYTES));
+                    request(std::integral_constant<int, nxt>{});
+                    tm.multiply(acc, lds + par * (X_BYTES + W_BYTES));
+                    __syncthreads();
+                    par ^= 1;
+                }(), ...);
+            }(std::make_integer_sequence<int, R>{});
+        } while (++g < groups);
+        tm.write_tile(acc, braw, p, stage, m0, n0);
     }
 }
 
@@ -270,9 +456,50 @@ int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
     return 0;
 }
 
+// The ring form: 16-bit weights, contractions that are a multiple of kRing steps, operands addressable with 32-bit byte
+// offsets from their bases.
+inline bool ring_form_takes(const LinearBatch& batch, int n_problems, bool geglu) {
+    for (int i = 0; i < n_problems; ++i) {
+        const LinearProblem& p = batch.p[i];
+        if (p.w_scale != nullptr || p.K % (kRing * kBK) != 0) return false;
+        if (static_cast<long>(p.M) * p.ldx * 2 >= (1L << 32) || static_cast<long>(p.N) * (geglu ? 2 : 1) * p.ldw * 2 >= (1L << 32)) return false;
+    }
+    return true;
+}
+
+template <typename T, int BM, int BN, bool GEGLU = false, int WM = 2, int WN = 2>
+int launch_ring(const LinearBatch& batch, int n_problems, hipStream_t st) {
+    using TM_ = TileMath<T, BM, BN, GEGLU, false, WM, WN>;
+    int max_tiles = 0;
+    for (int i = 0; i < n_problems; ++i) {
+        const LinearProblem& p = batch.p[i];
+        max_tiles = max(max_tiles, ((p.M + BM - 1) / BM) * ((p.N + TM_::BN_OUT - 1) / TM_::BN_OUT));
+    }
+    constexpr size_t lds = 2 * static_cast<size_t>(BM + BN) * kRowBytes + TM_::kOutBytes;
+    static_assert(lds <= 160 * 1024, "operand buffers and staged output exceed the LDS of a compute unit");
+    auto kern = linear_ring_kernel<T, BM, BN, GEGLU, WM, WN>;
+    static thread_local int per_cu = 0;   // work groups a compute unit holds at once
+    if (per_cu == 0) {
+        if (lds > 64 * 1024)
+            MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        int n = 0;
+        MI_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kern), TM_::NT, lds));
+        per_cu = max(n, 1);
+    }
+    // as many work groups as the GPU holds at once, split over the problems; a multiple of 8 (one run of tiles per XCD)
+    const int grid_x = min((max_tiles + 7) / 8 * 8, max(8, per_cu * device_cu_count() / n_problems / 8 * 8));
+    hipLaunchKernelGGL(kern, dim3(grid_x, n_problems), dim3(TM_::NT), lds, st, batch);
+    MI_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 template <typename T>
 int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool geglu) {
     if (geglu) {
+        // the ring form when its 256-token tiles give every compute unit one: FF1 of the U-Net's widest level
+        // (8192 x 320 -> 2 x 1280: 33 us against 40 for the streaming form)
+        if (ring_form_takes(batch, 1, true) && static_cast<long>((batch.p[0].M + 255) / 256) * ((batch.p[0].N + 63) / 64) >= device_cu_count())
+            return launch_ring<T, 256, 128, true, 4, 2>(batch, 1, st);
         // 64-token tiles unless 128-token tiles alone fill the GPU twice over
         const long big = static_cast<long>((batch.p[0].M + 127) / 128) * ((batch.p[0].N + 63) / 64);
         if (big >= 2L * device_cu_count() && batch.p[0].K >= 1024) return launch_tiles<T, 128, 128, true>(batch, 1, st);
@@ -280,7 +507,7 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool gegl
     }
     // 128 x 128 tiles when they alone fill the GPU twice over and the contraction is long enough to pay for their
     // longer prologue, else 64 x 64 (more, smaller work groups: the projections of one attention block are small
-    // problems; Q, K, V of 8192 x 320 x 320 in one launch: 15 us with 64 x 64 tiles, 22 us with 128 x 128)
+    // problems)
     long big = 0;
     int min_k = 0x7fffffff;
     for (int i = 0; i < n_problems; ++i) {

@@ -18,7 +18,10 @@ def uniform(seed, shape, scale, dtype, oracle, offset=0.0):
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
-@pytest.mark.parametrize("B,d_in,d_out", [(40, 64, 48), (128, 128, 96), (8192, 320, 1280), (2048, 640, 2560), (77, 1280, 5120), (1, 8, 8)])
+@pytest.mark.parametrize("B,d_in,d_out", [(40, 64, 48), (128, 128, 96), (8192, 320, 1280), (2048, 640, 2560), (77, 1280, 5120), (1, 8, 8),
+                                          # ragged last tiles of the 256-token-tile form (in_features a multiple of 320, at least one
+                                          # tile per compute unit): 160 of 256 tokens, 8 of 64 features
+                                          (4000, 320, 1032), (3000, 640, 1480)])
 def test_fused_linear_geglu(oracle, dtype, B, d_in, d_out):
     x = uniform(21, (B, d_in), 1.0, dtype, oracle)
     w = uniform(22, (2 * d_out, d_in), 0.1, dtype, oracle)
