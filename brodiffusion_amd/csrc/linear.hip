@@ -3,14 +3,16 @@
 // X is (M, K) and W is (N, K), both with the contraction index contiguous, which is exactly the operand layout of
 // v_mfma_f32_32x32x16: a lane reads 8 consecutive contraction elements of ONE row of either operand. The product is
 // computed transposed (MFMA rows = output features, MFMA columns = tokens), so a lane ends up with 4 consecutive
-// output features of one token per accumulator group and writes them as one 8-byte store, bias added in FP32 before
-// the single rounding.
+// output features of one token per accumulator group; bias is added in FP32 before the single rounding and the tile
+// leaves through LDS as whole 16-byte pieces of rows of Y.
 //
-// Work group: 256 threads = 4 wavefronts in a 2 x 2 arrangement over a BM x BN output tile, contraction step 64.
-// Operand tiles go global -> registers -> LDS with 16-byte accesses, double buffered so that the loads of step t+1 are
-// in flight while step t multiplies; one barrier per step. LDS rows are 144 bytes (128 + 16): 16 consecutive rows start
-// on distinct 16-byte bank groups, so the ds_read_b128 fragment reads are conflict free.
+// Streaming form (linear_kernel): 256 threads = 4 wavefronts in a 2 x 2 arrangement over a BM x BN output tile,
+// contraction step 64. Operand tiles go global -> registers -> LDS with 16-byte accesses, double buffered so that the
+// loads of step t+1 are in flight while step t multiplies; one barrier per step. LDS rows are 144 bytes (128 + 16): 16
+// consecutive rows start on distinct 16-byte bank groups, so the ds_read_b128 fragment reads are conflict free.
 // Up to three problems share one launch (blockIdx.y): the Q, K and V projections of an attention block.
+// Ring form (linear_ring_kernel): work groups that stay and walk tiles with five contraction steps in flight, for the
+// GEGLU FF1 of the U-Net (launch_t decides).
 // Large problems with 16-bit weights go to the 256 x 256-tile kernel of linear_dma.hip instead (launch_linear decides).
 #include <type_traits>
 #include <utility>
