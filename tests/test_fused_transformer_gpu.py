@@ -40,6 +40,42 @@ def test_fused_linear_geglu(oracle, dtype, B, d_in, d_out):
     assert np.abs(to_np(y) - unfused).max() <= 0.008 + 0.01 * np.abs(unfused).max()
 
 
+@pytest.mark.parametrize("B,d_in,d_out", [(200, 64, 72), (4000, 320, 1032)])
+def test_fused_linear_geglu_without_bias(oracle, B, d_in, d_out):
+    """No bias (the C ABI takes a null pointer): both kernel forms, the small one and the one that walks 256-token tiles."""
+    dtype = "bf16"
+    x = uniform(25, (B, d_in), 1.0, dtype, oracle)
+    w = uniform(26, (2 * d_out, d_in), 0.1, dtype, oracle)
+    y = to_np(bd.fused_linear_geglu(to_dev(x, dtype), to_dev(w, dtype), None))
+    ref = oracle.geglu_exact(oracle.linear(x, w, None))
+    err = np.abs(y - ref)
+    assert np.all(err <= 2.0 ** -8 * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)
+
+
+def test_geglu_gate_tails(oracle):
+    """gelu_exact over the whole range of the gate, one gate value per output column: a zero weight and the gate's value as
+    its bias, value half = 1. The left tail keeps its relative accuracy (x Phi(x) down to the smallest normal numbers of
+    the output type), the right tail is the identity."""
+    dtype, B, d_in = "bf16", 64, 64
+    gates = np.concatenate([np.linspace(-12.0, 12.0, 193), [-0.0, 1e-3, -1e-3, 30.0, -30.0, 5.5, -5.5]]).astype(np.float32)
+    gates = oracle.round_to(gates, dtype)
+    d_out = len(gates)                                   # 200 columns: a multiple of 8
+    w = np.zeros((2 * d_out, d_in), np.float32)
+    b = np.concatenate([np.ones(d_out, np.float32), gates])
+    x = uniform(27, (B, d_in), 1.0, dtype, oracle)
+    y = to_np(bd.fused_linear_geglu(to_dev(x, dtype), to_dev(w, dtype), to_dev(b, dtype)))
+    # x Phi(x) with Phi from the complementary error function in double (scipy): 1 + erf loses the left tail to cancellation,
+    # in the checker's double arithmetic beyond x = -7 and in the reference's FP32 beyond x = -5.5, where it returns 0
+    from scipy.special import erfc
+    g64 = gates.astype(np.float64)
+    ref = np.tile((0.5 * g64 * erfc(-g64 / np.sqrt(2.0)))[None, :], (B, 1))
+    assert np.isfinite(y).all()
+    assert np.all(np.abs(y - ref) <= 2.0 ** -8 * np.abs(ref) * 1.05 + 1e-37)   # one bf16 rounding, relative, at every magnitude
+    near = np.abs(gates) <= 5.0                                               # where the checker's own formula is accurate
+    chk = oracle.geglu_exact(np.tile(b[None, :], (B, 1)))
+    assert np.all(np.abs(y[:, near] - chk[:, near]) <= 2.0 ** -8 * np.abs(chk[:, near]) * 1.05 + 1e-12)
+
+
 def test_geglu_halves_and_errors(oracle):
     """Value half first, gate half second: a weight whose gate rows are zero and gate bias is large gives a * g."""
     dtype, B, d_in, d_out = "fp16", 64, 64, 64
