@@ -519,6 +519,9 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool gegl
     const bool w8 = batch.p[0].w_scale != nullptr;
     if (big >= 2L * device_cu_count() && min_k >= 1024)
         return w8 ? launch_tiles<T, 128, 128, false, true>(batch, n_problems, st) : launch_tiles<T, 128, 128>(batch, n_problems, st);
+    // long contractions over few tiles (FF2 of the U-Net: 2048 x 2560 -> 640, 30 -> 21 us; 8192 x 1280 -> 320, 22 -> 17 us): the
+    // ring form, whose five steps in flight shorten the per-step chain of memory latencies; at 320 it measures the same
+    if (min_k >= 2 * kRing * kBK && ring_form_takes(batch, n_problems, false)) return launch_ring<T, 64, 64>(batch, n_problems, st);
     return w8 ? launch_tiles<T, 64, 64, false, true>(batch, n_problems, st) : launch_tiles<T, 64, 64>(batch, n_problems, st);
 }
 
