@@ -107,25 +107,29 @@ __device__ __forceinline__ void store_tile_int8(const u32x2 (&raw)[ROWS / 32], c
     }
 }
 
-// x * Phi(x), the erf form of GELU (gelu_exact_scalar, src/fused_transformer.cu:89-92), branch free: with z = |x| / sqrt 2,
+// x * Phi(x), the erf form of GELU (gelu_exact_scalar, src/fused_transformer.cu:89-92), branch free. With z = |x| / sqrt 2,
 // erfc(z) = t exp(-z^2 + P(t)), t = 1 / (1 + z / 2) (the Chebyshev fit of Numerical Recipes' erfcc, fractional error below
-// 1.2e-7 for all z >= 0), and 1 + erf(x / sqrt 2) = erfc(z) for x < 0, 2 - erfc(z) otherwise - so the left tail keeps its
-// relative accuracy, which the sum 1 + erf loses to cancellation.
+// 1.2e-7 for all z >= 0), and Phi(x) = erfc(z) / 2 for x < 0, 1 - erfc(z) / 2 otherwise - so the left tail keeps its
+// relative accuracy, which the sum 1 + erf loses to cancellation. Here in base 2 with the constants folded: the
+// coefficients of P are multiplied by log2 e, its constant term also takes the factor 1/2 (-1 in the exponent), and
+// z^2 log2 e = (|x| sqrt(log2 e / 2))^2. 19 FP32 instructions and 2 transcendentals; against x Phi(x) in double the
+// relative error stays below 4e-6 for |x| < 6 and 1.5e-5 down to x = -12.
 __device__ __forceinline__ float gelu_erf(float x) {
-    const float z = fabsf(x) * 0.70710678118654752f;
-    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.5f, z, 1.f));
-    float q = 0.17087277f;
-    q = __builtin_fmaf(q, t, -0.82215223f);
-    q = __builtin_fmaf(q, t, 1.48851587f);
-    q = __builtin_fmaf(q, t, -1.13520398f);
-    q = __builtin_fmaf(q, t, 0.27886807f);
-    q = __builtin_fmaf(q, t, -0.18628806f);
-    q = __builtin_fmaf(q, t, 0.09678418f);
-    q = __builtin_fmaf(q, t, 0.37409196f);
-    q = __builtin_fmaf(q, t, 1.00002368f);
-    q = __builtin_fmaf(q, t, -1.26551223f);
-    const float e = t * __builtin_amdgcn_exp2f(__builtin_fmaf(-z, z, q) * 1.4426950408889634f);
-    return 0.5f * x * (x < 0.f ? e : 2.f - e);
+    const float ax = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(ax, 0.35355339059327373f, 1.f));
+    const float zs = ax * 0.849321800288f;
+    float q = 0.246517298f;
+    q = __builtin_fmaf(q, t, -1.18611495f);
+    q = __builtin_fmaf(q, t, 2.14747446f);
+    q = __builtin_fmaf(q, t, -1.63775315f);
+    q = __builtin_fmaf(q, t, 0.402321582f);
+    q = __builtin_fmaf(q, t, -0.26875686f);
+    q = __builtin_fmaf(q, t, 0.139630057f);
+    q = __builtin_fmaf(q, t, 0.539700616f);
+    q = __builtin_fmaf(q, t, 1.4427292f);
+    q = __builtin_fmaf(q, t, -2.82574822f);
+    const float half_erfc = t * __builtin_amdgcn_exp2f(__builtin_fmaf(-zs, zs, q));
+    return x * (x < 0.f ? half_erfc : 1.f - half_erfc);
 }
 
 // What the two kernels below share: the MFMA step and the epilogue of a BM x BN tile held by WM x WN wavefronts. GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
@@ -498,10 +502,11 @@ int launch_ring(const LinearBatch& batch, int n_problems, hipStream_t st) {
 template <typename T>
 int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool geglu) {
     if (geglu) {
-        // the ring form when its 256-token tiles give every compute unit one: FF1 of the U-Net's widest level
-        // (8192 x 320 -> 2 x 1280: 33 us against 40 for the streaming form)
-        if (ring_form_takes(batch, 1, true) && static_cast<long>((batch.p[0].M + 255) / 256) * ((batch.p[0].N + 63) / 64) >= device_cu_count())
-            return launch_ring<T, 256, 128, true, 4, 2>(batch, 1, st);
+        // the ring form when its 128-token tiles give every compute unit two: FF1 of the U-Net's widest levels
+        // (8192 x 320 -> 2 x 1280: 31 us against 40 for the streaming form, 33 with 256-token tiles, whose 640 tiles are
+        // 2.5 per compute unit; 2048 x 640 -> 2 x 2560: 28 against 33)
+        if (ring_form_takes(batch, 1, true) && static_cast<long>((batch.p[0].M + 127) / 128) * ((batch.p[0].N + 63) / 64) >= 2L * device_cu_count())
+            return launch_ring<T, 128, 128, true, 4, 2>(batch, 1, st);
         // 64-token tiles unless 128-token tiles alone fill the GPU twice over
         const long big = static_cast<long>((batch.p[0].M + 127) / 128) * ((batch.p[0].N + 63) / 64);
         if (big >= 2L * device_cu_count() && batch.p[0].K >= 1024) return launch_tiles<T, 128, 128, true>(batch, 1, st);
@@ -521,7 +526,12 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool gegl
         return w8 ? launch_tiles<T, 128, 128, false, true>(batch, n_problems, st) : launch_tiles<T, 128, 128>(batch, n_problems, st);
     // long contractions over few tiles (FF2 of the U-Net: 2048 x 2560 -> 640, 30 -> 21 us; 8192 x 1280 -> 320, 22 -> 17 us): the
     // ring form, whose five steps in flight shorten the per-step chain of memory latencies; at 320 it measures the same
-    if (min_k >= 2 * kRing * kBK && ring_form_takes(batch, n_problems, false)) return launch_ring<T, 64, 64>(batch, n_problems, st);
+    // (with many tiles per compute unit the streaming form's work groups cover for each other: 2048 x 640 -> 5120, 2560
+    // tiles, 28 us against 34)
+    long tiles64 = 0;
+    for (int i = 0; i < n_problems; ++i) tiles64 += static_cast<long>((batch.p[i].M + 63) / 64) * ((batch.p[i].N + 63) / 64);
+    if (min_k >= 2 * kRing * kBK && tiles64 <= 4L * device_cu_count() && ring_form_takes(batch, n_problems, false))
+        return launch_ring<T, 64, 64>(batch, n_problems, st);
     return w8 ? launch_tiles<T, 64, 64, false, true>(batch, n_problems, st) : launch_tiles<T, 64, 64>(batch, n_problems, st);
 }
 
