@@ -42,6 +42,13 @@ def test_graph_replays_equal_eager():
     # a linear layer large enough for the 256 x 256-tile kernel
     xl, wl, bl = rnd(4608, 1024), rnd(3072, 1024) / 32, rnd(3072)
     o_big = torch.empty(4608, 3072, dtype=torch.bfloat16, device=dev)
+    # the tile-walking GEMM forms: FF1 + GEGLU with 128-token tiles (at least two per compute unit) and a long contraction
+    # over few tiles (FF2)
+    xr = rnd(4096, C, dt=torch.float16)
+    wr, br = rnd(2 * 1280, C, dt=torch.float16) / C ** 0.5, rnd(2 * 1280, dt=torch.float16)
+    o_ring = torch.empty(4096, 1280, dtype=torch.float16, device=dev)
+    x2, w2, b2 = rnd(512, 1280, dt=torch.float16), rnd(640, 1280, dt=torch.float16) / 36, rnd(640, dt=torch.float16)
+    o_ff2 = torch.empty(512, 640, dtype=torch.float16, device=dev)
 
     def step():
         bd.joint_attention(q, k, v, cos, sin, d, H, out=o_joint, Kr=kr)
@@ -52,15 +59,17 @@ def test_graph_replays_equal_eager():
         bd.add_inplace_vec(o_blk, x)
         bd.headnorm_rope(k, gain, 1e-6, cos, sin, d, H, out=o_hn)
         bd.linear_batched(wl, bl, xl, o_big)
+        bd.fused_linear_geglu(xr, wr, br, o_ring)
+        bd.linear_batched(w2, b2, x2, o_ff2)
 
-    outs = (o_joint, o_block, o_lin, o_blk, o_ff, o_hn, o_big, ws)
+    outs = (o_joint, o_block, o_lin, o_blk, o_ff, o_hn, o_big, o_ring, o_ff2, ws)
     step()                                            # warm-up outside the capture (first-use set-up of the library)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
     for it in range(4):
-        for t in (q, k, v, lq, lk, lv, x, xl):
+        for t in (q, k, v, lq, lk, lv, x, xl, xr, x2):
             t.copy_(rnd(*t.shape, dt=t.dtype))        # eager work between the replays: new input values
         step()
         torch.cuda.synchronize()
@@ -70,5 +79,5 @@ def test_graph_replays_equal_eager():
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
-        for name, a, b in zip(("joint", "block-causal", "linear attention", "attention block", "geglu", "headnorm", "large linear", "state"), eager, outs):
+        for name, a, b in zip(("joint", "block-causal", "linear attention", "attention block", "geglu", "headnorm", "large linear", "geglu, walked tiles", "ff2, walked tiles", "state"), eager, outs):
             assert torch.equal(a, b), f"replay {it}: {name} differs from the eager call"
