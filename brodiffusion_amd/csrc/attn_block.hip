@@ -92,11 +92,10 @@ int mi_linear_geglu_forward(const mi_linear_args* a) {
     if (a->struct_size != sizeof(mi_linear_args))
         return fail("mi_linear_geglu_forward: struct_size %u != %zu (header mismatch)", a->struct_size, sizeof(mi_linear_args));
     if (a->rows < 0) return fail("mi_linear_geglu_forward: negative rows");
-    if (a->w_scales) return fail("mi_linear_geglu_forward: there is no INT8-weight form (the reference does not fuse it either)");
     if (a->rows == 0) return 0;
     mi::LinearBatch b;
     std::memset(&b, 0, sizeof(b));
-    b.p[0] = mi::problem(a->x, a->w, a->bias, a->y, a->rows, a->out_features, a->in_features);
+    b.p[0] = mi::problem(a->x, a->w, a->bias, a->y, a->rows, a->out_features, a->in_features, a->w_scales);
     if (a->x_row_stride) b.p[0].ldx = a->x_row_stride;
     if (a->w_row_stride) b.p[0].ldw = a->w_row_stride;
     if (a->y_row_stride) b.p[0].ldy = a->y_row_stride;

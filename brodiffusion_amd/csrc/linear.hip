@@ -70,14 +70,16 @@ __device__ __forceinline__ void load_tile(u32x4 (&r)[ROWS / 32], const char* bas
 }
 // INT8 weight tile: the same 8 contraction elements per thread and row are 8 bytes in memory; they are widened to T
 // (exactly: |w| <= 128) on their way to LDS, the per-row scale is applied to the accumulator in the epilogue.
-template <int ROWS>
+template <int ROWS, bool GATED = false>
 __device__ __forceinline__ void load_tile_int8(u32x2 (&raw)[ROWS / 32], const char* base, long ld, int row0, int n_rows,
                                                int k0, int K, int tid) {
     const int kc = k0 + (tid & 7) * 8;
     const long col = kc < K ? kc : 0;
 #pragma unroll
     for (int i = 0; i < ROWS / 32; ++i) {
-        const int row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);
+        int row;
+        if constexpr (GATED) row = min(row0 + (tid >> 3) + 32 * (i >> 1), n_rows - 1) + (i & 1) * n_rows;   // as in load_tile
+        else row = min(row0 + (tid >> 3) + 32 * i, n_rows - 1);
         raw[i] = *reinterpret_cast<const u32x2*>(base + static_cast<long>(row) * ld + col);
     }
 }
@@ -132,11 +134,25 @@ __device__ __forceinline__ float gelu_erf(float x) {
     return x * (x < 0.f ? half_erfc : 1.f - half_erfc);
 }
 
+// acc * scale + bias of the INT8-weight forms as an FP32 value of its own. Left to itself the compiler merges the
+// multiply-add with the rounding to T that follows (v_fma_mixlo_f16: one rounding of the exact result) in some places and
+// not in others, and the plain and the GEGLU form of the same layer then disagree by a unit in the last place in about 3
+// outputs of 100 000; as a separate FP32 operation it is the FP32 multiply-add and conversion of the reference's kernel
+// everywhere.
+__device__ __forceinline__ float scaled_acc(float acc, float scale, float bias) {
+    float r = __builtin_fmaf(acc, scale, bias);
+    asm volatile("" : "+v"(r));
+    return r;
+}
+
 // What the two kernels below share: the MFMA step and the epilogue of a BM x BN tile held by WM x WN wavefronts. GEGLU: W is (2 N, K) and bias (2 N): value half on top, gate half below; the output (M, N) is
 // value * gelu_exact(gate) (diffusers' GEGLU with the erf form of GELU). A work group's 128 W-tile rows are 64 output
 // features times {value, gate}; each wavefront holds both accumulators of its 32 features, so the product of the two
 // halves never leaves registers and the (M, 2 N) intermediate does not exist.
 // W8: W is INT8 (N, K) with one FP32 scale per row (LinearProblem::w_scale): Y = (X Wq^T) * scale + bias.
+// GEGLU with W8 (2 N scales): the reference composes this one from its INT8-weight linear layer and a GEGLU pass over a
+// 16-bit (M, 2 N) buffer (src/fused_transformer.cu:360-396); here the two halves are rounded to T at the same point,
+// in registers, so the result is the composition's without the buffer.
 template <typename T, int BM, int BN, bool GEGLU, bool W8, int WM = 2, int WN = 2>
 struct TileMath {
     using M = Mma<T>;
@@ -144,7 +160,6 @@ struct TileMath {
     static constexpr int NT = 64 * WM * WN;                       // threads: WM x WN wavefronts over tokens x features
     static constexpr int TM = BM / (32 * WM), TN = BN / (32 * WN);  // 32 x 32 blocks per wavefront along tokens / features
     static_assert(!GEGLU || TN == 2, "the GEGLU form pairs the two feature blocks of a wavefront");
-    static_assert(!(GEGLU && W8), "no INT8-weight GEGLU form");
     static constexpr int BN_OUT = GEGLU ? BN / 2 : BN;   // output features per tile
     static constexpr int X_BYTES = BM * kRowBytes, W_BYTES = BN * kRowBytes;
     static constexpr int kOutRow = BN_OUT * 2 + 16;      // staged output row (bytes)
@@ -212,13 +227,26 @@ struct TileMath {
                 float bv[4], bg[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) { bv[i] = static_cast<float>(braw[0][g][i]); bg[i] = static_cast<float>(braw[1][g][i]); }
+                float sv[4] = {1.f, 1.f, 1.f, 1.f}, sg[4] = {1.f, 1.f, 1.f, 1.f};
+                if constexpr (W8) {
+                    if (n0 + feat < p.N) {   // N is a multiple of 8, so the 4 features are in or out together
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { sv[i] = p.w_scale[n0 + feat + i]; sg[i] = p.w_scale[p.N + n0 + feat + i]; }
+                    }
+                }
 #pragma unroll
                 for (int b = 0; b < TM; ++b) {
                     V4 o;
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const float val = acc[0][b][4 * g + i] + bv[i];
-                        const float gate = acc[1][b][4 * g + i] + bg[i];
+                        float val, gate;
+                        if constexpr (W8) {
+                            val = static_cast<float>(static_cast<T>(scaled_acc(acc[0][b][4 * g + i], sv[i], bv[i])));
+                            gate = static_cast<float>(static_cast<T>(scaled_acc(acc[1][b][4 * g + i], sg[i], bg[i])));
+                        } else {
+                            val = acc[0][b][4 * g + i] + bv[i];
+                            gate = acc[1][b][4 * g + i] + bg[i];
+                        }
                         o[i] = static_cast<T>(val * gelu_erf(gate));
                     }
                     *reinterpret_cast<V4*>(stage + ((wm * TM + b) * 32 + lq) * kOutRow + feat * 2) = o;
@@ -245,7 +273,7 @@ struct TileMath {
                         V4 o;
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            if constexpr (W8) o[i] = static_cast<T>(__builtin_fmaf(acc[a][b][4 * g + i], sc[i], bv[i]));
+                            if constexpr (W8) o[i] = static_cast<T>(scaled_acc(acc[a][b][4 * g + i], sc[i], bv[i]));
                             else o[i] = static_cast<T>(acc[a][b][4 * g + i] + bv[i]);
                         }
                         *reinterpret_cast<V4*>(stage + ((wm * TM + b) * 32 + lq) * kOutRow + feat * 2) = o;
@@ -299,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void linear_kernel(const LinearBatch batc
     u32x2 wr8[W8 ? BN / 32 : 1];
     auto load_tiles = [&](int k0) {
         load_tile<BM>(xr, xg, p.ldx, m0, p.M, k0, p.K, tid);
-        if constexpr (W8) load_tile_int8<BN>(wr8, wg, p.ldw, n0, p.N, k0, p.K, tid);
+        if constexpr (W8) load_tile_int8<BN, GEGLU>(wr8, wg, p.ldw, n0, p.N, k0, p.K, tid);
         else load_tile<BN, GEGLU>(wr, wg, p.ldw, n0, p.N, k0, p.K, tid);
     };
     auto store_tiles = [&](char* dst, int k0) {
@@ -509,8 +537,10 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st, bool gegl
             return launch_ring<T, 128, 128, true, 4, 2>(batch, 1, st);
         // 64-token tiles unless 128-token tiles alone fill the GPU twice over
         const long big = static_cast<long>((batch.p[0].M + 127) / 128) * ((batch.p[0].N + 63) / 64);
-        if (big >= 2L * device_cu_count() && batch.p[0].K >= 1024) return launch_tiles<T, 128, 128, true>(batch, 1, st);
-        return launch_tiles<T, 64, 128, true>(batch, 1, st);
+        const bool w8g = batch.p[0].w_scale != nullptr;
+        if (big >= 2L * device_cu_count() && batch.p[0].K >= 1024)
+            return w8g ? launch_tiles<T, 128, 128, true, true>(batch, 1, st) : launch_tiles<T, 128, 128, true>(batch, 1, st);
+        return w8g ? launch_tiles<T, 64, 128, true, true>(batch, 1, st) : launch_tiles<T, 64, 128, true>(batch, 1, st);
     }
     // 128 x 128 tiles when they alone fill the GPU twice over and the contraction is long enough to pay for their
     // longer prologue, else 64 x 64 (more, smaller work groups: the projections of one attention block are small
@@ -545,7 +575,6 @@ int launch_linear(const LinearBatch& batch, int n_problems, int dtype, hipStream
         if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail("linear: empty problem %d (%d x %d x %d)", i, p.M, p.N, p.K);
         if (p.N % 8 || p.K % 8) return fail("linear: in_features %d and out_features %d must be multiples of 8", p.K, p.N);
         if ((p.w_scale != nullptr) != (batch.p[0].w_scale != nullptr)) return fail("linear: INT8 and 16-bit weights cannot share a launch");
-        if (p.w_scale && geglu) return fail("linear: there is no INT8-weight GEGLU form");
         if (reinterpret_cast<uintptr_t>(p.w_scale) & 3u) return fail("linear: weight scales must be 4-byte aligned");
         if (p.ldx % 8 || p.ldw % 8 || p.ldy % 8) return fail("linear: row strides must be multiples of 8 elements");
         if (p.ldx < p.K || p.ldw < p.K || p.ldy < p.N) return fail("linear: a row stride is smaller than the row");

@@ -397,10 +397,18 @@ void mha_forward(const Tensor& X, const Tensor& Wq, const Tensor& Wk, const Tens
 
 }  // namespace bt
 
-void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y) {
-    const char* op = "fused_linear_geglu";
+namespace {
+void geglu_impl(const char* op, const Tensor& X, const Tensor& W, const Tensor* scales, const Tensor& b, Tensor& Y) {
     need_gpu(op, X); need_gpu(op, W); need_gpu(op, b);
-    if (W.rows % 2 != 0 || W.cols != X.cols || W.dtype != X.dtype) fail(std::string(op) + ": W must be (2*D_out, D_in) of X's dtype");
+    if (scales) need_gpu(op, *scales);
+    if (W.rows % 2 != 0 || W.cols != X.cols) fail(std::string(op) + ": W must be (2*D_out, D_in)");
+    if (scales) {
+        if (W.dtype != Dtype::INT8) fail(std::string(op) + ": W_int8 must be INT8");
+        if (scales->dtype != Dtype::FP32 || scales->size() != static_cast<std::size_t>(W.rows))
+            fail(std::string(op) + ": W_scales must hold one FP32 value per row of W");
+    } else if (W.dtype != X.dtype) {
+        fail(std::string(op) + ": W must have X's dtype");
+    }
     const int d_out = W.rows / 2;
     if (b.dtype != X.dtype || b.size() != static_cast<std::size_t>(W.rows)) fail(std::string(op) + ": b must hold 2*D_out values of X's dtype");
     if (Y.data == nullptr || Y.rows != X.rows || Y.cols != d_out || Y.dtype != X.dtype) Y.resize(X.rows, d_out, X.dtype, X.device);
@@ -409,8 +417,15 @@ void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tenso
     a.struct_size = sizeof(a);
     a.dtype = dtype_code(op, X.dtype);
     a.x = X.data; a.w = W.data; a.bias = b.data; a.y = Y.data;
+    a.w_scales = scales ? static_cast<const float*>(scales->data) : nullptr;
     a.rows = X.rows; a.in_features = X.cols; a.out_features = d_out;
     check(op, mi_linear_geglu_forward(&a));
+}
+}  // namespace
+
+void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y) { geglu_impl("fused_linear_geglu", X, W, nullptr, b, Y); }
+void fused_linear_geglu(const Tensor& X, const Tensor& W_int8, const Tensor& W_scales, const Tensor& b, Tensor& Y) {
+    geglu_impl("fused_linear_geglu(int8w)", X, W_int8, &W_scales, b, Y);
 }
 
 void add_inplace_vec(Tensor& Y, const Tensor& X) {

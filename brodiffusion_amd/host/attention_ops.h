@@ -108,6 +108,9 @@ void mha_forward(const Tensor& X, const Tensor& Wq, const Tensor& Wk, const Tens
 //   add_inplace_vec      Y += X, same shape                                                                        (:50-53)
 //   add_inplace_row_bias Y[i][j] += bias[j], bias holds Y.cols values in any shape                                  (:55-61)
 void fused_linear_geglu(const Tensor& X, const Tensor& W, const Tensor& b, Tensor& Y);
+// ... and its W8A16 overload (:37-48): W_int8 (2*D_out, D_in) INT8, W_scales (2*D_out, 1) FP32. One GEMM; the two halves are
+// rounded to the tensor dtype where the reference's 16-bit (B, 2*D_out) buffer rounds them (src/fused_transformer.cu:360-396).
+void fused_linear_geglu(const Tensor& X, const Tensor& W_int8, const Tensor& W_scales, const Tensor& b, Tensor& Y);
 void add_inplace_vec(Tensor& Y, const Tensor& X);
 void add_inplace_row_bias(Tensor& Y, const Tensor& bias);
 

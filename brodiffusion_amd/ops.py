@@ -377,15 +377,16 @@ def linear_forward_batched_int8w_fp16(W_int8, scales, bias, X, Y: Optional[torch
     return linear_batched(W_int8, bias, X, Y, W_scales=scales, op="linear_forward_batched_int8w_fp16")
 
 
-def fused_linear_geglu(X, W, b, Y: Optional[torch.Tensor] = None):
+def fused_linear_geglu(X, W, b, Y: Optional[torch.Tensor] = None, W_scales: Optional[torch.Tensor] = None,
+                       op: str = "fused_linear_geglu"):
     """Y = a * gelu_exact(g), [a | g] = X W^T + b with W (2*D_out, D_in), b (2*D_out): the fused FF1 + GEGLU of the
-    U-Net transformer block (brodiffusion::fused_linear_geglu, include/brodiffusion/fused_transformer.h:20-35)."""
-    op = "fused_linear_geglu"
-    _dev(op, X, W, b, Y)
+    U-Net transformer block (brodiffusion::fused_linear_geglu, include/brodiffusion/fused_transformer.h:20-35). With
+    W_scales, W is INT8 with one FP32 scale per row (see fused_linear_geglu_int8w)."""
+    _dev(op, X, W, b, Y, W_scales)
     if W.dim() != 2 or W.shape[0] % 2 != 0 or X.shape[-1] != W.shape[1]:
         _fail(op, f"W must be (2*D_out, D_in) with D_in = {X.shape[-1]}, got {tuple(W.shape)}")
     d_out = W.shape[0] // 2
-    _mat(op, W, "W", X.dtype)
+    scales_ptr = _weight(op, W, W_scales, "W", X.dtype)
     _mat(op, X, "X", X.dtype)
     rows = X.numel() // X.shape[-1]
     if Y is None:
@@ -398,10 +399,19 @@ def fused_linear_geglu(X, W, b, Y: Optional[torch.Tensor] = None):
     a.dtype = _dtype_code(op, X)
     a.x, a.w, a.y = X.data_ptr(), W.data_ptr(), Y.data_ptr()
     a.bias = _bias(op, b, "b", X.dtype, W.shape[0])
+    a.w_scales = scales_ptr
     a.rows, a.in_features, a.out_features = rows, W.shape[1], d_out
     a.stream = _stream()
     capi.check(capi.lib().mi_linear_geglu_forward(C.byref(a)), op)
     return Y
+
+
+def fused_linear_geglu_int8w(X, W_int8, W_scales, b, Y: Optional[torch.Tensor] = None):
+    """The W8A16 overload of brodiffusion::fused_linear_geglu (include/brodiffusion/fused_transformer.h:37-48): W_int8
+    (2*D_out, D_in) INT8, W_scales (2*D_out, 1) FP32, b (2*D_out) of X's dtype. The reference runs its INT8-weight linear
+    layer into a 16-bit (B, 2*D_out) buffer and a GEGLU pass over it (src/fused_transformer.cu:360-396); this is one
+    GEMM that rounds the two halves where the buffer would."""
+    return fused_linear_geglu(X, W_int8, b, Y, W_scales=W_scales, op="fused_linear_geglu_int8w")
 
 
 def add_inplace_vec(Y, X):

@@ -373,7 +373,10 @@ MI_API int mi_linear_forward(const mi_linear_args* args);
  * (2*out_features): value half first, gate half second; gelu_exact(g) = 0.5 g (1 + erf(g / sqrt 2)). The fused FF1 +
  * GEGLU of the U-Net transformer block, brodiffusion::fused_linear_geglu (include/brodiffusion/fused_transformer.h:20-35,
  * src/fused_transformer.cu:56-68): the (rows, 2*out_features) intermediate never reaches memory. Same struct as
- * mi_linear_forward. */
+ * mi_linear_forward. With w_scales (2*out_features values) W is INT8: the W8A16 overload of the same operator
+ * (fused_transformer.h:37-48), which the reference composes from bt::linear_forward_batched_int8w_fp16 into a 16-bit
+ * (rows, 2*out_features) buffer and bt::geglu_exact_forward (src/fused_transformer.cu:360-396); here both halves are
+ * rounded to the tensor dtype where that buffer would round them, in registers, and the buffer does not exist. */
 MI_API int mi_linear_geglu_forward(const mi_linear_args* args);
 /* Y[i] += X[i] over n_elements of flat storage (brodiffusion::add_inplace_vec, fused_transformer.h:50-53) and
  * Y[r][c] += bias[c] (brodiffusion::add_inplace_row_bias, fused_transformer.h:55-61). Any element count; 16-byte

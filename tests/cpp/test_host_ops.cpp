@@ -470,6 +470,28 @@ static void gpu_checks() {
         const Err e = compare(ref, download_bf16(Y));
         std::printf("fused_linear_geglu    rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(Y.rows == B && Y.cols == d_out && e.rel_l2 <= 5e-3);
+        {   // the W8A16 overload: the reference's composition (INT8-weight linear into a 16-bit buffer, then GEGLU) from the
+            // checker fed the dequantised weight, the buffer rounded to bf16
+            std::vector<float> r(static_cast<size_t>(2) * d_out * d_in), deq(r.size()), sc(2 * d_out);
+            std::vector<int8_t> q8(r.size());
+            orc_torch_randn_f32(7408, r.size(), r.data());
+            for (int i = 0; i < 2 * d_out; ++i) sc[i] = (0.75f + 0.5f * static_cast<float>(i % 7) / 7.0f) / (42.0f * std::sqrt(static_cast<float>(d_in)));
+            for (size_t i = 0; i < r.size(); ++i) {
+                const float v = std::fmax(-127.f, std::fmin(127.f, std::nearbyint(r[i] * 42.0f)));
+                q8[i] = static_cast<int8_t>(v);
+                deq[i] = v * sc[i / d_in];
+            }
+            Tensor W8 = Tensor::from_host(q8.data(), 2 * d_out, d_in, Dtype::INT8), S8 = Tensor::from_host(sc.data(), 2 * d_out, 1, Dtype::FP32), Y8;
+            fused_linear_geglu(X, W8, S8, Bv, Y8);
+            std::vector<float> t8(static_cast<size_t>(B) * 2 * d_out), ref8(static_cast<size_t>(B) * d_out);
+            orc_linear(x.data(), deq.data(), b.data(), B, 2 * d_out, d_in, t8.data(), 0);
+            orc_round_bf16(t8.data(), t8.size());
+            orc_geglu_exact(t8.data(), B, d_out, ref8.data());
+            const Err e8 = compare(ref8, download_bf16(Y8));
+            std::printf("fused_linear_geglu i8 rel_l2=%.3e max_abs=%.3e\n", e8.rel_l2, e8.max_abs);
+            CHECK(Y8.rows == B && Y8.cols == d_out && e8.rel_l2 <= 5e-3);
+            CHECK(throws_with([&] { fused_linear_geglu(X, W, S8, Bv, Y8); }, "must be INT8"));
+        }
         // Y += X on 10 x 37 and Y += row bias on 13 x 29: exact (one FP32 add, one rounding)
         std::vector<float> y0 = randn_bf16(7404, 370), xa = randn_bf16(7405, 370), want(370);
         for (int i = 0; i < 370; ++i) want[i] = y0[i] + xa[i];

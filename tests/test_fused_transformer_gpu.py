@@ -52,6 +52,38 @@ def test_fused_linear_geglu_without_bias(oracle, B, d_in, d_out):
     assert np.all(err <= 2.0 ** -8 * np.maximum(np.abs(ref), 2.0 ** -6) * 1.05 + 2e-6)
 
 
+def _quantised(seed, n_out, n_in):
+    rng = np.random.default_rng(seed)
+    q = rng.integers(-127, 128, (n_out, n_in)).astype(np.int8)
+    scales = (rng.uniform(0.5, 1.5, n_out) / (73.0 * np.sqrt(n_in))).astype(np.float32)     # rows of unit-variance weights
+    return q, scales, q.astype(np.float32) * scales[:, None]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("B,d_in,d_out", [(40, 64, 48), (8192, 320, 1280), (300, 1280, 5120), (1000, 328, 72)])
+def test_fused_linear_geglu_int8w(oracle, dtype, B, d_in, d_out):
+    """The W8A16 overload (include/brodiffusion/fused_transformer.h:37-48). The reference composes it from its INT8-weight
+    linear layer into a 16-bit (B, 2*D_out) buffer and a GEGLU pass over that buffer (src/fused_transformer.cu:360-396);
+    the single GEMM here rounds the two halves where the buffer would, so it must agree with that composition run on the
+    device (the linear layer's output, then the checker's GEGLU) to the final rounding, and with the checker end to end."""
+    x = uniform(41, (B, d_in), 1.0, dtype, oracle)
+    q, scales, w = _quantised(42 + d_out, 2 * d_out, d_in)
+    b = uniform(43, (2 * d_out,), 0.2, dtype, oracle)
+    dx, db = to_dev(x, dtype), to_dev(b, dtype)
+    dq, ds = torch.from_numpy(q).cuda(), torch.from_numpy(scales).cuda()
+    y = to_np(bd.fused_linear_geglu_int8w(dx, dq, ds, db))
+    assert y.shape == (B, d_out)
+    unit = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    composed = oracle.geglu_exact(to_np(bd.linear_forward_batched_int8w_fp16(dq, ds, db, dx)))
+    assert np.all(np.abs(y - composed) <= unit * np.maximum(np.abs(composed), 2.0 ** -6) * 1.05 + 2e-6)
+    ref = oracle.geglu_exact(oracle.round_to(oracle.linear(x, w, b), dtype))
+    assert np.abs(y - ref).max() <= 0.008 + 0.01 * np.abs(ref).max()        # the reference's bound for the 16-bit form
+    with pytest.raises(RuntimeError, match="scales must hold"):
+        bd.fused_linear_geglu_int8w(dx, dq, ds[:-1], db)
+    with pytest.raises(RuntimeError, match="int8"):
+        bd.fused_linear_geglu_int8w(dx, dq.to(torch.int16), ds, db)
+
+
 def test_geglu_gate_tails(oracle):
     """gelu_exact over the whole range of the gate, one gate value per output column: a zero weight and the gate's value as
     its bias, value half = 1. The left tail keeps its relative accuracy (x Phi(x) down to the smallest normal numbers of
