@@ -526,19 +526,19 @@ int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st)
                                accumulate ? 1 : 0, p.old_weight);
         }
     }
-    // Apply pass: chunks are multiples of the tile; two resident work groups per CU hide each other's latencies, beyond
-    // that larger chunks keep the staging of S small against the streamed tokens.
-    auto pick = [&](int tile, int min_tiles) {
-        int t = tile * min_tiles;
-        while (t < p.N && static_cast<long>(BH) * ((p.N + 2 * t - 1) / (2 * t)) >= 2L * n_cu) t *= 2;
-        return t;
-    };
+    // Apply pass: chunks are whole tiles, and as few of them per group as keep every group resident at once (two work
+    // groups per CU hide each other's latencies): the staging of S is paid once per group, and a second, partly filled round of
+    // groups would pay it again (N = 4096, 40 heads: 440 groups of 3 tiles instead of 640 of 2, 45.6 -> 43.4 us for the call).
     auto grid_of = [&](LinDev& q) {
         q.n_chunks = (q.N + q.tokens_per_group - 1) / q.tokens_per_group;
         q.n_blocks = BH * q.n_chunks;
         return dim3(((q.n_blocks + 7) / 8) * 8);
     };
-    p.tokens_per_group = pick(128, 1);
+    {
+        const int tiles = (p.N + 127) / 128;
+        const int per_bh = std::max(1, 2 * n_cu / BH);
+        p.tokens_per_group = 128 * ((tiles + per_bh - 1) / per_bh);
+    }
     hipLaunchKernelGGL((linattn_apply_kernel<T, D>), grid_of(p), dim3(kThreads), 0, st, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail("mi_linear_attn_relu_forward launch: %s", hipGetErrorString(e));
