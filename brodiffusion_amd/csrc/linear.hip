@@ -477,15 +477,17 @@ int launch_tiles(const LinearBatch& batch, int n_problems, hipStream_t st) {
     }
     constexpr size_t lds = 2 * static_cast<size_t>(BM + BN) * kRowBytes;
     static_assert(lds <= 160 * 1024, "operand ring exceeds the LDS of a compute unit");
-    auto kern = linear_kernel<T, BM, BN, GEGLU, W8>;
+    // (launched by name: a launch through a pointer variable is dropped by this compiler when the host code is built with
+    // -fsanitize=undefined)
+    const void* const kern = reinterpret_cast<const void*>(&linear_kernel<T, BM, BN, GEGLU, W8>);
     if (lds > 64 * 1024) {
         static thread_local bool raised = false;
         if (!raised) {
-            MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            MI_HIP_CHECK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
             raised = true;
         }
     }
-    hipLaunchKernelGGL(kern, dim3(max_tiles, n_problems), dim3(kThreads), lds, st, batch);
+    hipLaunchKernelGGL((linear_kernel<T, BM, BN, GEGLU, W8>), dim3(max_tiles, n_problems), dim3(kThreads), lds, st, batch);
     MI_HIP_CHECK(hipGetLastError());
     return 0;
 }
@@ -511,18 +513,18 @@ int launch_ring(const LinearBatch& batch, int n_problems, hipStream_t st) {
     }
     constexpr size_t lds = 2 * static_cast<size_t>(BM + BN) * kRowBytes + TM_::kOutBytes;
     static_assert(lds <= 160 * 1024, "operand buffers and staged output exceed the LDS of a compute unit");
-    auto kern = linear_ring_kernel<T, BM, BN, GEGLU, WM, WN>;
+    const void* const kern = reinterpret_cast<const void*>(&linear_ring_kernel<T, BM, BN, GEGLU, WM, WN>);
     static thread_local int per_cu = 0;   // work groups a compute unit holds at once
     if (per_cu == 0) {
         if (lds > 64 * 1024)
-            MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+            MI_HIP_CHECK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         int n = 0;
-        MI_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void*>(kern), TM_::NT, lds));
+        MI_HIP_CHECK(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, TM_::NT, lds));
         per_cu = max(n, 1);
     }
     // as many work groups as the GPU holds at once, split over the problems; a multiple of 8 (one run of tiles per XCD)
     const int grid_x = min((max_tiles + 7) / 8 * 8, max(8, per_cu * device_cu_count() / n_problems / 8 * 8));
-    hipLaunchKernelGGL(kern, dim3(grid_x, n_problems), dim3(TM_::NT), lds, st, batch);
+    hipLaunchKernelGGL((linear_ring_kernel<T, BM, BN, GEGLU, WM, WN>), dim3(grid_x, n_problems), dim3(TM_::NT), lds, st, batch);
     MI_HIP_CHECK(hipGetLastError());
     return 0;
 }

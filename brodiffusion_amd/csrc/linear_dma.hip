@@ -244,13 +244,12 @@ int launch_t(const LinearBatch& batch, int n_problems, hipStream_t st) {
         const LinearProblem& p = batch.p[i];
         max_tiles = max(max_tiles, ((p.M + kTile - 1) / kTile) * ((p.N + kTile - 1) / kTile));
     }
-    auto kern = linear_dma_kernel<T>;
     static thread_local bool raised = false;
     if (!raised) {
-        MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
+        MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_dma_kernel<T>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3(((max_tiles + 7) / 8) * 8, n_problems), dim3(kThreads), kLdsBytes, st, batch);
+    hipLaunchKernelGGL((linear_dma_kernel<T>), dim3(((max_tiles + 7) / 8) * 8, n_problems), dim3(kThreads), kLdsBytes, st, batch);
     MI_HIP_CHECK(hipGetLastError());
     return 0;
 }
