@@ -73,6 +73,35 @@ def event_ms(torch, fn, iters, warm=0.05):
     return min(ts), sum(ts) / len(ts)
 
 
+def graph_ms(torch, fn, calls=20, reps=5):
+    """Per-call milliseconds of `fn` as the GPU sees it: `calls` calls captured into one HIP graph, the replay timed with
+    events (min over `reps` replays). For calls of a few microseconds the event timing above measures how fast Python
+    submits them, not how long the GPU takes. None if the call cannot be captured."""
+    try:
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(calls):
+                fn()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            g.replay()
+            b.record()
+            torch.cuda.synchronize()
+            t = a.elapsed_time(b) / calls
+            best = t if best is None else min(best, t)
+        return round(best, 4)
+    except Exception as e:   # a failed capture must not take the benchmark line with it
+        sys.stderr.write("graph timing skipped: %s\n" % e)
+        return None
+
+
 def seeded(torch, seed, shape, dtype):
     """N(0,1) values of torch's CPU generator for `seed` (what torch_randn_f32(seed, n) of the reference's torch_rng.h
     reproduces), rounded once to `dtype`, on the GPU."""
@@ -111,7 +140,7 @@ def all_configs(torch, bd, cin, keep):
         mn, av = event_ms(torch, fn, 20)
         out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "tflops": round(flops / (mn * 1e-3) / 1e12, 1),
                      "frac_mfma_peak": round(flops / (mn * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, 4), "dtype": dtype,
-                     "gflop": round(flops / 1e9, 2)}
+                     "gflop": round(flops / 1e9, 2), "ms_graph": graph_ms(torch, fn)}
 
     q, k, v = cin["cfg1"]
     o1 = torch.empty_like(q)
@@ -168,11 +197,12 @@ def all_configs(torch, bd, cin, keep):
     out["cfg4_qwen_blockcausal_prefixkv_d128_bf16"]["dense_equivalent_gflop"] = round(4 * 24 * 4096 * 4608 * 128 / 1e9, 2)
     xh, gh = rnd(4608, 3072), rnd(128)
     oh = torch.empty_like(xh)
-    mn, av = event_ms(torch, lambda: bd.headnorm_rope(xh, gh, 1e-6, cos, sin, 128, 24, out=oh), 20)
+    hn = lambda: bd.headnorm_rope(xh, gh, 1e-6, cos, sin, 128, 24, out=oh)   # noqa: E731
+    mn, av = event_ms(torch, hn, 20)
     nbytes = 2 * xh.numel() * 2
     out["headnorm_rope_4608x24x128_bf16"] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
                                              "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4), "dtype": "bf16",
-                                             "mbytes": round(nbytes / 1e6, 2)}
+                                             "mbytes": round(nbytes / 1e6, 2), "ms_graph": graph_ms(torch, hn)}
     # measured ceiling for the HBM-bound rows: a device-to-device copy of the size of cfg5b's four streams
     # (73.4 MB read + 73.4 MB written), by the same timing method
     csrc = torch.empty(73_400_320, dtype=torch.uint8, device="cuda").fill_(1)
@@ -187,12 +217,13 @@ def all_configs(torch, bd, cin, keep):
         ws = torch.empty(40 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
         sc = torch.empty(8 * ws.numel(), dtype=torch.float32, device="cuda")     # partial states (mi_linear_attn_scratch_bytes)
         o = torch.empty_like(ql)
-        mn, av = event_ms(torch, lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc), 20)
+        la = lambda: bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc)   # noqa: E731
+        mn, av = event_ms(torch, la, 20)
         nbytes = 4 * 2 * n * 2240 * 2
         out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "gbs": round(nbytes / (mn * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (mn * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                      "frac_copy_ceiling": round(nbytes / (mn * 1e-3) / 1e9 / copy_gbs, 4), "dtype": "bf16 in, f32 accumulate",
-                     "mbytes": round(nbytes / 1e6, 2)}
+                     "mbytes": round(nbytes / 1e6, 2), "ms_graph": graph_ms(torch, la)}
         keep[key] = o
     return out
 
