@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <unordered_map>
 
 namespace bdamd {
 namespace {
@@ -37,10 +38,20 @@ void init_args(mi_sdpa_args& a, const char* op, const Tensor& Q, const Tensor& K
     a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.num_kv_heads = num_kv_heads;
     a.q_len = Q.rows; a.kv_len = K.rows;
 }
-// Launch with this thread's split scratch lent when the call can use one (grown on demand, then kept: no allocation
-// after warm-up; never destroyed, see thread_scratch below for why).
+// Scratch that this layer owns exists once per (thread, library stream of that thread at the time of the call) and use
+// (Tag): calls on one stream run in order and may share it, calls that a thread puts on different streams may overlap on
+// the GPU and get one each. Grown on demand, then kept (no allocation after warm-up), and never destroyed: a destructor
+// running at thread or process exit could call into a GPU runtime that is already gone.
+template <typename T, typename Tag> T& per_stream() {
+    static thread_local std::unordered_map<void*, T*>* m = new std::unordered_map<void*, T*>;
+    T*& t = (*m)[mi_get_stream()];
+    if (t == nullptr) t = new T;
+    return *t;
+}
+// Launch with the split scratch lent when the call can use one.
 void run_sdpa(const char* op, mi_sdpa_args& a) {
-    static thread_local Tensor* scratch = new Tensor;
+    struct SplitScratch;
+    Tensor* const scratch = &per_stream<Tensor, SplitScratch>();
     const std::size_t need = mi_sdpa_split_scratch_bytes(&a);
     if (need > 0) {
         if (scratch->data == nullptr || scratch->bytes() < need) scratch->resize(1, static_cast<int>((need + 3) / 4), Dtype::FP32, Device::GPU);
@@ -200,9 +211,8 @@ const float* need_weight(const char* op, const Tensor& W, const char* name, Dtyp
     return scales ? static_cast<const float*>(scales->data) : nullptr;
 }
 Tensor& thread_scratch() {
-    // never destroyed: a destructor running at thread or process exit could call into a GPU runtime that is already gone
-    static thread_local Tensor* t = new Tensor;
-    return *t;
+    struct BlockScratch;
+    return per_stream<Tensor, BlockScratch>();
 }
 void lend_scratch(mi_attn_block_args& a, Tensor* scratch, bool with_kv) {
     Tensor& s = scratch ? *scratch : thread_scratch();
@@ -350,9 +360,9 @@ void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const
         if (logit_bias->dtype != Dtype::FP32 || logit_bias->rows != Lq || logit_bias->cols != Lk) fail(std::string(op) + ": logit_bias must be FP32 (Lq, Lk)");
         bias = static_cast<const float*>(logit_bias->data);
     }
-    // per-thread scratch, never destroyed (see thread_scratch): projected Q, K, V, the attention output, the denominators
+    // scratch of this layer (see per_stream): projected Q, K, V, the attention output, the denominators
     struct Work { Tensor q, k, v, a, lse; };
-    static thread_local Work* w = new Work;
+    Work* const w = &per_stream<Work, Work>();
     linear_impl(op, Wq, nullptr, nullptr, X, w->q);
     linear_impl(op, Wk, nullptr, nullptr, Ctx, w->k);
     linear_impl(op, Wv, nullptr, nullptr, Ctx, w->v);
@@ -587,7 +597,8 @@ void joint_attention_traced(const Tensor& Q, const Tensor& K, const Tensor& V, c
         need_gpu(op, *image_text_bias);
         if (txt_len > 0 && txt_len < L) bias = static_cast<const float*>(image_text_bias->data);
     }
-    static thread_local Tensor* lse = new Tensor;   // per-thread scratch, never destroyed (see thread_scratch)
+    struct TracedLse;
+    Tensor* const lse = &per_stream<Tensor, TracedLse>();   // scratch of this layer (see per_stream)
     if (lse->data == nullptr || lse->size() < static_cast<std::size_t>(num_heads) * L) lse->resize(num_heads, L, Dtype::FP32, Device::GPU);
     mi_sdpa_args a;
     init_args(a, op, Qr, Kr, V, num_heads, num_heads, out);

@@ -87,7 +87,7 @@ void flash_attention_project_kv_int8w_fp16(const Tensor& ctx, const Tensor& Wk, 
 // The U-Net's traced cross attention (src/unet_blocks.cpp:282-290): Q = X Wq^T, K = Ctx Wk^T, V = Ctx Wv^T (no biases),
 // attention with the optional additive logit bias (FP32 (Lq, Lk)) and key mask, out = A Wo^T (no bias: the caller adds
 // it), AttnAvg = the FP32 (Lq, Lk) softmax averaged over the heads. Everything stays on the device; the projected
-// tensors live in a per-thread scratch.
+// tensors live in a scratch this layer keeps per thread and stream.
 void cross_attention_forward_with_attn(const Tensor& X, const Tensor& Ctx, const Tensor& Wq, const Tensor& Wk, const Tensor& Wv,
                                        const Tensor& Wo, const float* d_mask, const Tensor* logit_bias, int num_heads,
                                        Tensor& out, Tensor& AttnAvg);

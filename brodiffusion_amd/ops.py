@@ -246,10 +246,13 @@ _split_scratch_cache = {}
 
 
 def _own_split_scratch(device, nbytes: int) -> torch.Tensor:
-    t = _split_scratch_cache.get(device)
+    """The scratch this layer lends when the caller brings none: one per (device, current stream), grown on demand. Calls
+    on one stream run in order and may share it; calls on different streams may overlap on the GPU and must not."""
+    key = (device, _stream())
+    t = _split_scratch_cache.get(key)
     if t is None or t.numel() < nbytes:
         t = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _split_scratch_cache[device] = t
+        _split_scratch_cache[key] = t
     return t
 
 

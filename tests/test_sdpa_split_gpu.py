@@ -100,3 +100,29 @@ def test_calls_that_do_not_split():
     assert split_bytes(h, q[:512], q[:512], H) == 0                                   # 8 key tiles: nothing to gain
     q40 = torch.zeros(2, 4096, 320, device="cuda", dtype=torch.float16)
     assert split_bytes(q40, q40, q40, 8) == 0                                         # head_dim 40 runs on the kernel without split
+
+
+def test_own_split_scratch_is_per_stream():
+    """Two streams run split launches of different problems at the same time with the scratch the Python layer lends by
+    itself: each stream has its own (a shared one would be written by both launches at once), and every result equals the
+    one computed alone, bit for bit."""
+    H, d = 24, 128
+    probs = []
+    for i, L in enumerate((3328, 4096)):
+        q, k, v = (to_dev(randn(8300 + 3 * i + j, (1, L, H * d), "bf16"), "bf16") for j in range(3))
+        assert split_bytes(q, k, v, H) > 0
+        probs.append((q, k, v, bd.sdpa_forward(q, k, v, H)))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    for _ in range(4):                      # alternate the submissions so that the launches overlap on the GPU
+        for s, (q, k, v, _), o in zip(streams, probs, outs):
+            with torch.cuda.stream(s):
+                o.append(bd.sdpa_forward(q, k, v, H))
+    torch.cuda.synchronize()
+    from brodiffusion_amd import ops
+    keys = [key for key in ops._split_scratch_cache if key[1] in {s.cuda_stream for s in streams}]
+    assert len(keys) == 2 and ops._split_scratch_cache[keys[0]].data_ptr() != ops._split_scratch_cache[keys[1]].data_ptr()
+    for (_, _, _, ref), o in zip(probs, outs):
+        for got in o:
+            assert torch.equal(got, ref)
