@@ -72,9 +72,15 @@ def _dtype_code(op: str, t: torch.Tensor) -> int:
 
 
 def _dev(op: str, *ts):
+    """Every tensor on the GPU, and on the GPU that is current: the launch goes to the current device's stream (one process
+    per GPU is the intended use; with several visible, select the tensors' device first)."""
     for t in ts:
-        if t is not None and not t.is_cuda:
+        if t is None:
+            continue
+        if not t.is_cuda:
             _fail(op, "tensor is not on the GPU (CPU tensors are refused, not copied)")
+        if t.device.index != torch.cuda.current_device():
+            _fail(op, f"tensor is on cuda:{t.device.index} but the current device is cuda:{torch.cuda.current_device()}")
 
 
 def _stream() -> int:
