@@ -99,6 +99,9 @@ int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 // Scratch bytes with which launch_sdpa would split the last round of this launch (0: it would not split).
 size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim);
 bool sdpa_supported(int dtype, int head_dim);
+// Head dimensions 256 and 512 (sdpa_wide.hip): one 32-row query tile per work group, the head dimension dealt out to its wavefronts.
+bool sdpa_wide_head(int head_dim);
+int launch_sdpa_wide(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 
 // Device-side view of the head-averaged attention map launch (batch 1).
 struct MapDev {

@@ -1126,7 +1126,7 @@ int launch_t(const SdpaDev& p, int head_dim, int n_cu, hipStream_t stream) {
         case 112: return launch_d<T, 112>(p, n_cu, stream);
         case 128: return launch_d<T, 128>(p, n_cu, stream);
         case 160: return launch_d<T, 160>(p, n_cu, stream);
-        default: return fail("mi_sdpa_forward: head_dim %d has no kernel (40, 64, 72, 80, 96, 112, 128, 160)", head_dim);
+        default: return fail("mi_sdpa_forward: head_dim %d has no kernel (40, 64, 72, 80, 96, 112, 128, 160, 256, 512)", head_dim);
     }
 }
 
@@ -1136,7 +1136,7 @@ bool sdpa_supported(int dtype, int head_dim) {
     if (dtype != MI_DTYPE_F16 && dtype != MI_DTYPE_BF16) return false;
     switch (head_dim) {
         case 40: case 64: case 72: case 80: case 96: case 112: case 128: case 160: return true;
-        default: return false;
+        default: return sdpa_wide_head(head_dim);
     }
 }
 
@@ -1149,6 +1149,7 @@ size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim) {
 }
 
 int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream) {
+    if (sdpa_wide_head(head_dim)) return launch_sdpa_wide(p, dtype, head_dim, stream);
     const int n_cu = device_cu_count();
     if (dtype == MI_DTYPE_BF16) return launch_t<__bf16>(p, head_dim, n_cu, stream);
     if (dtype == MI_DTYPE_F16) return launch_t<_Float16>(p, head_dim, n_cu, stream);
