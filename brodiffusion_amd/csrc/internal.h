@@ -99,7 +99,7 @@ int launch_sdpa(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 // Scratch bytes with which launch_sdpa would split the last round of this launch (0: it would not split).
 size_t sdpa_split_scratch_bytes(const SdpaDev& p, int dtype, int head_dim);
 bool sdpa_supported(int dtype, int head_dim);
-// Head dimensions 256 and 512 (sdpa_wide.hip): one 32-row query tile per work group, the head dimension dealt out to its wavefronts.
+// Head dimensions 256, 384 and 512 (sdpa_wide.hip): one 32-row query tile per work group, the head dimension dealt out to its wavefronts.
 bool sdpa_wide_head(int head_dim);
 int launch_sdpa_wide(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream);
 

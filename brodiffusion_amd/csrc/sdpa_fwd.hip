@@ -1126,7 +1126,7 @@ int launch_t(const SdpaDev& p, int head_dim, int n_cu, hipStream_t stream) {
         case 112: return launch_d<T, 112>(p, n_cu, stream);
         case 128: return launch_d<T, 128>(p, n_cu, stream);
         case 160: return launch_d<T, 160>(p, n_cu, stream);
-        default: return fail("mi_sdpa_forward: head_dim %d has no kernel (40, 64, 72, 80, 96, 112, 128, 160, 256, 512)", head_dim);
+        default: return fail("mi_sdpa_forward: head_dim %d has no kernel (40, 64, 72, 80, 96, 112, 128, 160, 256, 384, 512)", head_dim);
     }
 }
 

@@ -1,6 +1,6 @@
-// Softmax attention for head dimensions 256 and 512 on gfx950: the single wide head of a VAE mid-block
-// (src/vae.cpp:259-277: one head over all 512 channels of a 64 x 64 latent), through the same entry point as every
-// other head dimension.
+// Softmax attention for head dimensions 256, 384 and 512 on gfx950: the single wide head of a VAE mid-block
+// (src/vae.cpp:259-277: one head over all 512 channels of a 64 x 64 latent; src/vae_qwenimage.cpp:322-340: 384 channels),
+// through the same entry point as every other head dimension.
 //
 // At these widths the output accumulator of a query row (head_dim floats per lane pair) no longer fits the registers of one
 // wavefront, so the head dimension is dealt out to the four wavefronts of a work group instead of the query rows: all four
@@ -200,7 +200,7 @@ int launch_wide_d(const SdpaDev& p, hipStream_t stream) {
 
 }  // namespace
 
-bool sdpa_wide_head(int head_dim) { return head_dim == 256 || head_dim == 512; }
+bool sdpa_wide_head(int head_dim) { return head_dim == 256 || head_dim == 384 || head_dim == 512; }
 
 int launch_sdpa_wide(const SdpaDev& p, int dtype, int head_dim, hipStream_t stream) {
     const char* what = nullptr;
@@ -210,9 +210,14 @@ int launch_sdpa_wide(const SdpaDev& p, int dtype, int head_dim, hipStream_t stre
     else if (p.lse) what = "lse_out";
     else if (p.cu_q) what = "packed variable-length sequences";
     if (what) return fail("mi_sdpa_forward: head_dim %d does not offer %s", head_dim, what);
-    if (dtype == MI_DTYPE_BF16) return head_dim == 256 ? launch_wide_d<__bf16, 256>(p, stream) : launch_wide_d<__bf16, 512>(p, stream);
-    if (dtype == MI_DTYPE_F16) return head_dim == 256 ? launch_wide_d<_Float16, 256>(p, stream) : launch_wide_d<_Float16, 512>(p, stream);
-    return fail("mi_sdpa_forward: dtype %d not supported (fp16 = 1, bf16 = 2)", dtype);
+    if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_F16) return fail("mi_sdpa_forward: dtype %d not supported (fp16 = 1, bf16 = 2)", dtype);
+    const bool bf = dtype == MI_DTYPE_BF16;
+    switch (head_dim) {
+        case 256: return bf ? launch_wide_d<__bf16, 256>(p, stream) : launch_wide_d<_Float16, 256>(p, stream);
+        case 384: return bf ? launch_wide_d<__bf16, 384>(p, stream) : launch_wide_d<_Float16, 384>(p, stream);
+        case 512: return bf ? launch_wide_d<__bf16, 512>(p, stream) : launch_wide_d<_Float16, 512>(p, stream);
+        default: return fail("mi_sdpa_forward: head_dim %d has no kernel", head_dim);
+    }
 }
 
 }  // namespace mi

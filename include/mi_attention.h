@@ -198,7 +198,7 @@ MI_API size_t mi_sdpa_split_scratch_bytes(const mi_sdpa_args* args);
  * would move tiles by LDS DMA (head_dim 72 and 128). Results agree to rounding; no reference counterpart. */
 MI_API int mi_sdpa_set_kernel_choice(int32_t choice);
 /* 1 if (dtype, head_dim) has a compiled kernel, else 0: fp16 / bf16 at head_dim 40, 64, 72, 80, 96, 112, 128, 160, and at
- * 256 and 512 (one wide head, src/vae.cpp:259-277) without cached prefix, logit bias, lse_out and packed sequences. */
+ * 256, 384 and 512 (one wide head, src/vae.cpp:259-277, src/vae_qwenimage.cpp:322-340) without cached prefix, logit bias, lse_out and packed sequences. */
 MI_API int mi_sdpa_supported(int32_t dtype, int32_t head_dim);
 
 /* ── head-averaged attention map ───────────────────────────────────────────

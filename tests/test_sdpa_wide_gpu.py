@@ -1,4 +1,4 @@
-"""Head dimensions 256 and 512 (the single wide head of the VAE mid-block attention, src/vae.cpp:259-277, reached through
+"""Head dimensions 256, 384 and 512 (the single wide head of the VAE mid-block attention, src/vae.cpp:259-277, reached through
 flash_attention_qkvo_forward with one head) against the CPU checker: plain, ragged, causal / windowed, key padding three
 ways, a scattered key mask, grouped K/V heads, batch, and the block operator itself with one head of 512 channels."""
 import numpy as np
@@ -16,6 +16,8 @@ pytestmark = pytest.mark.gpu
     ("fp16", 1, 512, 256, 256),
     ("fp16", 1, 256, 65, 64),
     ("bf16", 2, 256, 100, 333),
+    ("bf16", 1, 384, 200, 131),    # the Qwen-Image VAE's width (src/vae_qwenimage.cpp:322-340)
+    ("fp16", 2, 384, 33, 64),
     ("bf16", 1, 512, 1, 1),
 ])
 def test_wide_head_matches_checker(oracle, dtype, H, d, Lq, Lk):
