@@ -102,6 +102,21 @@ def graph_ms(torch, fn, calls=20, reps=5):
         return None
 
 
+def calibration(torch, bd):
+    """What the matrix pipes of this box sustain right now: a bare v_mfma_f32_32x32x16_bf16 loop on every compute unit
+    (mi_mfma_probe) with all-zero and with N(0,1) operands, after the same preheat as the timed step. The clock is
+    power-managed, so the two differ, and boxes differ; MFMA-bound rows can be divided by the N(0,1) figure."""
+    g = torch.Generator(device="cuda").manual_seed(77)
+    rnd = torch.randn(1 << 20, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+    res = {"what": "bare v_mfma_f32_32x32x16_bf16 loop on all compute units (mi_mfma_probe), 8 wavefronts per work group, 2 work groups per CU"}
+    for name, ops in (("zeros", torch.zeros_like(rnd)), ("randn", rnd)):
+        preheat(torch, lambda: bd.mfma_probe(ops, trips=500, reps=1), 0.1)
+        r = bd.mfma_probe(ops, trips=4000, reps=5)
+        res[f"mfma_loop_{name}_tflops"] = round(r["tflops"], 1)
+        res[f"mfma_loop_{name}_shader_mhz"] = round(r["shader_mhz"], 0)
+    return res
+
+
 def seeded(torch, seed, shape, dtype):
     """N(0,1) values of torch's CPU generator for `seed` (what torch_randn_f32(seed, n) of the reference's torch_rng.h
     reproduces), rounded once to `dtype`, on the GPU."""
@@ -118,9 +133,11 @@ def config_inputs(torch):
     c = {}
     c["cfg1"] = tuple(seeded(torch, 1000 + i, (2, 4096, 320), f16) for i in (1, 2, 3))
     c["cfg2a"] = tuple(seeded(torch, 2000 + i, (2, 4096, 1152), b16) for i in (1, 2, 3))
-    gen = torch.Generator().manual_seed(2099)
-    valid = [int(20 + torch.randint(0, 281, (1,), generator=gen).item()) for _ in range(2)]
-    c["cfg2b"] = (c["cfg2a"][0], seeded(torch, 2012, (2, 300, 1152), b16), seeded(torch, 2013, (2, 300, 1152), b16), valid)
+    # text keys / values from seeds 2011 / 2012, valid length of batch item b = 20 + (first output of std::mt19937(2099 + b)) % 281:
+    # the tensors tests/test_baseline_configs_gpu.py checks (numpy's legacy seeding is the same init_genrand)
+    import numpy as np
+    valid = [20 + int(np.random.RandomState(2099 + b).randint(0, 2 ** 32, dtype=np.uint64)) % 281 for b in range(2)]
+    c["cfg2b"] = (c["cfg2a"][0], seeded(torch, 2011, (2, 300, 1152), b16), seeded(torch, 2012, (2, 300, 1152), b16), valid)
     c["cfg4"] = (seeded(torch, 4001, (4096, 3072), b16), seeded(torch, 4002, (4608, 3072), b16), seeded(torch, 4003, (4608, 3072), b16))
     c["cfg5a"] = tuple(seeded(torch, 5000 + i, (2, 1024, 2240), b16) for i in (1, 2, 3))
     c["cfg5b"] = tuple(seeded(torch, 5010 + i, (2, 4096, 2240), b16) for i in (1, 2, 3))
@@ -136,11 +153,18 @@ def all_configs(torch, bd, cin, keep):
 
     out = {}
 
-    def sdpa_entry(name, flops, fn, dtype):
+    def sdpa_entry(name, flops, fn, dtype, hbm_bytes=None):
+        """hbm_bytes: algorithmic bytes of a call that sits below the ridge (~312 FLOP/B) and is therefore bound by HBM,
+        not by the matrix pipes; such a row also carries GB/s and its fraction of the HBM peak (from the graph time: a
+        call this short is submitted more slowly than it runs)."""
         mn, av = event_ms(torch, fn, 20)
         out[name] = {"ms_min": round(mn, 4), "ms_mean": round(av, 4), "tflops": round(flops / (mn * 1e-3) / 1e12, 1),
                      "frac_mfma_peak": round(flops / (mn * 1e-3) / 1e12 / PEAK_MFMA_BF16_TFLOPS, 4), "dtype": dtype,
                      "gflop": round(flops / 1e9, 2), "ms_graph": graph_ms(torch, fn)}
+        if hbm_bytes is not None:
+            t = out[name]["ms_graph"] or mn
+            out[name].update({"bound": "hbm", "mbytes": round(hbm_bytes / 1e6, 2), "flop_per_byte": round(flops / hbm_bytes, 1),
+                              "gbs": round(hbm_bytes / (t * 1e-3) / 1e9, 1), "frac_hbm_peak": round(hbm_bytes / (t * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
 
     q, k, v = cin["cfg1"]
     o1 = torch.empty_like(q)
@@ -157,7 +181,9 @@ def all_configs(torch, bd, cin, keep):
                lambda: bd.flash_attention_qkvo_forward(x, None, wq, None, wk, None, wv, None, wo, bo, None, 8, False, out=blk_out, scratch=blk_scratch), "fp16")
     kc1, vc1 = bd.flash_attention_project_kv(ctx, wk2, None, wv2, None)
     sdpa_entry("sd15_unet_block_crossattn_kvcached_c320_fp16", 4 * 2 * 8 * 4096 * 77 * 40 + 2 * 2 * 8192 * 320 * 320,
-               lambda: bd.flash_attention_q_with_kv_cached_forward(x, kc1, vc1, wq, None, wo, bo, None, 8, False, out=blk_out, scratch=blk_scratch), "fp16")
+               lambda: bd.flash_attention_q_with_kv_cached_forward(x, kc1, vc1, wq, None, wo, bo, None, 8, False, out=blk_out, scratch=blk_scratch), "fp16",
+               # x in, Q out and in, attention out and in, block out (6 passes over 8192 x 320) + K / V + the two weights
+               hbm_bytes=2 * (6 * 8192 * 320 + 2 * 2 * 77 * 320 + 2 * 320 * 320))
     x2 = x.view(8192, 320)
     y2 = torch.empty(8192, 320, dtype=torch.float16, device="cuda")
     sdpa_entry("linear_8192x320x320_fp16", 2 * 8192 * 320 * 320, lambda: bd.linear_batched(wo, bo, x2, y2), "fp16")
@@ -176,7 +202,8 @@ def all_configs(torch, bd, cin, keep):
     _, kc, vc, valid = cin["cfg2b"]
     vl = torch.tensor(valid, dtype=torch.int32, device="cuda")
     o2b = torch.empty_like(q)
-    sdpa_entry("cfg2b_pixart_crossattn_d72_bf16", 4 * 16 * 4096 * sum(valid) * 72, lambda: bd.sdpa_forward(q, kc, vc, 16, kv_valid_len=vl, out=o2b), "bf16")
+    sdpa_entry("cfg2b_pixart_crossattn_d72_bf16", 4 * 16 * 4096 * sum(valid) * 72, lambda: bd.sdpa_forward(q, kc, vc, 16, kv_valid_len=vl, out=o2b), "bf16",
+               hbm_bytes=2 * (2 * q.numel() + 2 * sum(valid) * 1152))    # Q in, O out, the valid K and V rows
     out["cfg2b_pixart_crossattn_d72_bf16"]["valid_len"] = valid
     keep["cfg2b"] = o2b
     q, k, v = (rnd(4608, 3072) for _ in range(3))
@@ -195,6 +222,34 @@ def all_configs(torch, bd, cin, keep):
                lambda: bd.sdpa_forward(qb, kb, vb, 24, k_prefix=kp, v_prefix=vp, mask=mask, out=o4), "bf16")
     keep["cfg4"] = o4
     out["cfg4_qwen_blockcausal_prefixkv_d128_bf16"]["dense_equivalent_gflop"] = round(4 * 24 * 4096 * 4608 * 128 / 1e9, 2)
+    # dit::joint_attention_traced at Flux size (src/dit/common.cpp:198-329): RoPE of Q and K, attention with the image->text
+    # logit bias and the softmax denominators, the head-averaged (L, L) map; and the attention launch of that call alone
+    tb = rnd(4096, 512, dt=torch.float32) * 0.5
+    o3x = torch.empty_like(q)
+    qr3, tmap, lse3 = torch.empty_like(q), torch.empty(4608, 4608, dtype=torch.float32, device="cuda"), torch.empty(24, 4608, dtype=torch.float32, device="cuda")
+    sdpa_entry("flux_joint_attention_traced_bias_map_d128_bf16", 2 * 4 * 24 * 4608 * 4608 * 128 - 2 * 24 * 4608 * 4608 * 128,
+               lambda: bd.joint_attention_traced(q, k, v, cos, sin, 128, 24, out=o3x, attn_avg=tmap, Qr=qr3, Kr=kr3, txt_len=512, image_text_bias=tb), "bf16")
+    out["flux_joint_attention_traced_bias_map_d128_bf16"]["note"] = "FLOPs: attention (QK^T, PV) + the map's second QK^T"
+    sdpa_entry("flux_traced_attention_half_bias_lse_d128_bf16", 4 * 24 * 4608 * 4608 * 128,
+               lambda: bd.sdpa_forward(qr3, kr3, v, 24, out=o3x, logit_bias=tb, bias_q0=512, lse_out=lse3), "bf16")
+    del tmap, tb
+    # dit::gqa_attention_masked at the shape the reference's kernel benchmark uses for it (tools/bench_krea2_kernels.cpp:78-79,
+    # :179-192: 48 query heads, 12 K/V heads, head_dim 128, 512 text + 4096 image rows), key padding mask hiding text keys
+    # 77..511; and the same call without a mask
+    qg, kg, vg = rnd(4608, 48 * 128), rnd(4608, 12 * 128), rnd(4608, 12 * 128)
+    og = torch.empty_like(qg)
+    dm = torch.ones(4608, dtype=torch.float32, device="cuda")
+    dm[77:512] = 0
+    sdpa_entry("gqa_attention_masked_48q12kv_d128_L4608_bf16", 4 * 48 * 4608 * (4608 - 435) * 128,
+               lambda: bd.gqa_attention_masked(qg, kg, vg, None, None, 128, 48, 12, dm, out=og), "bf16")
+    sdpa_entry("gqa_attention_unmasked_48q12kv_d128_L4608_bf16", 4 * 48 * 4608 * 4608 * 128,
+               lambda: bd.gqa_attention_masked(qg, kg, vg, None, None, 128, 48, 12, None, out=og), "bf16")
+    del qg, kg, vg, og
+    # bt::flash_attention_windowed_forward (src/dit/qwenimage21_forward.cpp:662): window 0 = causal, and a 1024-key window
+    pairs_causal = 4608 * 4609 // 2
+    pairs_win = sum(min(r + 1, 1024) for r in range(4608))
+    sdpa_entry("windowed_causal_w0_d128_L4608_bf16", 4 * 24 * pairs_causal * 128, lambda: bd.flash_attention_windowed_forward(q, k, v, None, 24, 0, out=o3x), "bf16")
+    sdpa_entry("windowed_w1024_d128_L4608_bf16", 4 * 24 * pairs_win * 128, lambda: bd.flash_attention_windowed_forward(q, k, v, None, 24, 1024, out=o3x), "bf16")
     xh, gh = rnd(4608, 3072), rnd(128)
     oh = torch.empty_like(xh)
     hn = lambda: bd.headnorm_rope(xh, gh, 1e-6, cos, sin, 128, 24, out=oh)   # noqa: E731
@@ -399,6 +454,10 @@ def main():
                      "step_ms_events": round(step_ms_events, 4)},
         "device": bd.device_info(),
     }
+    cal = calibration(torch, bd)
+    cal["headline_kernel_frac_of_randn_loop"] = round(achieved / cal["mfma_loop_randn_tflops"], 4)
+    cal["headline_kernel_frac_of_zeros_loop"] = round(achieved / cal["mfma_loop_zeros_tflops"], 4)
+    res["calibration"] = cal
     step()                                    # `out` holds the result of a step: compared with the checker below
     torch.cuda.synchronize()
     cin, keep = None, {}

@@ -9,6 +9,7 @@ from .ops import (  # noqa: F401
     build_axial_rope_tables,
     build_qwen_rope_tables,
     device_info,
+    mfma_probe,
     flash_attention_forward,
     flash_attention_project_kv,
     flash_attention_project_kv_int8w_fp16,
@@ -45,7 +46,7 @@ from .ops import (  # noqa: F401
 )
 
 __all__ = [
-    "SdpaMask", "build_axial_rope_tables", "build_qwen_rope_tables", "qwen_rope_positions", "rope_tables_from_positions", "device_info", "flash_attention_forward",
+    "SdpaMask", "build_axial_rope_tables", "build_qwen_rope_tables", "qwen_rope_positions", "rope_tables_from_positions", "device_info", "mfma_probe", "flash_attention_forward",
     "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
     "linear_attention_relu_forward", "linear_attention_relu_forward_static_scratch", "rope_apply", "flash_attention_qkvo_forward", "flash_attention_q_with_kv_cached_forward",
     "flash_attention_project_kv", "flash_attention_scratch_bytes", "linear_batched", "headnorm_rope", "flash_attention_varlen_forward", "flash_attention_qkvo_int8w_fp16", "flash_attention_q_with_kv_cached_int8w_fp16",

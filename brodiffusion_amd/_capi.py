@@ -20,7 +20,7 @@ MI_MAX_SEGMENTS = 32
 MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 
 EXPORTS = [
-    "mi_last_error", "mi_version", "mi_device_info", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
+    "mi_last_error", "mi_version", "mi_device_info", "mi_mfma_probe", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
     "mi_malloc", "mi_free", "mi_memcpy_h2d", "mi_memcpy_d2h", "mi_memcpy_d2d_async", "mi_memset_async",
     "mi_sdpa_forward", "mi_sdpa_split_scratch_bytes", "mi_sdpa_supported", "mi_sdpa_set_kernel_choice", "mi_attention_map_avg", "mi_rope_apply", "mi_headnorm_rope", "mi_scale_rows",
     "mi_linear_attn_workspace_bytes", "mi_linear_attn_scratch_bytes", "mi_linear_attn_relu_forward", "mi_linear_attn_supported", "mi_linear_attn_relu_forward_static_scratch",
@@ -33,6 +33,12 @@ class MiDeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("lds_bytes_per_cu", C.c_int32), ("l2_bytes", C.c_int32),
                 ("hbm_bytes", C.c_int64), ("peak_mfma_16bit_flops", C.c_double)]
+
+
+class MiMfmaProbeArgs(C.Structure):
+    _fields_ = [("struct_size", C.c_uint32), ("dtype", C.c_int32), ("operands", C.c_void_p), ("operand_bytes", C.c_size_t),
+                ("trips", C.c_int32), ("work_groups", C.c_int32), ("sink", C.c_void_p), ("sink_bytes", C.c_size_t),
+                ("clocks", C.c_void_p), ("clocks_bytes", C.c_size_t), ("flops", C.c_double), ("stream", C.c_void_p)]
 
 
 class MiSdpaArgs(C.Structure):
@@ -163,6 +169,7 @@ def lib() -> C.CDLL:
         L.mi_last_error.restype = C.c_char_p
         L.mi_version.restype = C.c_char_p
         L.mi_device_info.argtypes = [C.POINTER(MiDeviceInfo)]
+        L.mi_mfma_probe.argtypes = [C.POINTER(MiMfmaProbeArgs)]
         L.mi_set_stream.argtypes = [C.c_void_p]
         L.mi_get_stream.restype = C.c_void_p
         L.mi_stream_synchronize.argtypes = [C.c_void_p]

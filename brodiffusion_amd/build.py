@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmi_attention.so")
-SOURCES = ["capi.hip", "sdpa_fwd.hip", "sdpa_wide.hip", "rope.hip", "linear_attn.hip", "linear.hip", "linear_dma.hip", "attn_block.hip", "attn_map.hip", "elementwise.hip"]
+SOURCES = ["capi.hip", "sdpa_fwd.hip", "sdpa_wide.hip", "rope.hip", "linear_attn.hip", "linear.hip", "linear_dma.hip", "attn_block.hip", "attn_map.hip", "elementwise.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++20", "-fPIC", "-fvisibility=hidden",

@@ -228,6 +228,16 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
     }
     if (a->rope_k_scratch && !mi::aligned16(a->rope_k_scratch)) return fail("mi_sdpa_forward: rope_k_scratch must be 16-byte aligned");
     if (a->split_scratch && !mi::aligned16(a->split_scratch)) return fail("mi_sdpa_forward: split_scratch must be 16-byte aligned");
+    // what the wide-head kernel (head_dim 256 / 384 / 512) does not offer is refused here, before any work is enqueued
+    if (mi::sdpa_wide_head(a->head_dim)) {
+        const char* what = nullptr;
+        if (a->prefix_len > 0) what = "a cached prefix";
+        else if (p.cos_k && a->kv_len > 0 && !a->rope_k_scratch) what = "K rotated tile by tile (lend rope_k_scratch)";
+        else if (p.bias) what = "a logit bias";
+        else if (p.lse) what = "lse_out";
+        else if (p.cu_q) what = "packed variable-length sequences";
+        if (what) return fail("mi_sdpa_forward: head_dim %d does not offer %s", a->head_dim, what);
+    }
     // the grid pads batch*heads to a multiple of 8 for masked calls
     const long nb = ((static_cast<long>(a->batch) * a->num_heads + 7) & ~7L) * ((a->q_len + 127) / 128);
     if (nb > 0x7fffffffL) return fail("mi_sdpa_forward: problem too large for one launch");
@@ -289,7 +299,9 @@ int mi_attention_map_avg(const mi_attention_map_args* a) {
     const char* op = "mi_attention_map_avg";
     if (!a) return fail("%s: null args", op);
     if (a->struct_size != sizeof(mi_attention_map_args)) return fail("%s: struct_size mismatch", op);
-    if (!mi::sdpa_supported(a->dtype, a->head_dim)) return fail("%s: no kernel for dtype %d head_dim %d", op, a->dtype, a->head_dim);
+    // (the map kernel covers the head dimensions of the 128-row attention kernel, which writes the denominators it reads)
+    if (!mi::sdpa_supported(a->dtype, a->head_dim) || mi::sdpa_wide_head(a->head_dim))
+        return fail("%s: no kernel for dtype %d head_dim %d", op, a->dtype, a->head_dim);
     if (a->num_heads <= 0 || a->q_len < 0 || a->kv_len < 0) return fail("%s: bad shape", op);
     if (a->q_len == 0 || a->kv_len == 0) return 0;
     if (!a->q || !a->k || !a->lse || !a->map) return fail("%s: q, k, lse and map must not be null", op);

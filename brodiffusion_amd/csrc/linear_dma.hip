@@ -76,8 +76,11 @@ __global__ void __launch_bounds__(kThreads, 2) linear_dma_kernel(const LinearBat
     // consecutive work-group ids go to the 8 XCDs in turn: give every XCD (one L2) a contiguous run of tiles, which
     // share their X rows and walk W together
     const int chunk = (n_tiles + 7) >> 3;
-    const int logical = (static_cast<int>(blockIdx.x) & 7) * chunk + (static_cast<int>(blockIdx.x) >> 3);
-    if (logical >= n_tiles) return;
+    // (the grid is sized for the problem of the launch with the most tiles: a smaller problem's run is shorter than the
+    //  grid's, and a group past the end of its XCD's run would repeat a tile of the next XCD's)
+    const int in_run = static_cast<int>(blockIdx.x) >> 3;
+    const int logical = (static_cast<int>(blockIdx.x) & 7) * chunk + in_run;
+    if (in_run >= chunk || logical >= n_tiles) return;
     const int m0 = (logical / tiles_n) * kTile, n0 = (logical % tiles_n) * kTile;
 
     const int tid = threadIdx.x;

@@ -114,6 +114,41 @@ def device_info() -> dict:
             "hbm_bytes": info.hbm_bytes, "peak_mfma_16bit_flops": info.peak_mfma_16bit_flops}
 
 
+def mfma_probe(operands: torch.Tensor, trips: int = 2000, reps: int = 5) -> dict:
+    """Sustained rate of a bare MFMA loop on every compute unit with `operands` (a fp16 / bf16 device tensor: zeros,
+    N(0,1), ...) as its inputs (mi_mfma_probe): TFLOP/s from event timing (best of `reps` launches after one warm-up
+    launch) and the shader clock under that load, from the kernel's own cycle and 100 MHz counters."""
+    op = "mfma_probe"
+    _dev(op, operands)
+    if not operands.is_contiguous():
+        _fail(op, "operands must be contiguous")
+    info = device_info()
+    n_wg = 2 * info["compute_units"]
+    sink = torch.empty(1024, dtype=torch.float32, device=operands.device)
+    clocks = torch.zeros(2 * n_wg, dtype=torch.int64, device=operands.device)
+    a = capi.MiMfmaProbeArgs()
+    a.struct_size = C.sizeof(a)
+    a.dtype = _dtype_code(op, operands)
+    a.operands, a.operand_bytes = operands.data_ptr(), operands.numel() * operands.element_size()
+    a.trips = trips
+    a.sink, a.sink_bytes = sink.data_ptr(), sink.numel() * 4
+    a.clocks, a.clocks_bytes = clocks.data_ptr(), clocks.numel() * 8
+    a.stream = _stream()
+    best = None
+    for i in range(reps + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        capi.check(capi.lib().mi_mfma_probe(C.byref(a)), "mi_mfma_probe")
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        if i > 0 and (best is None or ms < best):
+            best = ms
+    c = clocks.view(-1, 2).double()
+    mhz = float((c[:, 0] / c[:, 1].clamp(min=1)).mean().item() * 100.0)
+    return {"tflops": a.flops / (best * 1e-3) / 1e12, "ms": best, "shader_mhz": mhz, "flops": a.flops}
+
+
 def sdpa_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, num_heads: int, *, out: Optional[torch.Tensor] = None,
                  num_kv_heads: int = 0, k_prefix: Optional[torch.Tensor] = None, v_prefix: Optional[torch.Tensor] = None,
                  scale: Optional[float] = None, mask: Optional[SdpaMask] = None,

@@ -61,6 +61,30 @@ typedef struct mi_device_info_t {
 } mi_device_info_t;
 MI_API int mi_device_info(mi_device_info_t* out);
 
+/* Calibration probe for benchmarks; no counterpart in the reference. One launch on every compute unit of a loop of
+ * nothing but independent v_mfma_f32_32x32x16 instructions (`trips` trips of 8 per wavefront) on operands taken from
+ * `operands` (device memory of 16-bit values of `dtype`: all zeros, N(0,1), ...). The caller times the launch with
+ * events on `stream`; `flops` returns the FLOPs it performs. The sustained rate depends on the operand values because
+ * the clock is power-managed, so an MFMA-bound figure quoted against the nominal peak can be read against what the
+ * matrix pipes of this GPU sustain on comparable data at this moment. If `clocks` is given, work group g stores the
+ * shader cycles and the 100 MHz constant-rate ticks of its loop at clocks[2g], clocks[2g + 1]
+ * (cycles / ticks * 100 = MHz under this load). Writes 4096 bytes of `sink`. */
+typedef struct mi_mfma_probe_args {
+    uint32_t struct_size;
+    int32_t dtype;
+    const void* operands;
+    size_t operand_bytes;     /* >= 4096 */
+    int32_t trips;
+    int32_t work_groups;      /* out: work groups of the launch (2 per compute unit) */
+    float* sink;
+    size_t sink_bytes;        /* >= 4096 */
+    uint64_t* clocks;         /* NULL, or 2 * work_groups counts (ask with a first call, or size for 2 * 2 * compute_units) */
+    size_t clocks_bytes;
+    double flops;             /* out */
+    void* stream;
+} mi_mfma_probe_args;
+MI_API int mi_mfma_probe(mi_mfma_probe_args* args);
+
 /* The library's current stream (void* is a hipStream_t). Entry points whose args carry a
  * NULL stream launch here. Mirrors brotensor's cuda_current_stream() contract
  * (src/fused_transformer.cu:38-54). */

@@ -13,7 +13,7 @@ import torch
 
 import brodiffusion_amd as bd
 from brodiffusion_amd import _capi as capi
-from helpers import TORCH_DT, randn, to_dev, to_np
+from helpers import TORCH_DT, assert_close, randn, to_dev, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -100,3 +100,30 @@ def test_large_linear_agrees_with_small_tile_kernel():
     big = bd.linear_batched(w, b, x)                 # 18 x 12 tiles of 256 x 256: the large kernel
     small = bd.linear_batched(w, b, x[:2048])        # 8 x 12 tiles: the 128 x 128 kernel
     assert torch.equal(big[:2048], small)
+
+
+def test_unequal_problems_in_one_launch(oracle):
+    """The Q / K / V launch of a cross-attention block whose query rows far outnumber its context rows (12288 against
+    512): three problems of 192, 8 and 8 tiles in one launch of the large kernel, whose grid is sized for the largest.
+    Work groups beyond a small problem's own run of tiles must leave (they would repeat tiles of the neighbouring runs).
+    The block equals its parts bit for bit (the K / V projections alone run on the small-tile kernel, which accumulates
+    in the same order), and sampled rows of Q, K, V match the checker."""
+    dtype, L, Lc, C, H = "bf16", 12288, 512, 1024, 8
+    x, ctx = randn(51, (L, C), dtype), randn(52, (Lc, C), dtype)
+    wq, wk, wv, wo = (_weight(oracle, 53 + i, C, C, dtype) for i in range(4))
+    bq, bk, bv, bo = (oracle.round_to(randn(57 + i, (C,), dtype) * 0.25, dtype) for i in range(4))
+    dx, dctx = to_dev(x, dtype), to_dev(ctx, dtype)
+    dw = [to_dev(w, dtype) for w in (wq, wk, wv, wo)]
+    db = [to_dev(b, dtype) for b in (bq, bk, bv, bo)]
+    out = bd.flash_attention_qkvo_forward(dx, dctx, dw[0], db[0], dw[1], db[1], dw[2], db[2], dw[3], db[3], None, H, False)
+    q = bd.linear_batched(dw[0], db[0], dx)
+    k = bd.linear_batched(dw[1], db[1], dctx)
+    v = bd.linear_batched(dw[2], db[2], dctx)
+    parts = bd.linear_batched(dw[3], db[3], bd.flash_attention_forward(q, k, v, None, H, False))
+    assert torch.equal(parts, out)
+    rows = _rows(L, 64)
+    _one_ulp(oracle.linear(x[rows], wq, bq), to_np(q)[rows], dtype, "Q projection")
+    _one_ulp(oracle.linear(ctx, wk, bk), to_np(k), dtype, "K projection")
+    _one_ulp(oracle.linear(ctx, wv, bv), to_np(v), dtype, "V projection")
+    ref = oracle.attention_qkvo(x[rows], ctx, wq, bq, wk, bk, wv, bv, wo, bo, H, dtype)
+    assert_close(ref, to_np(out)[rows], dtype, "cross-attention block with unequal projections")

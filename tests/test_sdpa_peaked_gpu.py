@@ -12,10 +12,12 @@ softmax of every kernel form through what unit-spread inputs never reach:
   * +-300 queries against a few hundred keys with a valid length (the PixArt cross-attention shape).
 The bound is the one of every other parity test (helpers.TOL); the checker follows src/dit/common.cpp:269-293.
 
-V is N(0,1) / 4 here. A nearly one-hot row returns single V rows, so with unit-variance V the outputs reach magnitude 4,
+V is N(0,1) / 4 in the first group of tests. A nearly one-hot row returns single V rows, so with unit-variance V the outputs reach magnitude 4,
 where the 16-bit output format itself rounds by up to 1.6e-2 (bf16, half a unit in the last place): the absolute bound of
 2e-2 would then measure the storage format. At a quarter of that the outputs stay near 1, like the outputs of the
-unit-spread cases the bound was stated for; the relative bound does not depend on the scale of V at all.
+unit-spread cases the bound was stated for; the relative bound does not depend on the scale of V at all. The last group
+repeats the scaled-query and dominant-key cases on V of unit variance, with the absolute bound widened to one unit in the last
+place of the reference value where that exceeds it.
 """
 import numpy as np
 import pytest
@@ -156,3 +158,53 @@ def test_split_launch_scaled_queries(oracle, kernel_choice):
     rows = np.arange(3, L, 41, dtype=np.int32)
     ref = oracle.sdpa(q, k, v, H, rows=rows)
     assert_close(ref[rows], out[rows], dtype, "split")
+
+
+# ── the same cases on V of unit variance ──
+# Here nearly one-hot rows return single V rows of magnitude up to ~4, where the storage format alone rounds by half a unit
+# in the last place (bf16: 2^-7 = 7.8e-3 at |o| in [2, 4), 1.6e-2 at [4, 8)). The absolute bound therefore follows the
+# magnitude: max(the stated bound, one unit in the last place of |reference|), element by element; the relative bound is
+# the stated one.
+def _assert_close_ulp(ref, got, dtype, what):
+    import oracle
+    rel, mx = (5e-3, 2e-2) if dtype == "bf16" else (1e-3, 5e-3)
+    mant = 7 if dtype == "bf16" else 10
+    m = oracle.compare(ref, got)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    assert m["rel_l2"] <= rel, f"{what}: {m}"
+    ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - mant)
+    bound = np.maximum(mx, ulp)
+    worst = np.max(np.abs(got - ref) / bound)
+    assert worst <= 1.0, f"{what}: {m}, worst error / bound {worst:.3f}"
+    return m
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("d", [40, 72, 128])
+@pytest.mark.parametrize("qmul", [8.0, 16.0])
+def test_scaled_queries_dense_unit_v(oracle, d, dtype, qmul):
+    H, Lq, Lk = 2, 300, 640
+    q = randn(100 + d, (Lq, H * d), dtype) * np.float32(qmul)
+    k = randn(200 + d, (Lk, H * d), dtype); v = randn(300 + d, (Lk, H * d), dtype)
+    _assert_close_ulp(oracle.sdpa(q, k, v, H), _run(q, k, v, H, dtype), dtype, f"d={d} q x{qmul}, unit V")
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72)])
+def test_scaled_queries_masked_unit_v(oracle, d, dtype):
+    H, Lq, Lk, window, qmul = 2, 280, 470, 150, 16.0
+    q = randn(110 + d, (Lq, H * d), dtype) * np.float32(qmul)
+    k = randn(210 + d, (Lk, H * d), dtype); v = randn(310 + d, (Lk, H * d), dtype)
+    lo, hi = oracle.rows_causal(Lq, Lk, window=window)
+    out = _run(q, k, v, H, dtype, mask=bd.SdpaMask.causal(Lk - Lq, window))
+    _assert_close_ulp(oracle.sdpa(q, k, v, H, row_lo=lo, row_hi=hi), out, dtype, f"d={d} q x{qmul} windowed, unit V")
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72)])
+def test_one_dominant_key_unit_v(oracle, d, dtype):
+    H, Lq, Lk, jdom = 2, 260, 448, 200
+    k = randn(240 + d, (Lk, H * d), dtype); v = randn(340 + d, (Lk, H * d), dtype)
+    q = np.tile(k[jdom] * np.float32(4.0), (Lq, 1))
+    out = _run(q, k, v, H, dtype)
+    _assert_close_ulp(oracle.sdpa(q, k, v, H), out, dtype, f"d={d} dominant key, unit V")
+    unit = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11
+    assert np.all(np.abs(out - v[jdom]) <= unit * np.maximum(np.abs(v[jdom]), 1.0) * 1.01 + 5e-3)

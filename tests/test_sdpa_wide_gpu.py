@@ -102,3 +102,31 @@ def test_wide_head_refuses_what_it_does_not_offer():
     with pytest.raises(RuntimeError, match="does not offer packed"):
         cu = torch.tensor([0, 32, 64], dtype=torch.int32, device="cuda")
         bd.flash_attention_varlen_forward(q, q, q, cu, cu, 2, 32, 32, H, d, False)
+
+
+@pytest.mark.parametrize("split_half", [False, True], ids=["adjacent", "split_half"])
+@pytest.mark.parametrize("dtype,d", [("bf16", 256), ("fp16", 384), ("bf16", 512)])
+def test_wide_head_rope(oracle, dtype, d, split_half):
+    """Q rotated while it is staged and K rotated into the caller's scratch at the wide head dimensions, both pair
+    conventions: bit-equal to the stand-alone rotation followed by plain attention, and within the bound of the checker."""
+    H, L = 1, 150
+    q, k, v = (randn(8570 + d + i, (L, H * d), dtype) for i in range(3))
+    ang = np.random.default_rng(d).uniform(-3, 3, (L, d // 2))
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    dcos, dsin = torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    qr = bd.rope_apply(dq, dcos, dsin, d, H, split_half=split_half)
+    kr = bd.rope_apply(dk, dcos, dsin, d, H, split_half=split_half)
+    plain = bd.sdpa_forward(qr, kr, dv, H)
+    fused_q = bd.sdpa_forward(dq, kr, dv, H, rope_q=(dcos, dsin), rope_split_half=split_half)
+    assert torch.equal(fused_q, plain)
+    Kr = torch.empty_like(dk)
+    joint = bd.joint_attention(dq, dk, dv, dcos, dsin, d, H, Kr=Kr, split_half=split_half)
+    assert torch.equal(Kr, kr) and torch.equal(joint, plain)
+    ref = oracle.sdpa(oracle.rope_apply(q, cos, sin, H, d, split_half=split_half, round_to_dtype=dtype),
+                      oracle.rope_apply(k, cos, sin, H, d, split_half=split_half, round_to_dtype=dtype), v, H)
+    assert_close(ref, to_np(joint), dtype, f"wide head rope d={d} split_half={split_half}")
+    # without a scratch the rotation of K would have to happen tile by tile, which these widths do not offer: refused
+    # before anything is enqueued
+    with pytest.raises(RuntimeError, match="does not offer K rotated tile by tile|needs rope_k_scratch"):
+        bd.joint_attention(dq, dk, dv, dcos, dsin, d, H, split_half=split_half)

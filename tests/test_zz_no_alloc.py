@@ -45,8 +45,13 @@ def _both(oracle, B, H, d, N, seed, accumulate=False):
     # static route: outputs prefilled so that an entry point that writes nothing cannot pass
     o_st, ws_st = torch.full_like(dq, 7.0), state0.clone()
     a = _args(dq, dk, dv, o_st, ws_st, H, d, accumulate)
+    # the property the entry point exists for: no device memory is taken or returned during the call, neither through
+    # torch's allocator nor behind its back (free device memory as the driver reports it)
+    torch.cuda.synchronize()
+    free0, held0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     assert lib.mi_linear_attn_relu_forward_static_scratch(C.byref(a)) == 0, capi.last_error()
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == held0
     assert torch.equal(o_st, o_ref) and torch.equal(ws_st, ws_ref)
     if not accumulate:
         for b in range(B):
@@ -58,6 +63,23 @@ def test_static_scratch_entry_point_two_calls_in_a_row(oracle):
     _both(oracle, 1, 6, 112, 300, 9810)            # smaller: fewer heads, fewer and shorter chunks, same array
     _both(oracle, 2, 70, 32, 512, 9820)            # another head_dim: the slots are laid out differently
     _both(oracle, 1, 6, 112, 300, 9830, accumulate=True)
+
+
+def test_static_scratch_reduced_split(oracle):
+    """A state of 5.3 MB: the 16 MiB array holds three partial states per (batch, head) instead of eight, so the tokens are
+    split less far than with a caller scratch of full size and the two routes no longer add in the same order; the result
+    is held to the checker instead."""
+    lib = capi.lib()
+    dtype, B, H, d, N = "bf16", 2, 40, 128, 1536
+    need = lib.mi_linear_attn_workspace_bytes(B, H, d)
+    assert 1 <= capi.MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES // need < 8
+    q, k, v = (randn(9840 + i, (B, N, H * d), dtype) for i in range(3))
+    dq, dk, dv = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    o, ws = torch.full_like(dq, 7.0), torch.zeros(need // 4, device="cuda")
+    assert lib.mi_linear_attn_relu_forward_static_scratch(C.byref(_args(dq, dk, dv, o, ws, H, d))) == 0, capi.last_error()
+    torch.cuda.synchronize()
+    for b in range(B):
+        assert_close(oracle.linear_attn_relu(q[b], k[b], v[b], H), to_np(o[b]), dtype, f"reduced split, batch {b}")
 
 
 def test_static_scratch_entry_point_limits():
