@@ -199,6 +199,7 @@ int prepare_sdpa(const mi_sdpa_args* a, SdpaDev& p, long& Dkv_out) {
         p.bias_rs = a->bias_row_stride ? a->bias_row_stride : a->bias_cols;
         if (p.bias_rs < p.bias_cols) return fail("mi_sdpa_forward: bias_row_stride smaller than bias_cols");
         if (reinterpret_cast<uintptr_t>(a->logit_bias) & 3u) return fail("mi_sdpa_forward: logit_bias must be 4-byte aligned");
+        p.bias_vec_ok = ((reinterpret_cast<uintptr_t>(a->logit_bias) & 15u) == 0 && p.bias_rs % 4 == 0) ? 1 : 0;
         if (a->bias_cols == 0 || a->bias_q0 >= a->q_len) p.bias = nullptr;   // nothing to add
     }
     {

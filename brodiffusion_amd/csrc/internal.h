@@ -76,12 +76,14 @@ struct SdpaDev {
     int n_q_tiles; int n_blocks;  // logical work items = B*H*n_q_tiles
     // additive logit bias (natural-log units, added to the scaled score) for query rows >= bias_q0 and keys < bias_cols
     const float* bias; int bias_q0, bias_cols; long bias_rs;
+    int bias_vec_ok;              // bias base 16-byte aligned and bias_rs a multiple of 4: rows can be read 4 floats at a time
     float inv_scale;              // 1 / scale: the bias in units of the raw dot product
     const int* cu_q; const int* cu_k;   // packed variable-length sequences: [B + 1] row offsets, or null
     float* lse;                   // [B][H][Lq] base-2 log of the softmax denominator in exponent units, or null
     int prefix_scaled;            // the rows of the cached prefix carry factors: K rows pk_scale * pk_row[j], V rows pv_scale * pv_row[j]
     float pk_scale, pv_scale;
     const float* pk_row; const float* pv_row;   // [Lp] or null
+    int kbits_off;                // byte offset in dynamic LDS of the key-visibility words (256-row kernels with a key mask)
     SplitGeo split;               // enabled != 0: split the last round along the key axis
     unsigned char* split_scratch; // partial slots, [8 groups][max_tail][max_parts] of SplitGeo::slot_bytes
     size_t split_scratch_bytes;   // what the caller lent

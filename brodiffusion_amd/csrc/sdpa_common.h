@@ -472,6 +472,16 @@ __device__ __forceinline__ float pair_sum(const typename Mma<T>::v8& v, int i, f
     else return __builtin_amdgcn_fdot2(pr, one, acc, false);
 }
 
+// What the XTRA instances of the 256-row kernels bring to a tile's softmax: the visibility bits of the tile's 64 keys (bit i
+// of kw0: key i of the tile passes the key mask, kw1: key 32 + i; all ones without a mask) and this lane's row of the additive
+// logit bias (null: the tile or the row has none), which is given in natural-log units and added to the exponents times log2 e.
+struct TileExtra {
+    unsigned kw0 = ~0u, kw1 = ~0u;
+    const float* bias_row = nullptr;
+    int bias_cols = 0;
+    bool bias_vec = false;   // the whole tile lies below bias_cols and its 4-key pieces are 16-byte aligned in every row
+};
+
 struct RelSoftmaxState {
     float l = 0.f;          // this lane's share of the denominator
     float neg_ref = 0.f;    // minus the row's reference, in exponent (base-2) units
@@ -479,10 +489,10 @@ struct RelSoftmaxState {
 };
 constexpr float kRelSumMax = 1024.f;
 
-template <typename T, int D, bool PSCALE = false>
+template <typename T, int D, bool PSCALE = false, bool XTRA = false>
 __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma<T>::v8 (&pf)[4], f32x16 (&oacc)[HeadGeo<D>::VB],
                                                  RelSoftmaxState& st, bool masked, bool dead_row, int j0, int lo, int hi, int lh,
-                                                 PrefixScale prefix = PrefixScale()) {
+                                                 PrefixScale prefix = PrefixScale(), TileExtra xt = TileExtra()) {
     // Tile of the cached prefix whose rows carry factors (wave-uniform flag; PSCALE instances only, so that the other
     // instances keep their register budget). The scores arrive as exponents x = s * cl2 - ref; K's factor f belongs on s:
     // x' = f * (x + ref) - ref.
@@ -495,19 +505,58 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
     }
     if (masked) {
         const int d0 = j0 + 4 * lh - lo, top = hi - 1 - lo;   // keys outside [lo, hi) become -inf
+        if constexpr (XTRA) {
+            if (xt.bias_row) {
+                constexpr float kLog2e = 1.4426950408889634f;
+                if (xt.bias_vec) {
+                    // a lane's 32 keys are 8 pieces of 4 consecutive ones: all loads go out before the first is used
+                    f32x4 bv[2][4];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+                    for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float score = sacc[kb][e];
-                sacc[kb][e] = blank_outside(score, d0 + 32 * kb + 8 * (e >> 2) + (e & 3), top);
+                        for (int bb = 0; bb < 4; ++bb) bv[kb][bb] = *reinterpret_cast<const f32x4*>(xt.bias_row + j0 + 32 * kb + 8 * bb + 4 * lh);
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) sacc[kb][e] = __builtin_fmaf(bv[kb][e >> 2][e & 3], kLog2e, sacc[kb][e]);
+                } else {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int key = key_of(j0, kb, e, lh);
+                            if (key < xt.bias_cols) sacc[kb][e] = __builtin_fmaf(xt.bias_row[key], kLog2e, sacc[kb][e]);
+                        }
+                }
             }
+            // hidden keys as set bits, this lane half's keys first: accumulator element e of block kb is key
+            // 32 kb + 4 lh + c with c = 8 (e / 4) + e % 4, and bit c moved to the sign position blanks the score
+            const unsigned h0 = ~(xt.kw0 >> (4 * lh)), h1 = ~(xt.kw1 >> (4 * lh));
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float score = sacc[kb][e];
+                    const int c = 8 * (e >> 2) + (e & 3);
+                    sacc[kb][e] = blank_outside(score, d0 + 32 * kb + c, top, static_cast<int>((kb ? h1 : h0) << (31 - c)));
+                }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float score = sacc[kb][e];
+                    sacc[kb][e] = blank_outside(score, d0 + 32 * kb + 8 * (e >> 2) + (e & 3), top);
+                }
+        }
     }
     // Row sum of the tile. Up to head_dim 96 the key step is bound by its VALU instructions, and the sum is taken from the
     // packed 16-bit P (one v_dot2c per pair against (1, 1), FP32 accumulation: half the instructions, and the denominator
     // sums exactly the values the PV product uses; measured 4 % faster at head_dim 40 and 72). From 112 on the matrix
     // pipe is the busier unit and the same change measured 6 % slower, so there the FP32 exponentials are added.
-    constexpr bool PAIR_SUM = HeadGeo<D>::VB < 4;
+    // (not in the XTRA instances: their denominators are an output, from which the attention map is rebuilt in FP32, so they
+    // sum the exponentials before the rounding to 16 bits.)
+    constexpr bool PAIR_SUM = HeadGeo<D>::VB < 4 && !XTRA;
     auto exponentiate = [&]() -> float {
         float s0 = 0.f, s1 = 0.f;
         if (PSCALE && prefix.on) {
@@ -573,6 +622,17 @@ __device__ __forceinline__ void softmax_tile_rel(f32x16 (&sacc)[2], typename Mma
         ls = exponentiate();
     }
     st.l += ls;
+}
+
+// 1 / l for a row with visible keys, 0 for a row without any (its output is zero, src/dit/common.cpp:293). The value is made
+// opaque to the optimiser on purpose: the library is compiled with -fno-honor-nans, under which O * select(l > 0, 1 / l, 0)
+// may be folded on the assumption that O is never NaN. A row whose scores were not finite has O = NaN and l = NaN and must
+// come out NaN (src/dit/common.cpp:269-305 makes it so); the hardware multiply delivers that (NaN * 0 = NaN) as long as it
+// is executed, whichever way the comparison on a NaN falls.
+__device__ __forceinline__ float row_inverse(float l_tot) {
+    float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    asm volatile("" : "+v"(inv));
+    return inv;
 }
 
 // Normalised output rows of one wavefront into the LDS staging area (row-major, O_STRIDE).

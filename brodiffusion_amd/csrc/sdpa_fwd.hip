@@ -167,7 +167,7 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
     }
 
     const float l_tot = exchange_sum(st.l);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const float inv = row_inverse(l_tot);
     // base-2 log of the row's denominator in exponent units: p(key) = exp2(score * scale_log2 [+ bias * log2 e] - lse);
     // +inf for a row without visible keys, so that every p is 0
     if (p.lse && qvalid && lh == 0)
@@ -178,52 +178,62 @@ __global__ void __launch_bounds__(kThreads4, (D > 128 ? 1 : 2)) sdpa_fwd_kernel(
 }
 
 // ───────────────────────── short key sequences (cross attention) ─────────────────────────
-// When all keys of a (batch, head) fit in LDS next to one query tile (cross attention to a text prompt: 77 to ~300
-// keys), the launch is pure overhead in the kernels above: every work group pays the prologue (Q staged, first K/V
-// tiles awaited) and the epilogue for a handful of key steps, and all work groups hit memory at the same moments.
-// Here a work group of 8 wavefronts loads the K and V of its (batch, head) ONCE, all tiles in flight together, and
-// then walks several 256-row query tiles: the Q rows of the next tile are already on their way (held in registers)
-// while the current tile is computed, the output of a tile drains while the next is computed, and the key loop has
-// no barrier at all (K and V never change), so the two wavefronts of a SIMD overlap their MFMA and softmax phases
-// freely. Unmasked calls (kv_valid_len allowed), no RoPE, no prefix.
+// When all keys of a (batch, head) fit in LDS (cross attention to a text prompt: 77 to ~300 keys) the call moves far more
+// bytes than it multiplies (Q in, O out: ~120 FLOP per byte at 77-105 keys of head_dim 72, below the ridge of ~312), so
+// it is bound by HBM and by fixed costs, and the kernels above, whose work groups all stage, wait and drain at the same
+// moments, are all prologue and epilogue. Here a work group of 8 wavefronts loads the K and V of its (batch, head) ONCE
+// (only the tiles below the batch item's valid length, all loads in flight together), meets at one barrier, and from
+// then on every wavefront is on its own: it walks 32-row query units, staging each through a private LDS slice (the
+// unit's rows are fetched with full-row coalescing one unit ahead, the output leaves the same way), so no barrier stands
+// in the key loop or between units and the eight wavefronts drift apart: while some wait for their rows, others
+// multiply, and the memory pipe sees a steady stream instead of bursts. Unmasked calls (kv_valid_len and a 0/1 key mask
+// allowed), no RoPE, no prefix. Same tile arithmetic as the 128-row kernel: bit-identical results.
 constexpr int kShortMaxTiles = 5;   // 320 keys
-template <int D> constexpr int shortkv_lds_bytes(int n_kt) {
+template <int D> constexpr int shortkv_lds_bytes(int n_kt, bool with_mask) {
     using G = HeadGeo<D>;
-    return 256 * G::O_STRIDE + n_kt * (G::K_BYTES + G::V_BYTES);
+    return 256 * G::O_STRIDE + n_kt * (G::K_BYTES + G::V_BYTES + (with_mask ? kBN * 4 : 0));
 }
 
 template <typename T, int D>
-__global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDev p, int n_kt, int n_strip, int strips_per_head) {
+__global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDev p, int n_kt, int units_per_group, int groups_per_head) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
-    constexpr int BM = 256;
-    constexpr int Q_BYTES = BM * G::O_STRIDE;
+    constexpr int UM = 32;                         // query rows of a unit (one wavefront)
+    constexpr int SLICE = UM * G::O_STRIDE;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    unsigned char* const Qs = smem;
-    unsigned char* const Kall = smem + Q_BYTES;
-    unsigned char* const Vall = Kall + n_kt * G::K_BYTES;
 
     const int logical = logical_block(p.n_blocks);
     if (logical < 0) return;
-    const int bh = logical / strips_per_head;
-    const int strip = logical - bh * strips_per_head;
+    const int bh = logical / groups_per_head;
+    const int grp = logical - bh * groups_per_head;
     const int h = bh % p.H, b = bh / p.H;
     const int hk = h / p.kv_group;
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, lq = lane & 31, lh = lane >> 5;
+    unsigned char* const Qs = smem + wave * SLICE;            // this wavefront's staging slice
+    unsigned char* const Kall = smem + 8 * SLICE;
+    unsigned char* const Vall = Kall + n_kt * G::K_BYTES;
+    float* const Mall = reinterpret_cast<float*>(Vall + n_kt * G::V_BYTES);
     const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
     T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D;
 
-    // ── Q rows of a tile: fetched with full-row coalescing into registers, stored to LDS one tile later ──
+    // keys of this batch item (uniform): only the tiles that hold one are loaded and multiplied
+    int kv_len = p.Lk;
+    if (p.kv_valid_len) kv_len = min(kv_len, max(p.kv_valid_len[b], 0));
+    kv_len = __builtin_amdgcn_readfirstlane(kv_len);
+    const int n_kt_b = (kv_len + kBN - 1) / kBN;
+
+    // ── a unit's Q rows: fetched with full-row coalescing into registers, stored to the slice when the unit's turn comes ──
     constexpr int CPRK = G::DK / 8;
-    constexpr int NQ = (BM * CPRK + kThreads8 - 1) / kThreads8;
+    constexpr int NQ = UM * CPRK / 64;
+    static_assert(UM * CPRK % 64 == 0, "a unit's chunks divide among the lanes");
     u32x4 qraw[NQ];
     auto q_issue = [&](int q0) {
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-            const int idx = min(tid + kThreads8 * i, BM * CPRK - 1);
+            const int idx = lane + 64 * i;
             const int row = idx / CPRK, cc = min(idx - row * CPRK, G::CPR - 1);
             qraw[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(min(q0 + row, p.Lq - 1)) * p.q_rs + cc * 8);
         }
@@ -231,28 +241,37 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
     auto q_store = [&](int q0) {
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-            const int idx = tid + kThreads8 * i;
+            const int idx = lane + 64 * i;
             const int row = idx / CPRK, cc = idx - row * CPRK;
             u32x4 v = qraw[i];
             if (q0 + row >= p.Lq || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
-            if (idx < BM * CPRK) *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
+            *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
         }
     };
-    const int qt_begin = strip * n_strip;
-    const int qt_end = min(qt_begin + n_strip, p.n_q_tiles);
-    q_issue(qt_begin * BM);
+    // LDS traffic of one wavefront is executed in order; the fences keep the compiler from reordering around them
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    const int n_units = (p.Lq + UM - 1) / UM;
+    const int u_end = min((grp + 1) * units_per_group, n_units);
+    int u = grp * units_per_group + wave;
+    if (u < u_end) q_issue(u * UM);
 
-    // ── all K and V tiles of this (batch, head): every load is issued before the first is stored ──
+    // ── the K and V tiles of this (batch, head) and the key-mask values: every load is issued before the first is stored ──
     {
         constexpr int NLD = (G::NCH + kThreads8 - 1) / kThreads8;
         const unsigned char* const k_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D);
         const unsigned char* const v_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D);
         const unsigned k_rsb = static_cast<unsigned>(p.k_rs) * 2u, v_rsb = static_cast<unsigned>(p.v_rs) * 2u;
         u32x4 kreg[kShortMaxTiles][NLD], vreg[kShortMaxTiles][NLD];
+        float mval = 0.f;
+        if (p.key_mask && tid < n_kt_b * kBN && tid < kv_len) mval = p.key_mask[b * p.key_mask_bs + tid];
 #pragma unroll
         for (int t = 0; t < kShortMaxTiles; ++t) {
-            if (t < n_kt) {
-                const int last = min(p.Lk - t * kBN, kBN) - 1;   // rows past the last key repeat it and are stored as zeros
+            if (t < n_kt_b) {
+                const int last = min(kv_len - t * kBN, kBN) - 1;   // rows past the last key repeat it and are stored as zeros
 #pragma unroll
                 for (int i = 0; i < NLD; ++i) {
                     const int idx = min(tid + kThreads8 * i, G::NCH - 1);
@@ -263,11 +282,12 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
                 }
             }
         }
-        zero_pads<D, kThreads8>(Kall, Vall, G::K_BYTES, G::V_BYTES, n_kt, tid);
+        zero_pads<D, kThreads8>(Kall, Vall, G::K_BYTES, G::V_BYTES, n_kt_b, tid);
+        if (p.key_mask && tid < n_kt * kBN) Mall[tid] = mval;
 #pragma unroll
         for (int t = 0; t < kShortMaxTiles; ++t) {
-            if (t < n_kt) {
-                const int nvalid = p.Lk - t * kBN;
+            if (t < n_kt_b) {
+                const int nvalid = kv_len - t * kBN;
 #pragma unroll
                 for (int i = 0; i < NLD; ++i) {
                     const int idx = tid + kThreads8 * i;
@@ -281,48 +301,47 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
             }
         }
     }
+    __syncthreads();   // K, V and the mask values are in place: the only barrier of the kernel
 
     const float cl2 = p.scale_log2;
     const float lazy_raw = kLazyLog2 / cl2;
-    for (int qt = qt_begin; qt < qt_end; ++qt) {
-        const int q0 = qt * BM;
+    for (; u < u_end; u += 8) {
+        const int q0 = u * UM;
         q_store(q0);
-        __syncthreads();   // Q tile (and, the first time, K and V) visible to all wavefronts
+        wave_sync();
         V8 qf[G::KC];
-        read_q_frags<T, D>(qf, Qs, wave * 32 + lq, lh);
-        __syncthreads();   // the staging area is free again
-        if (qt + 1 < qt_end) q_issue(q0 + BM);
+        read_q_frags<T, D>(qf, Qs, lq, lh);
+        wave_sync();       // the slice is free again (it takes the output next)
+        if (u + 8 < u_end) q_issue(q0 + 8 * UM);
 
-        const int qrow = q0 + wave * 32 + lq;
-        const bool qvalid = qrow < p.Lq;
-        int lo, hi;
-        row_interval(p, b, qrow, qvalid, lo, hi);
-        const WaveExtent we = wave_extent(lo, hi);
         f32x16 oacc[G::VB];
 #pragma unroll
         for (int vb = 0; vb < G::VB; ++vb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) oacc[vb][e] = 0.f;
         SoftmaxState st;
-        for (int t = 0; t < n_kt; ++t) {
+        for (int t = 0; t < n_kt_b; ++t) {
             const int j0 = t * kBN;
-            if (j0 < we.hi_max && j0 + kBN > we.lo_min) {
-                const unsigned char* Ks = Kall + t * G::K_BYTES;
-                const unsigned char* Vs = Vall + t * G::V_BYTES;
-                f32x16 sacc[2];
-                V8 pf[4];
-                mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
-                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, p.Lk));
-                softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, lo, min(hi, p.Lk), lh, nullptr);
-                mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
-            }
+            const unsigned char* Ks = Kall + t * G::K_BYTES;
+            const unsigned char* Vs = Vall + t * G::V_BYTES;
+            f32x16 sacc[2];
+            V8 pf[4];
+            mfma_stream<T, D, false, true>(Vs, Ks, pf, qf, oacc, sacc, lane);
+            const bool interior = j0 + kBN <= kv_len && p.key_mask == nullptr;
+            softmax_tile<T, D>(sacc, pf, oacc, st, cl2, lazy_raw, !interior, j0, 0, kv_len, lh, p.key_mask ? Mall + j0 : nullptr);
+            mfma_stream<T, D, true, false>(Vs, Ks, pf, qf, oacc, sacc, lane);
         }
         const float l_tot = exchange_sum(st.l);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        stage_output<T, D>(Qs, wave * 32 + lq, lh, oacc, inv);
-        __syncthreads();
-        write_output<T, D, kThreads8>(Qs, o_base, p.o_rs, q0, p.Lq, BM, tid);
-        __syncthreads();   // staged rows are read before the next tile's Q overwrites them
+        const float inv = row_inverse(l_tot);
+        stage_output<T, D>(Qs, lq, lh, oacc, inv);
+        wave_sync();
+        for (int idx = lane; idx < UM * G::CPR; idx += 64) {
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (q0 + row < p.Lq)
+                *reinterpret_cast<u32x4*>(o_base + static_cast<long>(q0 + row) * p.o_rs + cc * 8) =
+                    *reinterpret_cast<const u32x4*>(Qs + row * G::O_STRIDE + cc * 16);
+        }
+        wave_sync();       // the staged rows are read before the next unit's Q overwrites them
     }
 }
 
@@ -342,8 +361,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
 // operand suffice.
 // DENSE: as in the DMA form below (no mask, no prefix, whole key tiles only); instantiated for head_dim up to 64, where
 // it measures 2-3 % faster (at 80 the compiler's allocation of that instance goes wrong: twice as slow).
-template <typename T, int D, bool ROPE_K, bool DENSE = false>
+// XTRA: key mask, logit bias and softmax denominators (see sdpa_fwd_pp_dma_kernel).
+template <typename T, int D, bool ROPE_K, bool DENSE = false, bool XTRA = false>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev p) {
+    static_assert(!XTRA || (!DENSE && !ROPE_K), "key mask, bias and denominators belong to the general form");
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
     constexpr int BM = 256;
@@ -397,6 +418,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     }
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
     const int n_tiles = plan.n_tiles;
+    // XTRA: visibility words of the plan's tiles behind the tile buffers (visible after the barrier that ends the prologue)
+    const unsigned long long* const kbits = (XTRA && p.key_mask) ? reinterpret_cast<const unsigned long long*>(smem + p.kbits_off) : nullptr;
+    if constexpr (XTRA) build_key_bits(p, plan, b, smem + p.kbits_off, wave, lane);
+    const float* const bias_row = (XTRA && p.bias && qvalid && qrow >= p.bias_q0) ? p.bias + static_cast<long>(qrow - p.bias_q0) * p.bias_rs : nullptr;
+    TileExtra xt;
 
     f32x16 oacc[G::VB];
 #pragma unroll
@@ -468,11 +494,26 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
                     return;
                 }
             }
-            if (!DENSE && tile_active(tt)) {
+            if constexpr (XTRA) {
+                xt = TileExtra();
+                if (kbits) {
+                    const unsigned long long w = kbits[min(max(tt, 0), max(n_tiles - 1, 0))];
+                    xt.kw0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(w));
+                    xt.kw1 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(w >> 32));
+                }
+                xt.bias_cols = p.bias_cols;
+            }
+            if (!DENSE && tile_active(tt) && (!XTRA || (xt.kw0 | xt.kw1) != 0u)) {
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
-                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh);
+                bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
+                if constexpr (XTRA) {
+                    const bool biased = p.bias != nullptr && j0 < p.bias_cols;
+                    interior = interior && (xt.kw0 & xt.kw1) == ~0u && !biased;
+                    xt.bias_row = biased ? bias_row : nullptr;
+                    xt.bias_vec = p.bias_vec_ok && (j0 & 3) == 0 && j0 + kBN <= p.bias_cols;
+                }
+                softmax_tile_rel<T, D, false, XTRA>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh, PrefixScale(), xt);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -501,7 +542,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_kernel(const SdpaDev
     }
 
     const float l_tot = exchange_sum(st.l);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const float inv = row_inverse(l_tot);
+    if constexpr (XTRA) {
+        if (p.lse && qvalid && lh == 0)
+            p.lse[(static_cast<long>(b) * p.H + h) * p.Lq + qrow] = l_tot > 0.f ? __builtin_amdgcn_logf(l_tot) - st.neg_ref : __builtin_huge_valf();
+    }
     stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
     __syncthreads();
     write_output<T, D, kThreads8>(smem, o_base, p.o_rs, q0, p.Lq, BM, tid);
@@ -559,10 +604,13 @@ __device__ __forceinline__ int swz(int row) { return 4 * (row & 3) + ((row >> 2)
 // wavefront sees it whole) drop out of the kernel, and with them their registers: measured 6 % faster at head_dim 128
 // and 8 % at 72 than the general form on the same dense call.
 // PSCALE: the general form with the prefix-KV dial (factors on the rows of the cached prefix) in its softmax.
-template <typename T, int D, bool SPLIT, bool DENSE = false, bool PSCALE = false>
+// XTRA: the general form with a key mask (one visibility bit per key, 64-bit words per key tile built once per work group
+// in LDS behind the rings), an additive logit bias and the softmax denominators as an output (traced attention).
+template <typename T, int D, bool SPLIT, bool DENSE = false, bool PSCALE = false, bool XTRA = false>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const SdpaDev p) {
     static_assert(!(SPLIT && DENSE), "the split launch clips key ranges per part");
     static_assert(!PSCALE || (!SPLIT && !DENSE), "the dial belongs to the general form");
+    static_assert(!XTRA || (!SPLIT && !DENSE && !PSCALE), "key mask, bias and denominators belong to the general form");
     using G = HeadGeo<D>;
     using DG = DmaGeo<D>;
     using V8 = typename Mma<T>::v8;
@@ -669,6 +717,10 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     }
     const TilePlan plan(g_lo == 0x7fffffff ? 0 : g_lo, kv_stop, p.Lp);
     const int n_tiles = plan.n_tiles;
+    // XTRA: visibility words of the plan's tiles (made visible to all wavefronts by the barrier that ends the prologue)
+    const unsigned long long* const kbits = (XTRA && p.key_mask) ? reinterpret_cast<const unsigned long long*>(smem + p.kbits_off) : nullptr;
+    if constexpr (XTRA) build_key_bits(p, plan, b, smem + p.kbits_off, wave, lane);
+    const float* const bias_row = (XTRA && p.bias && qvalid && qrow >= p.bias_q0) ? p.bias + static_cast<long>(qrow - p.bias_q0) * p.bias_rs : nullptr;
 
     f32x16 oacc[G::VB];
 #pragma unroll
@@ -762,6 +814,9 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
             vaddr[vb][hh] = DG::VOFF + row * DG::ROWB + ((DG::SWZ ? (chunk ^ swz(row)) : chunk) << 4) + 8 * (j4 & 1);
         }
 
+    static_assert(G::DK == D || G::DK - D == 8, "the pad of a K row is the upper lane half of its last fragment");
+    const unsigned pad_keep = lh ? 0u : ~0u;
+
     f32x16 sacc[2];
     V8 pf[4];
 #pragma unroll
@@ -782,6 +837,17 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         constexpr int KD = ((S + 2) % 3) * DG::TILE, VD = DG::VOFF + ((S + 1) % 3) * DG::TILE;
         const bool load_k = t + 3 < n_tiles, load_v = t + 2 < n_tiles;
         int issued = 0;
+        // XTRA: the visibility word of the tile whose softmax this wavefront runs in this step, fetched here, ahead of this
+        // step's DMA instructions (an LDS read behind them would wait for them to land)
+        TileExtra xt;
+        if constexpr (XTRA) {
+            if (kbits) {
+                const unsigned long long w = kbits[min(max(grp == 1 ? t : t + 1, 0), max(n_tiles - 1, 0))];
+                xt.kw0 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(w));
+                xt.kw1 = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(w >> 32));
+            }
+            xt.bias_cols = p.bias_cols;
+        }
         auto softmax_of = [&](int tt) {
             if constexpr (DENSE) {
                 if (tt >= 0 && tt < n_tiles) {
@@ -789,12 +855,18 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                     return;
                 }
             }
-            if (!DENSE && tile_active(tt)) {
+            if (!DENSE && tile_active(tt) && (!XTRA || (xt.kw0 | xt.kw1) != 0u)) {
                 const int j0 = plan.j0(tt);
                 const int lim = plan.limit(tt);
-                const bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
-                softmax_tile_rel<T, D, PSCALE>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh,
-                                               PSCALE ? prefix_scale_of(p, plan.in_prefix(tt)) : PrefixScale());
+                bool interior = (j0 >= we.lo_max) && (j0 + kBN <= min(we.hi_min, lim));
+                if constexpr (XTRA) {
+                    const bool biased = p.bias != nullptr && j0 < p.bias_cols;
+                    interior = interior && (xt.kw0 & xt.kw1) == ~0u && !biased;
+                    xt.bias_row = biased ? bias_row : nullptr;
+                    xt.bias_vec = p.bias_vec_ok && (j0 & 3) == 0 && j0 + kBN <= p.bias_cols;
+                }
+                softmax_tile_rel<T, D, PSCALE, XTRA>(sacc, pf, oacc, st, !interior, dead_row, j0, lo, min(hi, lim), lh,
+                                                     PSCALE ? prefix_scale_of(p, plan.in_prefix(tt)) : PrefixScale(), xt);
             } else {
                 // nothing visible to this wavefront in that tile: the next PV pass must add zero
 #pragma unroll
@@ -837,7 +909,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
                     return __builtin_bit_cast(V8, a);
                 } else {
                     const int kb = i / G::KC, c = i % G::KC;
-                    const u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * DG::ROWB + kaddr[c]);
+                    u32x4 a = *reinterpret_cast<const u32x4*>(smem + KS + 32 * kb * DG::ROWB + kaddr[c]);
+                    // the upper lane half of the last fragment holds the first elements of the NEXT key row where the head
+                    // dimension is padded (unpadded rows): blanked, because Q's zero pad does not silence a NaN or an
+                    // infinity there, and the next row may be one that this query must not see
+                    if (G::DK > D && c == G::KC - 1) a &= pad_keep;
                     return __builtin_bit_cast(V8, a);
                 }
             };
@@ -906,7 +982,13 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
     }
 
     const float l_tot = exchange_sum(st.l);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const float inv = row_inverse(l_tot);
+    if constexpr (XTRA) {
+        // base-2 log of the row's denominator in exponent units: p(key) = exp2(score * scale_log2 [+ bias * log2 e] - lse);
+        // +inf for a row without visible keys, so that every p is 0
+        if (p.lse && qvalid && lh == 0)
+            p.lse[(static_cast<long>(b) * p.H + h) * p.Lq + qrow] = l_tot > 0.f ? __builtin_amdgcn_logf(l_tot) - st.neg_ref : __builtin_huge_valf();
+    }
     stage_output<T, D>(smem, wave * 32 + lq, lh, oacc, inv);
     __syncthreads();
     if constexpr (!SPLIT) {
@@ -957,10 +1039,19 @@ __global__ void __launch_bounds__(256) sdpa_combine_kernel(const SdpaDev p) {
         if (idx >= BM * CPR) return;
         const int row = idx / CPR, cc = idx - row * CPR;
         if (q0 + row >= p.Lq) return;
+        // a part without visible keys has denominator 0 and is skipped; one whose denominator is NaN (a non-finite score)
+        // must not be: it makes the row NaN, as it would in an unsplit launch. Hence the test on the bits.
+        // (the bits pass through an empty asm statement: left visible, the optimiser turns the integer test back into a
+        //  floating-point comparison that is false for a NaN, which -fno-honor-nans entitles it to)
+        auto empty = [](float l) {
+            unsigned bits = __builtin_bit_cast(unsigned, l);
+            asm volatile("" : "+v"(bits));
+            return (bits & 0x7fffffffu) == 0u;
+        };
         float ref = kNegInf;
         for (int k = 0; k < n_parts; ++k) {
             const float* stat = reinterpret_cast<const float*>(slots + k * SplitGeo::slot_bytes(D) + static_cast<long>(BM) * D * 2);
-            if (stat[BM + row] > 0.f) ref = fmaxf(ref, stat[row]);
+            if (!empty(stat[BM + row])) ref = fmaxf(ref, stat[row]);
         }
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float wsum = 0.f;
@@ -968,14 +1059,14 @@ __global__ void __launch_bounds__(256) sdpa_combine_kernel(const SdpaDev p) {
             const unsigned char* slot = slots + k * SplitGeo::slot_bytes(D);
             const float* stat = reinterpret_cast<const float*>(slot + static_cast<long>(BM) * D * 2);
             const float l = stat[BM + row];
-            if (!(l > 0.f)) continue;
+            if (empty(l)) continue;
             const float w = l * __builtin_amdgcn_exp2f(stat[row] - ref);
             wsum += w;
             const t8 o = *reinterpret_cast<const t8*>(slot + (static_cast<long>(row) * D + cc * 8) * 2);
 #pragma unroll
             for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(w, static_cast<float>(o[e]), acc[e]);
         }
-        const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+        const float inv = row_inverse(wsum);
         t8 out;
 #pragma unroll
         for (int e = 0; e < 8; ++e) out[e] = static_cast<T>(acc[e] * inv);
@@ -1055,24 +1146,27 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     // two wavefronts per SIMD and stays on the 128-row kernel.
     const long tiles256 = static_cast<long>(p.B) * p.H * ((p.Lq + 255) / 256);
     const int choice = sdpa_kernel_choice();
-    // calls with a key mask stay on the 128-row kernel, which stages the mask tile in LDS
-    // ... and so do calls with a logit bias or a request for the softmax denominators
-    // ... and so do calls with the prefix-KV dial, unless the DMA kernel (which has an instance for it) takes them
+    // calls with a key mask, a logit bias or a request for the softmax denominators take the XTRA instances of the 256-row
+    // kernels (visibility words of all key tiles in LDS behind the tile buffers), unless K is rotated tile by tile, the
+    // prefix-KV dial is on as well, or the key sequence is too long for the words to fit: then the 128-row kernel
+    const bool xtra = p.key_mask != nullptr || p.bias != nullptr || p.lse != nullptr;
+    const long kbits_bytes = p.key_mask ? 8L * ((p.Lk + kBN - 1) / kBN + 2) : 0;
+    const bool xtra_ok = !xtra || (!rope_k && !p.prefix_scaled && kbits_bytes <= 32 * 1024);
+    // calls with the prefix-KV dial stay on the 128-row kernel unless the DMA kernel (which has an instance for it) takes them
     const bool dial_ok = !p.prefix_scaled || (dma_kernel_available<D>() && !rope_k && choice != 3);
-    const bool pingpong = D <= 128 && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr && dial_ok &&
-                          (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
+    const bool pingpong = D <= 128 && xtra_ok && dial_ok && (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
     // short key sequences whose K and V fit in LDS next to a query tile: one work group walks several query tiles
     const int n_kt = (p.Lk + kBN - 1) / kBN;
-    if (D <= 128 && choice == 0 && p.mask_mode == MI_MASK_NONE && p.key_mask == nullptr && p.bias == nullptr && p.lse == nullptr &&
+    if (D <= 128 && choice == 0 && p.mask_mode == MI_MASK_NONE && p.bias == nullptr && p.lse == nullptr &&
         p.Lp == 0 && !rope_k && p.cos_q == nullptr && n_kt >= 1 && n_kt <= kShortMaxTiles && tiles256 >= n_cu &&
-        shortkv_lds_bytes<D>(n_kt) <= 160 * 1024) {
+        shortkv_lds_bytes<D>(n_kt, p.key_mask != nullptr) <= 160 * 1024) {
         if constexpr (D <= 128) {
             p.n_q_tiles = (p.Lq + 255) / 256;
-            const int n_strip = static_cast<int>(tiles256 / n_cu);   // query tiles per work group: about one work group per CU
+            const int n_strip = static_cast<int>(tiles256 / n_cu);   // 256 query rows per work group and round: about one work group per CU
             const int strips_per_head = (p.n_q_tiles + n_strip - 1) / n_strip;
             p.n_blocks = p.B * p.H * strips_per_head;
-            hipLaunchKernelGGL((sdpa_shortkv_kernel<T, D>), dim3(grid_blocks(p)), dim3(kThreads8), shortkv_lds_bytes<D>(n_kt), stream, p,
-                               n_kt, n_strip, strips_per_head);
+            hipLaunchKernelGGL((sdpa_shortkv_kernel<T, D>), dim3(grid_blocks(p)), dim3(kThreads8), shortkv_lds_bytes<D>(n_kt, p.key_mask != nullptr), stream, p,
+                               n_kt, 8 * n_strip, strips_per_head);
             const hipError_t e = hipGetLastError();
             if (e != hipSuccess) return fail("sdpa_fwd launch: %s", hipGetErrorString(e));
             return 0;
@@ -1083,7 +1177,21 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
         p.n_blocks = static_cast<int>(tiles256);
         const dim3 grid(grid_blocks(p)), block(kThreads8);
         if constexpr (D <= 128) {
-            if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
+            if (xtra) {
+                const bool dma = dma_kernel_available<D>() && sdpa_kernel_choice() != 3;
+                if constexpr (dma_kernel_available<D>()) {
+                    if (dma) {
+                        p.kbits_off = DmaGeo<D>::lds_bytes();
+                        hipLaunchKernelGGL((sdpa_fwd_pp_dma_kernel<T, D, false, false, false, true>), grid, block,
+                                           DmaGeo<D>::lds_bytes() + kbits_bytes, stream, p);
+                    }
+                }
+                if (!dma) {
+                    p.kbits_off = lds_bytes_8<D>();
+                    hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, false, false, true>), grid, block, lds_bytes_8<D>() + kbits_bytes, stream, p);
+                }
+            }
+            else if (rope_k) hipLaunchKernelGGL((sdpa_fwd_pp_kernel<T, D, true>), grid, block, lds_bytes_8<D>(), stream, p);
             else if (dma_kernel_available<D>() && sdpa_kernel_choice() != 3) {
                 if constexpr (dma_kernel_available<D>()) {
                     // whole key tiles only; a cached prefix may come first if it is whole tiles too and laid out like K / V

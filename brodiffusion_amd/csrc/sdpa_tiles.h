@@ -63,6 +63,23 @@ struct TilePlan {
     __device__ __forceinline__ int limit(int t) const { return t < n_pre ? pre_hi : fr_hi; }
 };
 
+// Visibility words of a plan's key tiles from a key mask (a key is hidden where the mask holds +0 or -0): bit i of word t
+// says whether key i of tile t is visible; keys at or past the tile's segment limit count as hidden. Built by the
+// wavefronts of a work group in turn (one ballot per tile) into LDS at `dst`; the caller's next barrier publishes them.
+__device__ __forceinline__ void build_key_bits(const SdpaDev& p, const TilePlan& plan, int b, unsigned char* dst, int wave, int lane,
+                                               int n_waves = 8) {
+    if (!p.key_mask) return;
+    const float* const km = p.key_mask + b * p.key_mask_bs;
+    unsigned long long* const out = reinterpret_cast<unsigned long long*>(dst);
+    for (int t = wave; t < plan.n_tiles; t += n_waves) {
+        const int j = plan.j0(t) + lane;
+        unsigned bits = 0;
+        if (j < plan.limit(t)) bits = __builtin_bit_cast(unsigned, km[j]) & 0x7fffffffu;
+        const unsigned long long w = __ballot(bits != 0u);
+        if (lane == 0) out[t] = w;
+    }
+}
+
 // Walks the tiles of one operand (K or V) in order, keeping the tile's base pointer, row stride and
 // the number of rows left in the current segment (prefix, then fresh) in scalar registers.
 struct TileCursor {

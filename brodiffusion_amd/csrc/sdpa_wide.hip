@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(kWideThreads) sdpa_wide_kernel(const SdpaDev p
     }
 
     const float l_tot = exchange_sum(st.l);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const float inv = row_inverse(l_tot);
     {
         typedef T t4 __attribute__((ext_vector_type(4)));
 #pragma unroll

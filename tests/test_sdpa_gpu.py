@@ -104,7 +104,7 @@ def test_key_mask_equals_trimmed(oracle, kernel_choice, dtype, d):
         assert_close(ref, to_np(o_len[b]), dtype, "kv_valid_len")
         assert_close(ref, to_np(o_mask[b]), dtype, "d_mask")
         o_trim = bd.flash_attention_forward(dq[b], dk[b, :valid[b]], dv[b, :valid[b]], None, H, False)
-        # calls with a 0/1 mask always run on the 128-row kernel, the others on the chosen one
+        # (the 256-row kernels take a 0/1 mask in an instance of their own, whose softmax blanks keys bit by bit)
         assert_same(o_trim, o_len[b], True, "trimmed vs kv_valid_len")
         assert_same(o_trim, o_mask[b], kernel_choice == "rows128", "trimmed vs d_mask")
 
@@ -119,6 +119,41 @@ def test_scattered_key_mask_and_empty_mask(oracle):
     assert_close(oracle.sdpa(q, k, v, H, key_mask=m), to_np(out), dtype)
     out0 = bd.flash_attention_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), torch.zeros(Lk, device="cuda"), H, False)
     assert not to_np(out0).any()
+
+
+@pytest.mark.parametrize("dtype,d", [("bf16", 128), ("fp16", 40), ("bf16", 72), ("fp16", 96), ("bf16", 64)])
+def test_key_mask_with_other_masks(oracle, dtype, d):
+    """A scattered 0/1 key mask (per batch item) together with a causal window, with a valid length, and over a cached
+    prefix (the mask is indexed over [prefix ; fresh]): every kernel form against the checker. Tiles that the mask hides
+    entirely, rows whose visible keys are all masked (zeros), and a mask of -0.0 entries (hidden like +0.0)."""
+    B, H, Lq, Lk = 2, 2, 200, 330
+    q = randn(81, (B, Lq, H * d), dtype); k = randn(82, (B, Lk, H * d), dtype); v = randn(83, (B, Lk, H * d), dtype)
+    rng = np.random.default_rng(d)
+    m = (rng.uniform(size=(B, Lk)) > 0.4).astype(np.float32)
+    m[0, 128:192] = 0                                # a whole key tile hidden in batch item 0
+    m[1, :70] = 0                                    # the first tile and a bit more hidden in batch item 1
+    m[1, 100] = -0.0
+    m[1, 101] = 1.0
+    dq, dk, dv, dm = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), torch.from_numpy(m).cuda()
+    window = 90
+    lo, hi = oracle.rows_causal(Lq, Lk, window=window)
+    out = bd.sdpa_forward(dq, dk, dv, H, key_mask=dm, mask=bd.SdpaMask.causal(Lk - Lq, window))
+    for b in range(B):
+        assert_close(oracle.sdpa(q[b], k[b], v[b], H, key_mask=m[b], row_lo=lo, row_hi=hi), to_np(out[b]), dtype, f"mask + window, batch {b}")
+    vl = torch.tensor([300, 150], dtype=torch.int32, device="cuda")
+    out = bd.sdpa_forward(dq, dk, dv, H, key_mask=dm, kv_valid_len=vl)
+    for b, n in enumerate((300, 150)):
+        assert_close(oracle.sdpa(q[b], k[b, :n], v[b, :n], H, key_mask=m[b, :n]), to_np(out[b]), dtype, f"mask + valid_len, batch {b}")
+    # cached prefix of 100 rows (a partly filled prefix tile), the other 230 keys fresh; one mask row shared by the batch
+    out = bd.sdpa_forward(dq, dk[:, 100:].contiguous(), dv[:, 100:].contiguous(), H, k_prefix=dk[:, :100].contiguous(),
+                          v_prefix=dv[:, :100].contiguous(), key_mask=dm[0])
+    for b in range(B):
+        assert_close(oracle.sdpa(q[b], k[b], v[b], H, key_mask=m[0]), to_np(out[b]), dtype, f"mask over prefix + fresh, batch {b}")
+    # early rows of batch item 1 see only masked keys under a causal mask without offset: zeros
+    out = to_np(bd.sdpa_forward(dq[1, :60], dk[1], dv[1], H, key_mask=dm[1], mask=bd.SdpaMask.causal(0)))
+    lo, hi = oracle.rows_causal(60, Lk, q_offset=0)
+    assert_close(oracle.sdpa(q[1, :60], k[1], v[1], H, key_mask=m[1], row_lo=lo, row_hi=hi), out, dtype, "rows without visible keys")
+    assert not out.any()
 
 
 def _block_causal_case(prefix, blocks):

@@ -57,3 +57,29 @@ def test_shortkv_strided_views_and_zero_valid(oracle):
     out = bd.sdpa_forward(dq, dk, dv, H, kv_valid_len=vl, out=wide_o[:, :, :D])
     assert (out[0] == 0).all() and (wide_o[:, :, D:] == 5).all()
     assert torch.equal(out, rows128(dq.contiguous(), dk.contiguous(), dv.contiguous(), H, kv_valid_len=vl))
+
+
+@pytest.mark.parametrize("dtype,B,H,d,Lq,Lk", [("bf16", 2, 16, 72, 4096, 200), ("fp16", 2, 8, 40, 4096, 77)])
+def test_shortkv_key_mask(oracle, dtype, B, H, d, Lq, Lk):
+    """A 0/1 key mask per batch item (text padding in the middle and at the end, one whole key tile hidden) on the shape
+    that takes the short-key kernel, alone and together with a valid length: bit-equal to the 128-row kernel, sampled rows
+    against the checker."""
+    q = randn(9900 + Lq, (B, Lq, H * d), dtype)
+    k, v = randn(9901 + Lk, (B, Lk, H * d), dtype), randn(9902 + Lk, (B, Lk, H * d), dtype)
+    m = (np.random.default_rng(Lk).uniform(size=(B, Lk)) > 0.3).astype(np.float32)
+    m[0, Lk - 9:] = 0
+    if Lk > 128:
+        m[1, 64:128] = 0
+    dq, dk, dv, dm = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), torch.from_numpy(m).cuda()
+    rows = np.unique(np.concatenate([np.arange(0, Lq, 173), [31, 32, Lq - 1]])).astype(np.int32)
+    out = bd.sdpa_forward(dq, dk, dv, H, key_mask=dm)
+    assert torch.equal(out, rows128(dq, dk, dv, H, key_mask=dm))
+    for b in range(B):
+        ref = oracle.sdpa(q[b], k[b], v[b], H, key_mask=m[b], rows=rows)
+        assert_close(ref[rows], to_np(out[b])[rows], dtype, f"short-kv key mask, batch {b}")
+    vl = torch.tensor([Lk - 20, 70], dtype=torch.int32, device="cuda")
+    out = bd.sdpa_forward(dq, dk, dv, H, key_mask=dm, kv_valid_len=vl)
+    assert torch.equal(out, rows128(dq, dk, dv, H, key_mask=dm, kv_valid_len=vl))
+    for b, n in enumerate((Lk - 20, 70)):
+        ref = oracle.sdpa(q[b], k[b, :n], v[b, :n], H, key_mask=m[b, :n], rows=rows)
+        assert_close(ref[rows], to_np(out[b])[rows], dtype, f"short-kv key mask + valid length, batch {b}")

@@ -14,6 +14,14 @@ from helpers import assert_close, randn, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=["by_size", "rows128", "rows256", "rows256_regs"])
+def kernel_choice(request):
+    """The bias and the softmax denominators exist in the 128-row kernel and in an instance of each 256-row kernel."""
+    bd.set_sdpa_kernel_choice({"by_size": 0, "rows128": 1, "rows256": 2, "rows256_regs": 3}[request.param])
+    yield request.param
+    bd.set_sdpa_kernel_choice(0)
+
+
 def tables(oracle, txt, hp, wp, d, axes):
     cos, sin = oracle.build_axial_rope_tables(txt, hp, wp, d, axes)
     return cos, sin, torch.from_numpy(cos).cuda(), torch.from_numpy(sin).cuda()
@@ -25,7 +33,7 @@ def tables(oracle, txt, hp, wp, d, axes):
     ("fp16", 3, 64, 64, 8, 8, (16, 24, 24), True),
     ("bf16", 2, 72, 5, 20, 13, (8, 32, 32), True),        # 265 rows: ragged tiles on both axes
 ])
-def test_traced_matches_checker(oracle, dtype, H, d, txt, hp, wp, axes, with_bias):
+def test_traced_matches_checker(oracle, kernel_choice, dtype, H, d, txt, hp, wp, axes, with_bias):
     L = txt + hp * wp
     q, k, v = (randn(9400 + i, (L, H * d), dtype) for i in range(3))
     cos, sin, dcos, dsin = tables(oracle, txt, hp, wp, d, axes)
@@ -52,8 +60,9 @@ def test_traced_matches_checker(oracle, dtype, H, d, txt, hp, wp, axes, with_bia
 def test_traced_at_a_shape_whose_plain_call_splits_its_last_round(oracle, with_bias):
     """Flux at 768 px (512 text + 48 x 48 image rows, 24 heads of 128): a plain attention call of this shape cuts its last
     round of work groups along the key axis when a scratch is lent. The traced call asks for the softmax denominators
-    (and a bias), which only the 128-row kernel provides, so it must not take that route: sampled rows of the output and
-    of the map against the checker, and no split scratch is asked for."""
+    (and a bias), which the split launch does not provide, so it must not take that route (it runs on the 256-row
+    kernel's instance with bias and denominators): sampled rows of the output and of the map against the checker, and no
+    split scratch is asked for."""
     import ctypes as C
     from brodiffusion_amd import _capi as capi
     dtype, H, d, txt, hp, wp = "bf16", 24, 128, 512, 48, 48
@@ -138,7 +147,7 @@ def test_traced_errors():
     ("fp16", 256, 77, 640, 768, 8, False, False),      # level 1 (head_dim 80), plain trace
     ("bf16", 300, 50, 128, 96, 2, True, True),         # ragged sizes, bias and key mask together
 ])
-def test_cross_attention_with_attn(oracle, dtype, Lq, Lk, C, Cctx, H, with_bias, with_mask):
+def test_cross_attention_with_attn(oracle, kernel_choice, dtype, Lq, Lk, C, Cctx, H, with_bias, with_mask):
     """bt::cross_attention_forward_with_attn as src/unet_blocks.cpp:282-290 calls it: projections, attention with logit
     bias / key mask, output projection, head-averaged map."""
     x, ctx = randn(9501, (Lq, C), dtype), randn(9502, (Lk, Cctx), dtype)
