@@ -15,6 +15,7 @@
 //                 is an exact FP32 dot of z with the lane's own Q values plus one exchange between
 //                 lanes l and l^32.
 #include <algorithm>
+#include <type_traits>
 
 #include <atomic>
 
@@ -85,7 +86,9 @@ struct LinDev {
     int tokens_per_group;
     int n_chunks;   // token chunks per (batch, head)
     int n_blocks;   // work groups with work = B * H * n_chunks
+    int form;       // MI_LINEAR_ATTN_FORM_*
 };
+constexpr int kFusedMaxTokens = 1024;   // up to here the one-launch form is taken for sliced heads when the kernel is picked by size
 
 template <int D> struct LGeo {
     static constexpr int DP = (D + 31) / 32 * 32;
@@ -496,10 +499,351 @@ __global__ void __launch_bounds__(kThreads) linattn_apply_kernel(const LinDev p)
     }
 }
 
+
+// ── one launch, no hand-over: the state is split along its VALUE-channel axis ──
+// Work group (batch, head, r) owns rows [32 r, 32 r + 32) of S (value channels) and every column. Pass 1 streams all of K
+// and the 64-byte slice of V that holds its channels, giving S[32 r .. 32 r + 32, :] and the whole z (it reads all of K
+// anyway); pass 2, the same work group, streams all of Q and writes its 64-byte slice of O. Nothing is exchanged between
+// work groups: no partial states in memory, no reduction kernel, no fence, no atomics, one launch. The price is that the
+// DP / 32 work groups of a head each read K and Q; they are numbered next to each other so that they share an XCD and the
+// repeats come out of its L2.
+// Inside a work group the 8 wavefronts are independent in both passes: each walks 32-token units of its own (unit u of
+// wavefront w is tokens [32 (w + 8 u), + 32)), fetched with full-row coalescing two units ahead into two register sets
+// and staged through a private LDS slice, so no work-group barrier stands in either streaming loop and about 150 KB of
+// loads are in flight per compute unit. All vector-memory instructions in the loops are unconditional (past the end a
+// wavefront re-fetches its last unit, and a lane without an output chunk of its own repeats another lane's store), so
+// that the compiler's wait counts stay exact and a wait for the older register set does not drain the younger one.
+// Between the passes the 8 partial states meet in LDS as FP32 images and are added in a fixed order: bit-reproducible.
+// z costs one accumulator: the A operand "ones in row j" sends the token sum of K's column block j to row j of it.
+constexpr int kFusedThreads = 512;
+constexpr int kFusedWaves = kFusedThreads / 64;
+constexpr int kFU = 32;                     // tokens per unit
+
+template <int D> struct FusedGeo {
+    using G = LGeo<D>;
+    static constexpr int NS = G::NB;                                   // work groups (value-channel slices) per (batch, head)
+    static constexpr int VT_STRIDE = 64;                               // V slice tile: 32 channels, rows back to back (64 mod 128)
+    static constexpr int P1_SLICE = kFU * (G::T_STRIDE + VT_STRIDE);   // pass 1: K rows then V rows of a unit
+    static constexpr int IMG_FLOATS = 32 * G::DP + G::DP;              // 32 rows of S and z
+    static constexpr int O_STRIDE = 64 + 16;                           // pass 2: staged output rows (32 channels)
+    static constexpr int P2_SLICE = kFU * G::S_STRIDE;                 // pass 2: Q rows of a unit (the output rows reuse it)
+    static constexpr int SB_BYTES = 32 * G::S_STRIDE;                  // the slice of S as 16-bit A operand
+    static constexpr int cmax(int a, int b) { return a > b ? a : b; }
+    static constexpr int WORK_BYTES = cmax(cmax(kFusedWaves * P1_SLICE, kFusedWaves * IMG_FLOATS * 4), kFusedWaves * P2_SLICE);
+    static constexpr int LDS_BYTES = WORK_BYTES + SB_BYTES + G::DP * 4;
+    static_assert(kFU * O_STRIDE <= P2_SLICE, "the staged output fits the unit's Q slice");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
+};
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kFusedThreads, 2) linattn_fused_kernel(const LinDev p) {
+    using G = LGeo<D>;
+    using FG = FusedGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    int bh, slice;
+    {
+        LinDev q = p;
+        q.n_chunks = FG::NS;
+        if (!lin_block(q, bh, slice)) return;
+    }
+    const int b = bh / p.H, h = bh % p.H;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int lq = lane & 31, lh = lane >> 5;
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + h * D;
+    const T* const k_base = static_cast<const T*>(p.k) + b * p.k_bs + h * D;
+    const T* const v_base = static_cast<const T*>(p.v) + b * p.v_bs + h * D + 32 * slice;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + h * D + 32 * slice;
+    constexpr int VCH = 4;                                   // 16-byte chunks of a slice row
+    const int v_chunks = min(VCH, (D - 32 * slice) / 8);     // ... that exist (the last slice of a padded head is narrower)
+    const int n_units = (p.N + kFU - 1) / kFU;
+    const int last_unit = n_units - 1;
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // ───────────── pass 1: S[slice rows, :] and z over this wavefront's units ─────────────
+    unsigned char* const Kp = lds + wave * FG::P1_SLICE;
+    unsigned char* const Vp = Kp + kFU * G::T_STRIDE;
+    constexpr int NK = (kFU * G::CPR + 63) / 64;             // K loads per lane and unit
+    constexpr int NV = kFU * VCH / 64;                       // V loads per lane and unit (2)
+    if constexpr (G::DP > D) {                               // pad columns of the K rows stay zero
+        constexpr int PC = (G::DP - D) / 8;
+        for (int i = lane; i < kFU * PC; i += 64)
+            *reinterpret_cast<u32x4*>(Kp + (i / PC) * G::T_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
+    }
+    auto issue_kv = [&](u32x4 (&kreg)[NK], u32x4 (&vreg)[NV], int unit) {
+        const long n0 = static_cast<long>(min(unit, last_unit)) * kFU;
+        const long last = p.N - 1;
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int idx = min(lane + 64 * i, kFU * G::CPR - 1);
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            kreg[i] = *reinterpret_cast<const u32x4*>(k_base + min(n0 + row, last) * p.k_rs + cc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / VCH, cc = min(idx - row * VCH, v_chunks - 1);
+            vreg[i] = *reinterpret_cast<const u32x4*>(v_base + min(n0 + row, last) * p.v_rs + cc * 8);
+        }
+    };
+    auto store_kv = [&](const u32x4 (&kreg)[NK], const u32x4 (&vreg)[NV], int unit) {
+        const int n0 = unit * kFU;
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < kFU * G::CPR) {
+                u32x4 kv = relu8<T>(kreg[i]);
+                if (n0 + row >= p.N) kv = u32x4{0, 0, 0, 0};     // a token that does not exist adds nothing to S and z
+                *reinterpret_cast<u32x4*>(Kp + row * G::T_STRIDE + cc * 16) = kv;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / VCH, cc = idx - row * VCH;
+            *reinterpret_cast<u32x4*>(Vp + row * FG::VT_STRIDE + cc * 16) = cc < v_chunks ? vreg[i] : u32x4{0, 0, 0, 0};
+        }
+    };
+    auto frag = [&](const unsigned char* ptr, int stride) -> V8 {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr + 8 * stride));
+        return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    f32x16 acc[G::NB], zacc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        zacc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < G::NB; ++j) acc[j][e] = 0.f;
+    }
+    // A operand "ones in row j, zeros elsewhere": lane (row lq) holds 8 ones if lq == j. One register pair of ones per
+    // lane and a mask per block (built where it is used) instead of four operands held through the loop.
+    const unsigned one2 = (std::is_same_v<T, __bf16> ? 0x3f803f80u : 0x3c003c00u);
+    auto sel = [&](int j) -> V8 {
+        const unsigned w = lq == j ? one2 : 0u;
+        return __builtin_bit_cast(V8, u32x4{w, w, w, w});
+    };
+    const int trow = (lane & 15) >> 2;
+    const int tcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    auto multiply_unit = [&]() {
+#pragma unroll
+        for (int s2 = 0; s2 < kFU / 16; ++s2) {
+            const int r0 = 16 * s2 + 4 * lh + trow;
+            const V8 a = frag(Vp + r0 * FG::VT_STRIDE + tcol * 2, FG::VT_STRIDE);
+            V8 bk[G::NB];
+#pragma unroll
+            for (int j = 0; j < G::NB; ++j) bk[j] = frag(Kp + r0 * G::T_STRIDE + (32 * j + tcol) * 2, G::T_STRIDE);
+#pragma unroll
+            for (int j = 0; j < G::NB; ++j) {
+                acc[j] = Mma<T>::run(a, bk[j], acc[j]);
+                zacc = Mma<T>::run(sel(j), bk[j], zacc);
+            }
+        }
+    };
+    {
+        u32x4 kA[NK], vA[NV], kB[NK], vB[NV];
+        int u = wave;
+        issue_kv(kA, vA, u);
+        issue_kv(kB, vB, u + kFusedWaves);
+        // two units per turn, one way out (at the bottom): on every path set A is the older one
+        for (; u < n_units; u += 2 * kFusedWaves) {
+            store_kv(kA, vA, u);
+            wave_sync();
+            issue_kv(kA, vA, u + 2 * kFusedWaves);
+            multiply_unit();
+            wave_sync();
+            if (u + kFusedWaves < n_units) {
+                store_kv(kB, vB, u + kFusedWaves);
+                wave_sync();
+            }
+            issue_kv(kB, vB, u + 3 * kFusedWaves);
+            if (u + kFusedWaves < n_units) {
+                multiply_unit();
+                wave_sync();
+            }
+        }
+    }
+    __syncthreads();     // every wavefront is done with its K / V slice: the space takes the FP32 images
+
+    // ───────────── the 8 partial states -> one; the state to memory, the slice as A operand to LDS ─────────────
+    // (the lane id is made opaque from here on: otherwise every per-lane address of pass 2 is computed in front of pass 1
+    //  and spilled around it)
+    int lane2 = lane;
+    asm volatile("" : "+v"(lane2));
+    const int lq2 = lane2 & 31, lh2 = lane2 >> 5;
+    float* const img = reinterpret_cast<float*>(lds) + wave * FG::IMG_FLOATS;
+#pragma unroll
+    for (int j = 0; j < G::NB; ++j) {
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) img[(8 * bb + 4 * lh2 + e) * G::DP + 32 * j + lq2] = acc[j][4 * bb + e];
+    }
+    if (lh2 == 0) {
+#pragma unroll
+        for (int j = 0; j < G::NB; ++j) img[32 * G::DP + 32 * j + lq2] = zacc[j];     // row j of the z accumulator: column block j
+    }
+    // the first two units of pass 2 are requested now: their latency passes while the state is put together
+    constexpr int NQ = (kFU * G::CPR + 63) / 64;
+    auto issue_q = [&](u32x4 (&qreg)[NQ], int unit) {
+        const long n0 = static_cast<long>(min(unit, last_unit)) * kFU;
+        const long last = p.N - 1;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = min(lane2 + 64 * i, kFU * G::CPR - 1);
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            qreg[i] = *reinterpret_cast<const u32x4*>(q_base + min(n0 + row, last) * p.q_rs + cc * 8);
+        }
+    };
+    u32x4 qA[NQ], qB[NQ];
+    issue_q(qA, wave);
+    issue_q(qB, wave + kFusedWaves);
+    __syncthreads();
+    unsigned char* const Sb = lds + FG::WORK_BYTES;
+    float* const Zs = reinterpret_cast<float*>(Sb + FG::SB_BYTES);
+    float* const ws = p.ws + static_cast<long>(bh) * G::WS_FLOATS;
+    const float* const img0 = reinterpret_cast<const float*>(lds);
+    for (int idx = tid; idx < FG::IMG_FLOATS / 4; idx += kFusedThreads) {
+        const int i = idx / (G::DP / 4), j = (idx - i * (G::DP / 4)) * 4;        // i == 32: the z row
+        f32x4 v = *reinterpret_cast<const f32x4*>(img0 + i * G::DP + j);
+#pragma unroll
+        for (int w = 1; w < kFusedWaves; ++w) v += *reinterpret_cast<const f32x4*>(img0 + w * FG::IMG_FLOATS + i * G::DP + j);
+        const int row = 32 * slice + i;
+        if (i < 32) {
+            typedef T t4 __attribute__((ext_vector_type(4)));
+            t4 tv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tv[e] = (row < D && j < D) ? static_cast<T>(v[e]) : static_cast<T>(0.f);
+            *reinterpret_cast<t4*>(Sb + i * G::S_STRIDE + j * 2) = tv;
+            if (row < D && j < D) *reinterpret_cast<f32x4*>(ws + row * D + j) = v;
+        } else {
+            *reinterpret_cast<f32x4*>(Zs + j) = j < D ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            if (slice == 0 && j < D) *reinterpret_cast<f32x4*>(ws + D * D + j) = v;
+        }
+    }
+    __syncthreads();     // S slice and z are in place; the image space becomes the Q slices
+
+    // ───────────── pass 2: O[:, slice] = (S[slice rows, :] relu(Q)) / (z . relu(Q) + eps) ─────────────
+    V8 sf[G::KC];        // this lane's row of the slice, all contraction steps
+#pragma unroll
+    for (int c = 0; c < G::KC; ++c) sf[c] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Sb + lq2 * G::S_STRIDE + (16 * c + 8 * lh2) * 2));
+    unsigned char* const Qp = lds + wave * FG::P2_SLICE;
+    if constexpr (G::DP > D) {
+        constexpr int PC = (G::DP - D) / 8;
+        for (int i = lane2; i < kFU * PC; i += 64)
+            *reinterpret_cast<u32x4*>(Qp + (i / PC) * G::S_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
+    }
+    auto apply_unit = [&](const u32x4 (&qreg)[NQ], int unit) {
+        const int n0 = unit * kFU;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = lane2 + 64 * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < kFU * G::CPR) *reinterpret_cast<u32x4*>(Qp + row * G::S_STRIDE + cc * 16) = relu8<T>(qreg[i]);
+        }
+        wave_sync();
+        V8 qf[G::KC];
+        float den = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) {
+            const int d0 = 16 * c + 8 * lh2;
+            qf[c] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Qp + lq2 * G::S_STRIDE + d0 * 2));
+            const f32x4 z0 = *reinterpret_cast<const f32x4*>(Zs + d0);
+            const f32x4 z1 = *reinterpret_cast<const f32x4*>(Zs + d0 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                den = __builtin_fmaf(z0[e], static_cast<float>(qf[c][e]), den);
+                den = __builtin_fmaf(z1[e], static_cast<float>(qf[c][4 + e]), den);
+            }
+        }
+        {
+            const int di = __builtin_bit_cast(int, den);
+            const i32x2 r = __builtin_amdgcn_permlane32_swap(di, di, false, false);
+            const int r0 = r[0], r1 = r[1];
+            den = __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+        }
+        const float rs = __builtin_amdgcn_rsqf(den + p.eps);       // the reference's reciprocal: rsqrt(den + eps)^2 in FP32
+        const float recip = rs * rs;
+        f32x16 o;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) o = Mma<T>::run(sf[c], qf[c], o);
+        wave_sync();          // every lane2 holds its Q fragments: the slice takes the results
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb) {
+            typedef T t4 __attribute__((ext_vector_type(4)));
+            t4 ov;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ov[e] = static_cast<T>(o[4 * bb + e] * recip);
+            *reinterpret_cast<t4*>(Qp + lq2 * FG::O_STRIDE + (8 * bb + 4 * lh2) * 2) = ov;
+        }
+        wave_sync();
+        const int last_row = min(kFU, p.N - n0) - 1;
+#pragma unroll
+        for (int i = 0; i < kFU * VCH / 64; ++i) {
+            const int idx = lane2 + 64 * i;
+            const int row = min(idx / VCH, last_row), cc = min(idx % VCH, v_chunks - 1);
+            *reinterpret_cast<u32x4*>(o_base + static_cast<long>(n0 + row) * p.o_rs + cc * 8) =
+                *reinterpret_cast<const u32x4*>(Qp + row * FG::O_STRIDE + cc * 16);
+        }
+        wave_sync();          // the staged rows are read before the next unit's Q rows overwrite them
+        if constexpr (G::DP > D) {
+            // the output rows (80-byte stride) ran over pad chunks of the Q rows: zero again
+            constexpr int PC = (G::DP - D) / 8;
+            for (int i = lane2; i < kFU * PC; i += 64)
+                *reinterpret_cast<u32x4*>(Qp + (i / PC) * G::S_STRIDE + D * 2 + (i % PC) * 16) = u32x4{0, 0, 0, 0};
+        }
+    };
+    {
+        for (int u = wave; u < n_units; u += 2 * kFusedWaves) {
+            apply_unit(qA, u);
+            issue_q(qA, u + 2 * kFusedWaves);
+            // (unconditional: past its last unit a wavefront applies the last unit of the call once more and stores the same
+            //  bytes again, so that the number of stores between two waits is fixed)
+            apply_unit(qB, min(u + kFusedWaves, last_unit));
+            issue_q(qB, u + 3 * kFusedWaves);
+        }
+    }
+}
+
 template <typename T, int D>
 int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st) {
     using G = LGeo<D>;
     const int BH = p.B * p.H;
+    // One launch with the state split along its value channels, when the call does not add to a state that is already
+    // there (every work group of a head would read the old z while one of them replaces it) and its work groups fill
+    // enough of the GPU; otherwise three launches (state per token chunk, reduction, apply).
+    {
+        using FG = FusedGeo<D>;
+        const int groups = BH * FG::NS;
+        const bool fits = !accumulate && static_cast<long>(BH) * FG::NS < (1L << 24);
+        // Picked by size (measured, 256 compute units): with one slice per head (head_dim 32) nothing is read twice and the
+        // single launch wins at every length once its work groups cover a quarter of the GPU; with several slices every
+        // work group pulls all of K and Q through its own compute unit's L2 port (about 50 GB/s each), which costs more
+        // than the two extra launches from about 2000 tokens on (head_dim 112, 40 heads: 13.6 against 18.5 us at 512
+        // tokens, 20.5 against 23.4 at 1024, 32 against 31 at 2048, 55 against 42 at 4096).
+        const bool by_size = fits && (FG::NS == 1 ? 4 * groups >= n_cu : (2 * groups >= n_cu && p.N <= kFusedMaxTokens));
+        if (fits && (p.form == MI_LINEAR_ATTN_FORM_ONE_LAUNCH || (p.form == MI_LINEAR_ATTN_FORM_BY_SIZE && by_size))) {
+            static thread_local bool raised = false;
+            if (!raised) {
+                MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&linattn_fused_kernel<T, D>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 FG::LDS_BYTES));
+                raised = true;
+            }
+            p.n_blocks = groups;
+            hipLaunchKernelGGL((linattn_fused_kernel<T, D>), dim3(((groups + 7) / 8) * 8), dim3(kFusedThreads), FG::LDS_BYTES, st, p);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return fail("mi_linear_attn_relu_forward launch: %s", hipGetErrorString(e));
+            return 0;
+        }
+    }
     // State pass. The tokens of a head are split over enough groups to keep most CUs streaming, if the caller lent a
     // scratch for the partial states; each group needs a few tiles to amortise its prologue and epilogue.
     {
@@ -606,6 +950,8 @@ int linear_attn_forward(const mi_linear_attn_args* a, const char* op, void* part
     p.part = max_split > 0 ? static_cast<float*>(part) : nullptr; p.n_part = 0; p.add_to_state = 0;
     p.old_weight = a->accumulate_weight != 0.f ? a->accumulate_weight : 1.f;
     p.tokens_per_group = 0;
+    if (a->form < MI_LINEAR_ATTN_FORM_BY_SIZE || a->form > MI_LINEAR_ATTN_FORM_ONE_LAUNCH) return fail("%s: form must be 0 (by size), 1 (three launches) or 2 (one launch)", op);
+    p.form = a->form;
     hipStream_t st = resolve_stream(a->stream);
     const int n_cu = device_cu_count();
     return launch_t<__bf16>(p, a->head_dim, a->accumulate_state != 0, max_split, n_cu, st);

@@ -193,6 +193,12 @@ template <int D> constexpr int shortkv_lds_bytes(int n_kt, bool with_mask) {
     using G = HeadGeo<D>;
     return 256 * G::O_STRIDE + n_kt * (G::K_BYTES + G::V_BYTES + (with_mask ? kBN * 4 : 0));
 }
+// most key tiles that fit in LDS next to the staging slices at head dimension D (the prologue holds that many in registers)
+template <int D> constexpr int shortkv_max_tiles() {
+    int n = kShortMaxTiles;
+    while (n > 1 && shortkv_lds_bytes<D>(n, false) > 160 * 1024) --n;
+    return n;
+}
 
 template <typename T, int D>
 __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDev p, int n_kt, int units_per_group, int groups_per_head) {
@@ -265,11 +271,12 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
         const unsigned char* const k_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.k) + b * p.k_bs + hk * D);
         const unsigned char* const v_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(p.v) + b * p.v_bs + hk * D);
         const unsigned k_rsb = static_cast<unsigned>(p.k_rs) * 2u, v_rsb = static_cast<unsigned>(p.v_rs) * 2u;
-        u32x4 kreg[kShortMaxTiles][NLD], vreg[kShortMaxTiles][NLD];
+        constexpr int MAXT = shortkv_max_tiles<D>();
+        u32x4 kreg[MAXT][NLD], vreg[MAXT][NLD];
         float mval = 0.f;
         if (p.key_mask && tid < n_kt_b * kBN && tid < kv_len) mval = p.key_mask[b * p.key_mask_bs + tid];
 #pragma unroll
-        for (int t = 0; t < kShortMaxTiles; ++t) {
+        for (int t = 0; t < MAXT; ++t) {
             if (t < n_kt_b) {
                 const int last = min(kv_len - t * kBN, kBN) - 1;   // rows past the last key repeat it and are stored as zeros
 #pragma unroll
@@ -285,7 +292,7 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
         zero_pads<D, kThreads8>(Kall, Vall, G::K_BYTES, G::V_BYTES, n_kt_b, tid);
         if (p.key_mask && tid < n_kt * kBN) Mall[tid] = mval;
 #pragma unroll
-        for (int t = 0; t < kShortMaxTiles; ++t) {
+        for (int t = 0; t < MAXT; ++t) {
             if (t < n_kt_b) {
                 const int nvalid = kv_len - t * kBN;
 #pragma unroll
@@ -312,7 +319,11 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
         V8 qf[G::KC];
         read_q_frags<T, D>(qf, Qs, lq, lh);
         wave_sync();       // the slice is free again (it takes the output next)
-        if (u + 8 < u_end) q_issue(q0 + 8 * UM);
+        // The next unit's rows, unconditionally (past its last unit a wavefront fetches the current one again, from cache):
+        // vector-memory loads and stores complete in one order here, so the wait in front of the next q_store can pass over
+        // this unit's output stores only if the compiler can count them, i.e. if neither the loads nor the stores sit
+        // under a condition. With a conditional load the next unit waited for this unit's stores to land.
+        q_issue(u + 8 < u_end ? q0 + 8 * UM : q0);
 
         f32x16 oacc[G::VB];
 #pragma unroll
@@ -335,11 +346,15 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_shortkv_kernel(const SdpaDe
         const float inv = row_inverse(l_tot);
         stage_output<T, D>(Qs, lq, lh, oacc, inv);
         wave_sync();
-        for (int idx = lane; idx < UM * G::CPR; idx += 64) {
-            const int row = idx / G::CPR, cc = idx - row * G::CPR;
-            if (q0 + row < p.Lq)
-                *reinterpret_cast<u32x4*>(o_base + static_cast<long>(q0 + row) * p.o_rs + cc * 8) =
-                    *reinterpret_cast<const u32x4*>(Qs + row * G::O_STRIDE + cc * 16);
+        // (a fixed number of unconditional stores, see above: a lane without a chunk of its own, or whose row lies past the
+        //  end of Q, stores a chunk that another lane stores too, same bytes to the same address)
+        const int last_row = min(UM, p.Lq - q0) - 1;
+#pragma unroll
+        for (int i = 0; i < (UM * G::CPR + 63) / 64; ++i) {
+            const int idx = min(lane + 64 * i, UM * G::CPR - 1);
+            const int row = min(idx / G::CPR, last_row), cc = idx % G::CPR;
+            *reinterpret_cast<u32x4*>(o_base + static_cast<long>(q0 + row) * p.o_rs + cc * 8) =
+                *reinterpret_cast<const u32x4*>(Qs + row * G::O_STRIDE + cc * 16);
         }
         wave_sync();       // the staged rows are read before the next unit's Q overwrites them
     }
@@ -1158,7 +1173,7 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     // short key sequences whose K and V fit in LDS next to a query tile: one work group walks several query tiles
     const int n_kt = (p.Lk + kBN - 1) / kBN;
     if (D <= 128 && choice == 0 && p.mask_mode == MI_MASK_NONE && p.bias == nullptr && p.lse == nullptr &&
-        p.Lp == 0 && !rope_k && p.cos_q == nullptr && n_kt >= 1 && n_kt <= kShortMaxTiles && tiles256 >= n_cu &&
+        p.Lp == 0 && !rope_k && p.cos_q == nullptr && n_kt >= 1 && n_kt <= shortkv_max_tiles<(D <= 128 ? D : 128)>() && tiles256 >= n_cu &&
         shortkv_lds_bytes<D>(n_kt, p.key_mask != nullptr) <= 160 * 1024) {
         if constexpr (D <= 128) {
             p.n_q_tiles = (p.Lq + 255) / 256;

@@ -919,11 +919,13 @@ def _linear_attn_args(op: str, Q, K, V, num_heads: int, out, eps: float, workspa
 
 def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
                                   workspace: Optional[torch.Tensor] = None, accumulate_state: bool = False,
-                                  scratch: Optional[torch.Tensor] = None):
+                                  scratch: Optional[torch.Tensor] = None, form: int = 0):
     """Sana's ReLU linear attention core (src/dit/sana.cpp:470-586) on token-major (N, heads*head_dim)
     or (batch, N, heads*head_dim) operands. `workspace` (float32, batch*heads*(d*d+d)) receives the
     (S, z) state; pass it to capture the state or, with accumulate_state, to inject one. `scratch` (float32) holds
-    partial states of token chunks; None allocates one, False runs without (one work group per batch item and head)."""
+    partial states of token chunks; None allocates one, False runs without (one work group per batch item and head).
+    `form`: 0 = the library picks, 1 = three launches (state per token chunk, reduction, apply), 2 = one launch with the
+    state split along its value channels (mi_linear_attn_args.form)."""
     op = "linear_attention_relu_forward"
     _dev(op, Q, K, V, out, workspace, scratch if scratch is not False else None)
     if out is None:
@@ -947,6 +949,7 @@ def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.T
         _fail(op, "scratch must be contiguous float32")
     if scratch.numel() > 0:
         a.scratch, a.scratch_bytes = scratch.data_ptr(), scratch.numel() * 4
+    a.form = int(form)
     capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
     return out
 

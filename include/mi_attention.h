@@ -351,8 +351,13 @@ typedef struct mi_linear_attn_args {
     size_t workspace_bytes;
     void* scratch;          /* device, 16-byte aligned, or NULL */
     size_t scratch_bytes;
+    int32_t form;           /* MI_LINEAR_ATTN_FORM_BY_SIZE (0): the library picks. _THREE_LAUNCHES: state per token chunk, reduction
+                               of the partial states (in `scratch`), apply. _ONE_LAUNCH: the state split along its value channels,
+                               every work group streams K, its slice of V, then Q, and writes its slice of O; no scratch is used.
+                               A call that accumulates onto a state always takes the three launches */
     void* stream;
 } mi_linear_attn_args;
+enum { MI_LINEAR_ATTN_FORM_BY_SIZE = 0, MI_LINEAR_ATTN_FORM_THREE_LAUNCHES = 1, MI_LINEAR_ATTN_FORM_ONE_LAUNCH = 2 };
 MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API int mi_linear_attn_relu_forward(const mi_linear_attn_args* args);

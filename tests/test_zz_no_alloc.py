@@ -24,6 +24,7 @@ def _args(q, k, v, o, ws, H, d, accumulate=False):
     a.eps = 1e-15
     a.accumulate_state = int(accumulate)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel() * 4
+    a.form = capi.MI_LINEAR_ATTN_FORM_THREE_LAUNCHES      # the form whose partial states need the scratch this file is about
     a.stream = torch.cuda.current_stream().cuda_stream
     return a
 
