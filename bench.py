@@ -280,6 +280,17 @@ def all_configs(torch, bd, cin, keep):
                      "frac_copy_ceiling": round(nbytes / (mn * 1e-3) / 1e9 / copy_gbs, 4), "dtype": "bf16 in, f32 accumulate",
                      "mbytes": round(nbytes / 1e6, 2), "ms_graph": graph_ms(torch, la)}
         keep[key] = o
+        # the two kernel forms side by side (the row above is the library's own choice by size), and the same values as
+        # (heads*head_dim, N) channel-major tensors, the layout of the reference's core (src/dit/sana.cpp:424-444)
+        for form, tag in ((1, "three_launches"), (2, "one_launch")):
+            out[name]["us_graph_" + tag] = round(1e3 * (graph_ms(torch, lambda: bd.linear_attention_relu_forward(
+                ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc, form=form)) or 0.0), 1)
+        qc, kc_, vc_ = (t.transpose(1, 2).contiguous() for t in (ql, kl, vl_))
+        oc = torch.empty_like(qc)
+        out[name]["us_graph_channel_major"] = round(1e3 * (graph_ms(torch, lambda: bd.linear_attention_relu_forward_channel_major(
+            qc, kc_, vc_, 20, out=oc, workspace=ws)) or 0.0), 1)
+        bd.linear_attention_relu_forward(ql, kl, vl_, 20, out=o, workspace=ws, scratch=sc)     # `o` holds the by-size result again
+        del qc, kc_, vc_, oc
     return out
 
 
@@ -405,12 +416,27 @@ def main():
         lq, lk, lv = (torch.randn(2, 4096, 2240, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(3))
         lo = torch.empty_like(lq)
         lws = torch.empty(2 * 20 * (112 * 112 + 112), dtype=torch.float32, device="cuda")
+        lsc = torch.empty(8 * lws.numel(), dtype=torch.float32, device="cuda")
+        # cfg5a (N=1024, the one-launch form) and cfg2b (PixArt cross attention, the short-key kernel) ride along as well
+        sq, sk, sv = (torch.randn(2, 1024, 2240, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(3))
+        so = torch.empty_like(sq)
+        cq = torch.randn(2, 4096, 1152, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
+        ck, cv = (torch.randn(2, 300, 1152, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16) for _ in range(2))
+        co = torch.empty_like(cq)
+        cvl = torch.tensor([77, 105], dtype=torch.int32, device="cuda")
+        zeros = torch.zeros(1 << 20, dtype=torch.bfloat16, device="cuda")
+        noise = torch.randn(1 << 20, device="cuda", dtype=torch.float32, generator=g).to(torch.bfloat16)
         for _ in range(3):
             dst.copy_(src)
             step()
-            bd.linear_attention_relu_forward(lq, lk, lv, 20, out=lo, workspace=lws)
+            bd.linear_attention_relu_forward(lq, lk, lv, 20, out=lo, workspace=lws, scratch=lsc)
+            bd.linear_attention_relu_forward(sq, sk, sv, 20, out=so, workspace=lws, scratch=lsc)
+            bd.sdpa_forward(cq, ck, cv, 16, kv_valid_len=cvl, out=co)
+            bd.mfma_probe(zeros, trips=2000, reps=1)
+            bd.mfma_probe(noise, trips=2000, reps=1)
         torch.cuda.synchronize()
-        print(json.dumps({"traffic_probe": "3 x (256 MiB copy, headline step, Sana linear attention N=4096)"}))
+        print(json.dumps({"traffic_probe": "3 x (256 MiB copy, headline step, Sana linear attention N=4096 and N=1024, PixArt cross attention, "
+                                           "MFMA loop on zeros and on N(0,1))"}))
         return
     preheat(torch, step)
     for _ in range(args.warmup):

@@ -33,6 +33,7 @@ from .ops import (  # noqa: F401
     cross_attention_forward_with_attn, mha_forward,
     linear_attention_relu_forward,
     linear_attention_relu_forward_static_scratch,
+    linear_attention_relu_forward_channel_major,
     linear_batched,
     qwen_rope_positions,
     rms_norm_rows,
@@ -48,7 +49,7 @@ from .ops import (  # noqa: F401
 __all__ = [
     "SdpaMask", "build_axial_rope_tables", "build_qwen_rope_tables", "qwen_rope_positions", "rope_tables_from_positions", "device_info", "mfma_probe", "flash_attention_forward",
     "flash_attention_windowed_forward", "gqa_attention_masked", "joint_attention",
-    "linear_attention_relu_forward", "linear_attention_relu_forward_static_scratch", "rope_apply", "flash_attention_qkvo_forward", "flash_attention_q_with_kv_cached_forward",
+    "linear_attention_relu_forward", "linear_attention_relu_forward_static_scratch", "linear_attention_relu_forward_channel_major", "rope_apply", "flash_attention_qkvo_forward", "flash_attention_q_with_kv_cached_forward",
     "flash_attention_project_kv", "flash_attention_scratch_bytes", "linear_batched", "headnorm_rope", "flash_attention_varlen_forward", "flash_attention_qkvo_int8w_fp16", "flash_attention_q_with_kv_cached_int8w_fp16",
     "flash_attention_project_kv_int8w_fp16", "linear_forward_batched_int8w_fp16", "fused_linear_geglu", "fused_linear_geglu_int8w", "add_inplace_vec", "add_inplace_row_bias", "joint_attention_traced", "cross_attention_forward_with_attn", "mha_forward", "attention_map_avg", "scale_rows", "rope_apply_perhead", "rms_norm_rows", "sana_self_attention", "sdpa_forward", "set_sdpa_kernel_choice",
 ]

@@ -21,6 +21,8 @@ MI_LINEAR_ATTN_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 MI_LINEAR_ATTN_FORM_BY_SIZE = 0
 MI_LINEAR_ATTN_FORM_THREE_LAUNCHES = 1
 MI_LINEAR_ATTN_FORM_ONE_LAUNCH = 2
+MI_LAYOUT_TOKEN_MAJOR = 0
+MI_LAYOUT_CHANNEL_MAJOR = 1
 
 EXPORTS = [
     "mi_last_error", "mi_version", "mi_device_info", "mi_mfma_probe", "mi_set_stream", "mi_get_stream", "mi_stream_synchronize",
@@ -126,7 +128,7 @@ class MiLinearAttnArgs(C.Structure):
         ("o_row_stride", C.c_int64), ("o_batch_stride", C.c_int64),
         ("eps", C.c_float), ("accumulate_state", C.c_int32), ("accumulate_weight", C.c_float),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("form", C.c_int32), ("stream", C.c_void_p),
+        ("scratch", C.c_void_p), ("scratch_bytes", C.c_size_t), ("form", C.c_int32), ("layout", C.c_int32), ("stream", C.c_void_p),
     ]
 
 

@@ -87,6 +87,7 @@ struct LinDev {
     int n_chunks;   // token chunks per (batch, head)
     int n_blocks;   // work groups with work = B * H * n_chunks
     int form;       // MI_LINEAR_ATTN_FORM_*
+    int channel_major;   // operands are (heads * head_dim, tokens) per batch item; row strides are between channel rows
 };
 constexpr int kFusedMaxTokens = 1024;   // up to here the one-launch form is taken for sliced heads when the kernel is picked by size
 
@@ -813,6 +814,301 @@ __global__ void __launch_bounds__(kFusedThreads, 2) linattn_fused_kernel(const L
     }
 }
 
+
+// ── the same one-launch form on CHANNEL-MAJOR operands ──
+// Q, K, V, O as (heads * head_dim, tokens) per batch item, a row per channel: the layout in which the reference keeps
+// these tensors around its core (src/dit/sana.cpp:424-444, :470-586). The contraction of pass 1 runs over tokens, which
+// are contiguous here, so K and V rows go to LDS as they are (64-byte pieces of a row per 32-token unit, rows padded to
+// 80 bytes) and every MFMA operand is one 16-byte read; pass 2 contracts over channels, so its B operand (a token's
+// channels) comes out of the channel-by-token tile through transpose reads, and the result tile is turned back into
+// channel rows in LDS before it is stored. Everything else — one work group per (batch, head, 32 value channels),
+// independent wavefronts, two register sets, unconditional vector-memory instructions, the merge of the eight partial
+// states in a fixed order — is the token-major kernel's. Consecutive units go to the same wavefront in pairs: the two
+// halves of a 128-byte line of a channel row are then fetched by one wavefront back to back.
+template <int D> struct FusedCmGeo {
+    using G = LGeo<D>;
+    static constexpr int NS = G::NB;
+    static constexpr int KV_STRIDE = kFU * 2 + 16;                      // pass 1: a unit's 32 tokens of one channel, padded
+    static constexpr int P1_SLICE = (G::DP + 32) * KV_STRIDE;           // K channels, then the slice's V channels
+    static constexpr int IMG_FLOATS = 32 * G::DP + G::DP;
+    static constexpr int Q_STRIDE = kFU * 2;                            // pass 2: channel rows back to back (64 mod 128: transpose reads)
+    static constexpr int O_STRIDE = kFU * 2 + 16;
+    static constexpr int cmax(int a, int b) { return a > b ? a : b; }
+    static constexpr int P2_SLICE = cmax(G::DP * Q_STRIDE, 32 * O_STRIDE);   // the staged output rows reuse the unit's Q slice
+    static constexpr int SB_BYTES = 32 * G::S_STRIDE;
+    static constexpr int WORK_BYTES = cmax(cmax(kFusedWaves * P1_SLICE, kFusedWaves * IMG_FLOATS * 4), kFusedWaves * P2_SLICE);
+    static constexpr int LDS_BYTES = WORK_BYTES + SB_BYTES + G::DP * 4;
+    static_assert(32 * O_STRIDE <= P2_SLICE, "the staged output fits the unit's Q slice");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a compute unit");
+};
+
+template <typename T, int D>
+__global__ void __launch_bounds__(kFusedThreads, 2) linattn_fused_cm_kernel(const LinDev p) {
+    using G = LGeo<D>;
+    using FG = FusedCmGeo<D>;
+    using V8 = typename Mma<T>::v8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    int bh, slice;
+    {
+        LinDev q = p;
+        q.n_chunks = FG::NS;
+        if (!lin_block(q, bh, slice)) return;
+    }
+    const int b = bh / p.H, h = bh % p.H;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int lq = lane & 31, lh = lane >> 5;
+    // channel rows of this head; strides are in elements between channel rows
+    const T* const q_base = static_cast<const T*>(p.q) + b * p.q_bs + static_cast<long>(h) * D * p.q_rs;
+    const T* const k_base = static_cast<const T*>(p.k) + b * p.k_bs + static_cast<long>(h) * D * p.k_rs;
+    const T* const v_base = static_cast<const T*>(p.v) + b * p.v_bs + (static_cast<long>(h) * D + 32 * slice) * p.v_rs;
+    T* const o_base = static_cast<T*>(p.o) + b * p.o_bs + (static_cast<long>(h) * D + 32 * slice) * p.o_rs;
+    const int v_rows = min(32, D - 32 * slice);              // value channels of this slice that exist
+    constexpr int UCH = kFU / 8;                             // 16-byte chunks of a unit's tokens in one channel row (4)
+    const int n_units = (p.N + kFU - 1) / kFU;               // N is a multiple of 8: a chunk is whole or absent
+    const int last_unit = n_units - 1;
+    auto wave_sync = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    // units go to wavefronts in pairs: turn t of wavefront w is units 16 t + 2 w and 16 t + 2 w + 1
+    constexpr int kTurn = 2 * kFusedWaves;
+
+    // ───────────── pass 1 ─────────────
+    unsigned char* const Kp = lds + wave * FG::P1_SLICE;
+    unsigned char* const Vp = Kp + G::DP * FG::KV_STRIDE;
+    constexpr int NK = (D * UCH + 63) / 64;
+    constexpr int NV = 32 * UCH / 64;                        // 2
+    if constexpr (G::DP > D) {                               // channel rows past the head dimension stay zero
+        for (int i = lane; i < (G::DP - D) * UCH; i += 64)
+            *reinterpret_cast<u32x4*>(Kp + (D + i / UCH) * FG::KV_STRIDE + (i % UCH) * 16) = u32x4{0, 0, 0, 0};
+    }
+    auto chunk_col = [&](int unit, int cc) { return static_cast<long>(min(unit, last_unit)) * kFU + 8 * cc; };
+    auto issue_kv = [&](u32x4 (&kreg)[NK], u32x4 (&vreg)[NV], int unit) {
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int idx = min(lane + 64 * i, D * UCH - 1);
+            const int row = idx / UCH, cc = idx - row * UCH;
+            kreg[i] = *reinterpret_cast<const u32x4*>(k_base + row * p.k_rs + min(chunk_col(unit, cc), static_cast<long>(p.N) - 8));
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = min(idx / UCH, v_rows - 1), cc = idx % UCH;
+            vreg[i] = *reinterpret_cast<const u32x4*>(v_base + row * p.v_rs + min(chunk_col(unit, cc), static_cast<long>(p.N) - 8));
+        }
+    };
+    auto store_kv = [&](const u32x4 (&kreg)[NK], const u32x4 (&vreg)[NV], int unit) {
+        const int n0 = unit * kFU;
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / UCH, cc = idx - row * UCH;
+            if (idx < D * UCH) {
+                u32x4 kv = relu8<T>(kreg[i]);
+                if (n0 + 8 * cc >= p.N) kv = u32x4{0, 0, 0, 0};          // tokens that do not exist add nothing
+                *reinterpret_cast<u32x4*>(Kp + row * FG::KV_STRIDE + cc * 16) = kv;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / UCH, cc = idx - row * UCH;
+            *reinterpret_cast<u32x4*>(Vp + row * FG::KV_STRIDE + cc * 16) = row < v_rows ? vreg[i] : u32x4{0, 0, 0, 0};
+        }
+    };
+    f32x16 acc[G::NB], zacc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        zacc[e] = 0.f;
+#pragma unroll
+        for (int j = 0; j < G::NB; ++j) acc[j][e] = 0.f;
+    }
+    const unsigned one2 = (std::is_same_v<T, __bf16> ? 0x3f803f80u : 0x3c003c00u);
+    auto sel = [&](int j) -> V8 {
+        const unsigned w = lq == j ? one2 : 0u;
+        return __builtin_bit_cast(V8, u32x4{w, w, w, w});
+    };
+    auto multiply_unit = [&]() {
+#pragma unroll
+        for (int s2 = 0; s2 < kFU / 16; ++s2) {
+            const int off = (16 * s2 + 8 * lh) * 2;              // this lane's 8 tokens of the step
+            const V8 a = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Vp + lq * FG::KV_STRIDE + off));
+            V8 bk[G::NB];
+#pragma unroll
+            for (int j = 0; j < G::NB; ++j) bk[j] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Kp + (32 * j + lq) * FG::KV_STRIDE + off));
+#pragma unroll
+            for (int j = 0; j < G::NB; ++j) {
+                acc[j] = Mma<T>::run(a, bk[j], acc[j]);
+                zacc = Mma<T>::run(sel(j), bk[j], zacc);
+            }
+        }
+    };
+    {
+        u32x4 kA[NK], vA[NV], kB[NK], vB[NV];
+        int u = 2 * wave;
+        issue_kv(kA, vA, u);
+        issue_kv(kB, vB, u + 1);
+        for (; u < n_units; u += kTurn) {
+            store_kv(kA, vA, u);
+            wave_sync();
+            issue_kv(kA, vA, u + kTurn);
+            multiply_unit();
+            wave_sync();
+            if (u + 1 < n_units) {
+                store_kv(kB, vB, u + 1);
+                wave_sync();
+            }
+            issue_kv(kB, vB, u + kTurn + 1);
+            if (u + 1 < n_units) {
+                multiply_unit();
+                wave_sync();
+            }
+        }
+    }
+    __syncthreads();
+
+    // ───────────── the 8 partial states -> one ─────────────
+    int lane2 = lane;
+    asm volatile("" : "+v"(lane2));
+    const int lq2 = lane2 & 31, lh2 = lane2 >> 5;
+    float* const img = reinterpret_cast<float*>(lds) + wave * FG::IMG_FLOATS;
+#pragma unroll
+    for (int j = 0; j < G::NB; ++j) {
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) img[(8 * bb + 4 * lh2 + e) * G::DP + 32 * j + lq2] = acc[j][4 * bb + e];
+    }
+    if (lh2 == 0) {
+#pragma unroll
+        for (int j = 0; j < G::NB; ++j) img[32 * G::DP + 32 * j + lq2] = zacc[j];
+    }
+    constexpr int NQ = (D * UCH + 63) / 64;
+    auto issue_q = [&](u32x4 (&qreg)[NQ], int unit) {
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = min(lane2 + 64 * i, D * UCH - 1);
+            const int row = idx / UCH, cc = idx - row * UCH;
+            qreg[i] = *reinterpret_cast<const u32x4*>(q_base + row * p.q_rs + min(chunk_col(unit, cc), static_cast<long>(p.N) - 8));
+        }
+    };
+    u32x4 qA[NQ], qB[NQ];
+    issue_q(qA, 2 * wave);
+    issue_q(qB, 2 * wave + 1);
+    __syncthreads();
+    unsigned char* const Sb = lds + FG::WORK_BYTES;
+    float* const Zs = reinterpret_cast<float*>(Sb + FG::SB_BYTES);
+    float* const ws = p.ws + static_cast<long>(bh) * G::WS_FLOATS;
+    const float* const img0 = reinterpret_cast<const float*>(lds);
+    for (int idx = tid; idx < FG::IMG_FLOATS / 4; idx += kFusedThreads) {
+        const int i = idx / (G::DP / 4), j = (idx - i * (G::DP / 4)) * 4;
+        f32x4 v = *reinterpret_cast<const f32x4*>(img0 + i * G::DP + j);
+#pragma unroll
+        for (int w = 1; w < kFusedWaves; ++w) v += *reinterpret_cast<const f32x4*>(img0 + w * FG::IMG_FLOATS + i * G::DP + j);
+        const int row = 32 * slice + i;
+        if (i < 32) {
+            typedef T t4 __attribute__((ext_vector_type(4)));
+            t4 tv;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) tv[e] = (row < D && j < D) ? static_cast<T>(v[e]) : static_cast<T>(0.f);
+            *reinterpret_cast<t4*>(Sb + i * G::S_STRIDE + j * 2) = tv;
+            if (row < D && j < D) *reinterpret_cast<f32x4*>(ws + row * D + j) = v;
+        } else {
+            *reinterpret_cast<f32x4*>(Zs + j) = j < D ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+            if (slice == 0 && j < D) *reinterpret_cast<f32x4*>(ws + D * D + j) = v;
+        }
+    }
+    __syncthreads();
+
+    // ───────────── pass 2 ─────────────
+    // The transpose reads below hand a lane the channels 16 c + 4 lh + {0..3} and 16 c + 8 + 4 lh + {0..3} of its token (two
+    // 4 x 4 blocks), not 8 consecutive ones; the A operand and z take their contraction elements in the same order.
+    V8 sf[G::KC];
+#pragma unroll
+    for (int c = 0; c < G::KC; ++c) {
+        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+        const u32x2 a0 = *reinterpret_cast<const u32x2*>(Sb + lq2 * G::S_STRIDE + (16 * c + 4 * lh2) * 2);
+        const u32x2 a1 = *reinterpret_cast<const u32x2*>(Sb + lq2 * G::S_STRIDE + (16 * c + 8 + 4 * lh2) * 2);
+        sf[c] = __builtin_bit_cast(V8, u32x4{a0[0], a0[1], a1[0], a1[1]});
+    }
+    unsigned char* const Qp = lds + wave * FG::P2_SLICE;
+    if constexpr (G::DP > D) {
+        for (int i = lane2; i < (G::DP - D) * UCH; i += 64)
+            *reinterpret_cast<u32x4*>(Qp + (D + i / UCH) * FG::Q_STRIDE + (i % UCH) * 16) = u32x4{0, 0, 0, 0};
+    }
+    auto frag = [&](const unsigned char* ptr) -> V8 {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(ptr + 8 * FG::Q_STRIDE));
+        return __builtin_bit_cast(V8, (s16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    const int trow = (lane2 & 15) >> 2;
+    const int tcol = 16 * ((lane2 >> 4) & 1) + 4 * (lane2 & 3);
+    auto apply_unit = [&](const u32x4 (&qreg)[NQ], int unit) {
+        const int n0 = unit * kFU;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            const int idx = lane2 + 64 * i;
+            const int row = idx / UCH, cc = idx - row * UCH;
+            if (idx < D * UCH) *reinterpret_cast<u32x4*>(Qp + row * FG::Q_STRIDE + cc * 16) = relu8<T>(qreg[i]);
+        }
+        wave_sync();
+        V8 qf[G::KC];
+        float den = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) {
+            // token lq2 (a column of the tile), channels 16 c + 4 lh2 + {0..3} and 16 c + 8 + 4 lh2 + {0..3} (rows): the B
+            // operand of S relu(Q)
+            qf[c] = frag(Qp + (16 * c + 4 * lh2 + trow) * FG::Q_STRIDE + tcol * 2);
+            const int d0 = 16 * c + 4 * lh2;
+            const f32x4 z0 = *reinterpret_cast<const f32x4*>(Zs + d0);
+            const f32x4 z1 = *reinterpret_cast<const f32x4*>(Zs + d0 + 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                den = __builtin_fmaf(z0[e], static_cast<float>(qf[c][e]), den);
+                den = __builtin_fmaf(z1[e], static_cast<float>(qf[c][4 + e]), den);
+            }
+        }
+        {
+            const int di = __builtin_bit_cast(int, den);
+            const i32x2 r = __builtin_amdgcn_permlane32_swap(di, di, false, false);
+            const int r0 = r[0], r1 = r[1];
+            den = __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+        }
+        const float rs = __builtin_amdgcn_rsqf(den + p.eps);
+        const float recip = rs * rs;
+        f32x16 o;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) o = Mma<T>::run(sf[c], qf[c], o);
+        wave_sync();
+        // the result tile back into channel rows: element (channel 8 bb + 4 lh2 + e, token lq2)
+#pragma unroll
+        for (int bb = 0; bb < 4; ++bb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                *reinterpret_cast<T*>(Qp + (8 * bb + 4 * lh2 + e) * FG::O_STRIDE + lq2 * 2) = static_cast<T>(o[4 * bb + e] * recip);
+        wave_sync();
+        const int last_cc = min(UCH, (p.N - n0) / 8) - 1;
+#pragma unroll
+        for (int i = 0; i < 32 * UCH / 64; ++i) {
+            const int idx = lane2 + 64 * i;
+            const int row = min(idx / UCH, v_rows - 1), cc = min(idx % UCH, last_cc);
+            *reinterpret_cast<u32x4*>(o_base + row * p.o_rs + n0 + 8 * cc) =
+                *reinterpret_cast<const u32x4*>(Qp + row * FG::O_STRIDE + cc * 16);
+        }
+        wave_sync();
+    };
+    for (int u = 2 * wave; u < n_units; u += kTurn) {
+        apply_unit(qA, u);
+        issue_q(qA, u + kTurn);
+        apply_unit(qB, min(u + 1, last_unit));
+        issue_q(qB, u + kTurn + 1);
+    }
+}
+
 template <typename T, int D>
 int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st) {
     using G = LGeo<D>;
@@ -820,6 +1116,22 @@ int launch_d(LinDev p, bool accumulate, int max_split, int n_cu, hipStream_t st)
     // One launch with the state split along its value channels, when the call does not add to a state that is already
     // there (every work group of a head would read the old z while one of them replaces it) and its work groups fill
     // enough of the GPU; otherwise three launches (state per token chunk, reduction, apply).
+    if (p.channel_major) {
+        using FG = FusedCmGeo<D>;
+        const long groups = static_cast<long>(BH) * FG::NS;
+        if (groups >= (1L << 24)) return fail("mi_linear_attn_relu_forward: too many (batch, head) pairs for one launch");
+        static thread_local bool raised_cm = false;
+        if (!raised_cm) {
+            MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&linattn_fused_cm_kernel<T, D>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             FG::LDS_BYTES));
+            raised_cm = true;
+        }
+        p.n_blocks = static_cast<int>(groups);
+        hipLaunchKernelGGL((linattn_fused_cm_kernel<T, D>), dim3(((p.n_blocks + 7) / 8) * 8), dim3(kFusedThreads), FG::LDS_BYTES, st, p);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail("mi_linear_attn_relu_forward launch: %s", hipGetErrorString(e));
+        return 0;
+    }
     {
         using FG = FusedGeo<D>;
         const int groups = BH * FG::NS;
@@ -929,19 +1241,31 @@ int linear_attn_forward(const mi_linear_attn_args* a, const char* op, void* part
         max_split = static_cast<int>(std::min<size_t>(part_bytes / need, kMaxStateSplit));
     }
     const long D = static_cast<long>(a->num_heads) * a->head_dim;
+    if (a->layout != MI_LAYOUT_TOKEN_MAJOR && a->layout != MI_LAYOUT_CHANNEL_MAJOR) return fail("%s: layout must be 0 (token-major) or 1 (channel-major)", op);
+    const bool cm = a->layout == MI_LAYOUT_CHANNEL_MAJOR;
     LinDev p;
     p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o;
     p.B = a->batch; p.H = a->num_heads; p.N = a->n_tokens;
-    auto rs = [D](int64_t s) { return s ? static_cast<long>(s) : D; };
+    p.channel_major = cm ? 1 : 0;
+    // token-major: a row is a token (heads*head_dim values); channel-major: a row is a channel (n_tokens values)
+    const long row_len = cm ? a->n_tokens : D, n_rows = cm ? D : a->n_tokens;
+    auto rs = [row_len](int64_t s) { return s ? static_cast<long>(s) : row_len; };
     p.q_rs = rs(a->q_row_stride); p.k_rs = rs(a->k_row_stride); p.v_rs = rs(a->v_row_stride); p.o_rs = rs(a->o_row_stride);
-    p.q_bs = a->q_batch_stride ? a->q_batch_stride : p.q_rs * a->n_tokens;
-    p.k_bs = a->k_batch_stride ? a->k_batch_stride : p.k_rs * a->n_tokens;
-    p.v_bs = a->v_batch_stride ? a->v_batch_stride : p.v_rs * a->n_tokens;
-    p.o_bs = a->o_batch_stride ? a->o_batch_stride : p.o_rs * a->n_tokens;
+    p.q_bs = a->q_batch_stride ? a->q_batch_stride : p.q_rs * n_rows;
+    p.k_bs = a->k_batch_stride ? a->k_batch_stride : p.k_rs * n_rows;
+    p.v_bs = a->v_batch_stride ? a->v_batch_stride : p.v_rs * n_rows;
+    p.o_bs = a->o_batch_stride ? a->o_batch_stride : p.o_rs * n_rows;
+    if (cm) {
+        // 16-byte pieces of a channel row hold 8 tokens each; the state cannot be added onto in place in the only form
+        // these operands have (every work group of a head reads the old z while one of them replaces it)
+        if (a->n_tokens % 8 != 0) return fail("%s: channel-major operands need n_tokens to be a multiple of 8 (got %d)", op, a->n_tokens);
+        if (a->accumulate_state) return fail("%s: accumulate_state is not offered for channel-major operands (run into a second workspace and add the states)", op);
+    }
     const long strides[] = {p.q_rs, p.k_rs, p.v_rs, p.o_rs, p.q_bs, p.k_bs, p.v_bs, p.o_bs};
     for (long s : strides)
         if (s % 8 != 0) return fail("%s: strides must be multiples of 8 elements", op);
-    if (p.q_rs < D || p.k_rs < D || p.v_rs < D || p.o_rs < D) return fail("%s: row stride smaller than heads*head_dim", op);
+    if (p.q_rs < row_len || p.k_rs < row_len || p.v_rs < row_len || p.o_rs < row_len)
+        return fail("%s: row stride smaller than a row (%ld elements)", op, row_len);
     const uintptr_t al = reinterpret_cast<uintptr_t>(a->q) | reinterpret_cast<uintptr_t>(a->k) | reinterpret_cast<uintptr_t>(a->v) |
                          reinterpret_cast<uintptr_t>(a->o) | reinterpret_cast<uintptr_t>(a->workspace);
     if (al & 15u) return fail("%s: pointers must be 16-byte aligned", op);

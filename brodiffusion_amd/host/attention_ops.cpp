@@ -186,6 +186,31 @@ void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tenso
     check(op, mi_linear_attn_relu_forward(&a));
 }
 
+void linear_attention_relu_forward_channel_major(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
+                                                 Tensor& state, Tensor& out) {
+    const char* op = "linear_attention_relu_forward_channel_major";
+    need_gpu(op, Q); need_gpu(op, K); need_gpu(op, V);
+    if (num_heads <= 0 || Q.rows % num_heads != 0) fail(std::string(op) + ": D must equal head_dim * num_heads");
+    if (K.rows != Q.rows || V.rows != Q.rows || K.cols != Q.cols || V.cols != Q.cols || K.dtype != Q.dtype || V.dtype != Q.dtype)
+        fail(std::string(op) + ": Q/K/V must share shape (D, N) and dtype");
+    const int hd = Q.rows / num_heads;
+    const int per_head = hd * hd + hd;
+    if (state.data == nullptr || state.rows != num_heads || state.cols != per_head || state.dtype != Dtype::FP32)
+        state.resize(num_heads, per_head, Dtype::FP32, Q.device);
+    if (out.data == nullptr || out.rows != Q.rows || out.cols != Q.cols || out.dtype != Q.dtype)
+        out.resize(Q.rows, Q.cols, Q.dtype, Q.device);
+    mi_linear_attn_args a;
+    std::memset(&a, 0, sizeof(a));
+    a.struct_size = sizeof(a);
+    a.dtype = dtype_code(op, Q.dtype);
+    a.q = Q.data; a.k = K.data; a.v = V.data; a.o = out.data;
+    a.batch = 1; a.num_heads = num_heads; a.head_dim = hd; a.n_tokens = Q.cols;
+    a.eps = eps;
+    a.layout = MI_LAYOUT_CHANNEL_MAJOR;
+    a.workspace = state.data; a.workspace_bytes = state.bytes();
+    check(op, mi_linear_attn_relu_forward(&a));
+}
+
 namespace {
 const void* bias_ptr(const char* op, const Tensor* b, const char* name, Dtype dt, int n) {
     if (!b) return nullptr;

@@ -52,6 +52,12 @@ void rope_apply_perhead(const Tensor& X, const Tensor& cos, const Tensor& sin, i
 void linear_attention_relu_forward(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
                                    Tensor& state, Tensor& out, bool accumulate_state = false, Tensor* scratch = nullptr);
 
+// The same core on the reference's own operands: q, k, v and out as (heads*head_dim, N) channel-major tensors, the
+// shape of q_, k_, v_ and attn_c_ in SanaDenoiser::self_attention_ (src/dit/sana.cpp:424-444, :470-586), for a binding
+// that keeps the reference's projections and replaces the core alone. N must be a multiple of 8.
+void linear_attention_relu_forward_channel_major(const Tensor& Q, const Tensor& K, const Tensor& V, int num_heads, float eps,
+                                                 Tensor& state, Tensor& out);
+
 // Y = X W^T + bias, W (out_features, in_features); bias may be null.
 void linear_batched(const Tensor& W, const Tensor* bias, const Tensor& X, Tensor& Y);
 

@@ -954,6 +954,48 @@ def linear_attention_relu_forward(Q, K, V, num_heads: int, out: Optional[torch.T
     return out
 
 
+def linear_attention_relu_forward_channel_major(Q, K, V, num_heads: int, out: Optional[torch.Tensor] = None, eps: float = 1e-15,
+                                                workspace: Optional[torch.Tensor] = None):
+    """The ReLU linear-attention core on the reference's own operands: Q, K, V (and out) as (heads*head_dim, N) or
+    (batch, heads*head_dim, N) channel-major tensors, the layout of q_, k_, v_ and attn_c_ around the core in
+    src/dit/sana.cpp:424-444, :470-586 (mi_linear_attn_args.layout = MI_LAYOUT_CHANNEL_MAJOR). N must be a multiple of 8;
+    rows may be slices of longer rows (a row stride)."""
+    op = "linear_attention_relu_forward_channel_major"
+    _dev(op, Q, K, V, out, workspace)
+    dt = _dtype_code(op, Q)
+    if K.dtype != Q.dtype or V.dtype != Q.dtype or K.shape != Q.shape or V.shape != Q.shape:
+        _fail(op, "Q, K, V must share one shape and dtype")
+    if out is None:
+        out = torch.empty_like(Q)
+    if out.shape != Q.shape or out.dtype != Q.dtype:
+        _fail(op, "out must have Q's shape and dtype")
+    B, D, N, q_rs, q_bs = _as3(op, Q, "Q")
+    _, _, _, k_rs, k_bs = _as3(op, K, "K")
+    _, _, _, v_rs, v_bs = _as3(op, V, "V")
+    _, _, _, o_rs, o_bs = _as3(op, out, "out")
+    if num_heads <= 0 or D % num_heads != 0:
+        _fail(op, "D must equal head_dim * num_heads")
+    hd = D // num_heads
+    need = capi.lib().mi_linear_attn_workspace_bytes(B, num_heads, hd)
+    if workspace is None:
+        workspace = torch.empty(need // 4, dtype=torch.float32, device=Q.device)
+    if workspace.dtype != torch.float32 or not workspace.is_contiguous() or workspace.numel() * 4 < need:
+        _fail(op, f"workspace must be contiguous float32 with at least {need // 4} elements")
+    a = capi.MiLinearAttnArgs()
+    a.struct_size = C.sizeof(capi.MiLinearAttnArgs)
+    a.dtype = dt
+    a.q, a.k, a.v, a.o = Q.data_ptr(), K.data_ptr(), V.data_ptr(), out.data_ptr()
+    a.batch, a.num_heads, a.head_dim, a.n_tokens = B, num_heads, hd, N
+    a.q_row_stride, a.q_batch_stride, a.k_row_stride, a.k_batch_stride = q_rs, q_bs, k_rs, k_bs
+    a.v_row_stride, a.v_batch_stride, a.o_row_stride, a.o_batch_stride = v_rs, v_bs, o_rs, o_bs
+    a.eps = eps
+    a.layout = capi.MI_LAYOUT_CHANNEL_MAJOR
+    a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel() * 4
+    a.stream = _stream()
+    capi.check(capi.lib().mi_linear_attn_relu_forward(C.byref(a)), op)
+    return out
+
+
 def linear_attention_relu_forward_static_scratch(Q, K, V, num_heads: int, out: torch.Tensor, workspace: torch.Tensor,
                                                  eps: float = 1e-15, accumulate_state: bool = False):
     """linear_attention_relu_forward for callers that must not allocate: `out` and `workspace` are the caller's, the

@@ -355,8 +355,16 @@ typedef struct mi_linear_attn_args {
                                of the partial states (in `scratch`), apply. _ONE_LAUNCH: the state split along its value channels,
                                every work group streams K, its slice of V, then Q, and writes its slice of O; no scratch is used.
                                A call that accumulates onto a state always takes the three launches */
+    int32_t layout;         /* MI_LAYOUT_TOKEN_MAJOR (0): q, k, v, o are (batch, n_tokens, heads*head_dim), a row per token, as
+                               everywhere in this header. MI_LAYOUT_CHANNEL_MAJOR: (batch, heads*head_dim, n_tokens), a row per
+                               channel, head h in rows [h*head_dim, (h+1)*head_dim) — the layout in which the reference keeps
+                               q_, k_, v_ and attn_c_ around its core (src/dit/sana.cpp:424-444, :470-586), so that a binding
+                               which keeps the reference's projections can call the core alone. Row strides are then between
+                               channel rows (0 = n_tokens), batch strides default to heads*head_dim rows; n_tokens must be a
+                               multiple of 8; always one launch; accumulate_state is not offered */
     void* stream;
 } mi_linear_attn_args;
+enum { MI_LAYOUT_TOKEN_MAJOR = 0, MI_LAYOUT_CHANNEL_MAJOR = 1 };
 enum { MI_LINEAR_ATTN_FORM_BY_SIZE = 0, MI_LINEAR_ATTN_FORM_THREE_LAUNCHES = 1, MI_LINEAR_ATTN_FORM_ONE_LAUNCH = 2 };
 MI_API size_t mi_linear_attn_workspace_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);
 MI_API size_t mi_linear_attn_scratch_bytes(int32_t batch, int32_t num_heads, int32_t head_dim);

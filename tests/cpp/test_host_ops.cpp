@@ -261,6 +261,19 @@ static void gpu_checks() {
         std::printf("linear attention      rel_l2=%.3e max_abs=%.3e\n", e.rel_l2, e.max_abs);
         CHECK(within_bf16(e));
         CHECK(state.rows == Hl && state.cols == dl * dl + dl);
+        // the same values as (D, N) channel-major tensors, the reference's own layout around its core (src/dit/sana.cpp:424-444)
+        auto transposed = [&](const std::vector<float>& x) {
+            std::vector<float> t(x.size());
+            for (int n = 0; n < N; ++n)
+                for (int c = 0; c < Dl; ++c) t[static_cast<size_t>(c) * N + n] = x[static_cast<size_t>(n) * Dl + c];
+            return t;
+        };
+        Tensor Qc = upload_bf16(transposed(ql), Dl, N), Kc = upload_bf16(transposed(kl), Dl, N), Vc = upload_bf16(transposed(vl), Dl, N), state_c, out_c;
+        bt::linear_attention_relu_forward_channel_major(Qc, Kc, Vc, Hl, 1e-15f, state_c, out_c);
+        CHECK(out_c.rows == Dl && out_c.cols == N);
+        const Err ec = compare(transposed(ref), download_bf16(out_c));
+        std::printf("linear attention (D,N) rel_l2=%.3e max_abs=%.3e\n", ec.rel_l2, ec.max_abs);
+        CHECK(within_bf16(ec));
     }
     {   // traced joint attention: output and head-averaged map against the checker's restatement of the host loop
         const std::vector<int> axes = {16, 56, 56};

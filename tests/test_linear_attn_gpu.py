@@ -105,6 +105,49 @@ def test_one_launch_form_at_sizes_it_is_picked_for(oracle, B, H, d, N):
     assert np.max(np.abs(wsn[b, :, d * d:] - z)) <= 1e-4 * max(1.0, np.max(np.abs(z)))
 
 
+@pytest.mark.parametrize("B,H,d,N", [(2, 20, 112, 256), (1, 70, 32, 200), (2, 3, 64, 328), (1, 2, 72, 1000), (1, 2, 128, 136),
+                                     (1, 1, 112, 8), (2, 2, 32, 56), (2, 20, 112, 1024)])
+def test_linear_attention_channel_major(oracle, B, H, d, N):
+    """The core on the reference's own operand layout, (heads*head_dim, N) with a row per channel
+    (src/dit/sana.cpp:424-444): output and FP32 state against the checker on the transposed tensors, bit-reproducible,
+    and equal to the token-major call on the same values up to the order of the FP32 additions."""
+    dtype, D = "bf16", H * d
+    q, k, v = (randn(5051 + i, (B, N, D), dtype) for i in range(3))
+    cm = lambda x: to_dev(np.ascontiguousarray(x.transpose(0, 2, 1)), dtype)
+    ws = torch.empty(B * H * (d * d + d), dtype=torch.float32, device="cuda")
+    out = bd.linear_attention_relu_forward_channel_major(cm(q), cm(k), cm(v), H, workspace=ws)
+    assert tuple(out.shape) == (B, D, N)
+    got = to_np(out).transpose(0, 2, 1)
+    wsn = to_np(ws).reshape(B, H, d * d + d)
+    for b in range(B):
+        ref, S, z = oracle.linear_attn_relu(q[b], k[b], v[b], H, return_state=True)
+        assert_close(ref, got[b], dtype, f"channel-major b={b}")
+        assert np.max(np.abs(wsn[b, :, :d * d].reshape(H, d, d) - S)) <= 1e-4 * max(1.0, np.max(np.abs(S)))
+        assert np.max(np.abs(wsn[b, :, d * d:] - z)) <= 1e-4 * max(1.0, np.max(np.abs(z)))
+    ws2 = torch.empty_like(ws)
+    assert torch.equal(bd.linear_attention_relu_forward_channel_major(cm(q), cm(k), cm(v), H, workspace=ws2), out) and torch.equal(ws2, ws)
+    tm = bd.linear_attention_relu_forward(to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype), H, scratch=False, form=2)
+    assert (tm.float() - out.transpose(1, 2).float()).abs().max().item() <= 2.0 ** -7 * max(1.0, tm.float().abs().max().item())
+
+
+def test_linear_attention_channel_major_strided_and_errors(oracle):
+    """Channel rows as slices of longer rows (a token window of a wider buffer); what lies beside the output stays
+    untouched; token counts that are not a multiple of 8 and state accumulation are refused."""
+    dtype, H, d, N, pad = "bf16", 4, 112, 200, 24
+    D = H * d
+    q, k, v = (randn(5061 + i, (N, D), dtype) for i in range(3))
+    wide = [torch.zeros(D, N + pad, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+    for w, x in zip(wide, (q, k, v)):
+        w[:, 8:8 + N] = to_dev(np.ascontiguousarray(x.T), dtype)
+    o_wide = torch.full((D, N + pad), 3.0, dtype=torch.bfloat16, device="cuda")
+    out = bd.linear_attention_relu_forward_channel_major(wide[0][:, 8:8 + N], wide[1][:, 8:8 + N], wide[2][:, 8:8 + N], H, out=o_wide[:, 8:8 + N])
+    assert_close(oracle.linear_attn_relu(q, k, v, H), to_np(out).T, dtype, "strided channel-major")
+    assert (o_wide[:, :8] == 3).all() and (o_wide[:, 8 + N:] == 3).all()
+    x = torch.zeros((64, 104), dtype=torch.bfloat16, device="cuda")[:, :100]
+    with pytest.raises(RuntimeError, match="n_tokens to be a multiple of 8"):
+        bd.linear_attention_relu_forward_channel_major(x, x, x, 2)
+
+
 def test_linear_attention_form_argument():
     x = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
     with pytest.raises(RuntimeError, match="form must be"):

@@ -52,7 +52,7 @@ def _both(oracle, B, H, d, N, seed, accumulate=False):
     free0, held0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
     assert lib.mi_linear_attn_relu_forward_static_scratch(C.byref(a)) == 0, capi.last_error()
     torch.cuda.synchronize()
-    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() == held0
+    assert torch.cuda.mem_get_info()[0] == free0 and torch.cuda.memory_allocated() <= held0
     assert torch.equal(o_st, o_ref) and torch.equal(ws_st, ws_ref)
     if not accumulate:
         for b in range(B):
