@@ -152,62 +152,85 @@ __device__ __forceinline__ WaveExtent wave_extent(int lo, int hi) {
 // output staging uses later). All loads are issued before the first is used: out-of-range rows and the zero-pad
 // chunk are fetched from a clamped address and blanked at the store.
 // q_scale != 1 folds a factor (softmax scale times log2 e) into Q before its single rounding to T.
+// The loads and the stores of the staging are separate steps, so that a kernel can put other work (the first key tiles'
+// DMA) between them; `store<I0, I1>` stores the chunks of load rounds [I0, I1) with tile row `row_base` at the start of
+// `Qs` (a tile may be staged in pieces through a smaller buffer when its rounds fall on whole rows).
+template <typename T, int D, int NT, int ROWS>
+struct QTileLoad {
+    using G = HeadGeo<D>;
+    static constexpr int CPRK = G::DK / 8;     // chunks per staged row (data chunks, then the zero pad)
+    static constexpr int NCH = ROWS * CPRK;
+    static constexpr int NI = (NCH + NT - 1) / NT;
+    u32x4 raw[NI];
+    f32x4 cs[NI], sn[NI];
+    __device__ __forceinline__ void issue(const SdpaDev& p, const T* q_base, int q0, int tid, int last_row) {
+        const bool rope = p.cos_q != nullptr && !p.rope_split;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int idx = min(tid + NT * i, NCH - 1);
+            const int row = idx / CPRK, cc = min(idx - row * CPRK, G::CPR - 1);
+            const int qrow = min(q0 + row, last_row);
+            raw[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + cc * 8);
+            if (rope) {
+                cs[i] = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
+                sn[i] = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
+            }
+        }
+    }
+    template <int I0 = 0, int I1 = NI>
+    __device__ __forceinline__ void store(unsigned char* Qs, const SdpaDev& p, int q0, int tid, int last_row, float q_scale = 1.f, int row_base = 0) const {
+        const bool rope = p.cos_q != nullptr && !p.rope_split;
+#pragma unroll
+        for (int i = I0; i < I1; ++i) {
+            const int idx = tid + NT * i;
+            const int row = idx / CPRK, cc = idx - row * CPRK;
+            u32x4 v = raw[i];
+            if (rope) v = rope_chunk<T>(v, cs[i], sn[i], q_scale);
+            else if (q_scale != 1.f) v = scale_chunk<T>(v, q_scale);
+            if (q0 + row > last_row || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
+            if (idx < NCH) *reinterpret_cast<u32x4*>(Qs + (row - row_base) * G::O_STRIDE + cc * 16) = v;
+        }
+    }
+};
+
+// Split-half pairs (x[p], x[p + D/2]) sit in different 16-byte chunks, so that rotation is a second pass over staged
+// rows (tile rows [row_base, row_base + rows) at the start of `Qs`, stored and made visible by a barrier before): one
+// thread takes 4 pairs, i.e. 8 bytes from each half of a row (and the 4 table entries they share), and writes them back.
+// Same arithmetic and single rounding as the stand-alone pass; rows past the end are zero.
+template <typename T, int D, int NT>
+__device__ __forceinline__ void rope_split_staged(unsigned char* Qs, const SdpaDev& p, int q0, int tid, int last_row, float q_scale, int row_base, int rows) {
+    using G = HeadGeo<D>;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    constexpr int UPR = D / 8;             // units of 4 pairs per row
+    for (int u = tid; u < rows * UPR; u += NT) {
+        const int row = u / UPR, g = u - row * UPR;
+        const int qrow = min(q0 + row_base + row, last_row);
+        const f32x4 c4 = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + g * 4);
+        const f32x4 s4 = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + g * 4);
+        t4* const lo_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + g * 8);
+        t4* const hi_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + D + g * 8);
+        t4 lo = *lo_p, hi = *hi_p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float a = static_cast<float>(lo[e]), b = static_cast<float>(hi[e]);
+            lo[e] = static_cast<T>(rope_re(a, b, c4[e], s4[e]) * q_scale);
+            hi[e] = static_cast<T>(rope_im(a, b, c4[e], s4[e]) * q_scale);
+        }
+        *lo_p = lo;
+        *hi_p = hi;
+    }
+}
+
 template <typename T, int D, int NT, int ROWS>
 __device__ __forceinline__ void stage_q_tile(unsigned char* Qs, const SdpaDev& p, const T* q_base, int q0, int tid, float q_scale = 1.f,
                                              int last_row_override = -1) {
-    using G = HeadGeo<D>;
-    constexpr int CPRK = G::DK / 8;            // chunks per staged row (data chunks, then the zero pad)
-    constexpr int NCH = ROWS * CPRK;
-    constexpr int NI = (NCH + NT - 1) / NT;
     const int last_row = last_row_override >= 0 ? last_row_override : p.Lq - 1;   // (a packed sequence has its own length)
-    const bool rope = p.cos_q != nullptr && !p.rope_split;
-    u32x4 raw[NI];
-    f32x4 cs[NI], sn[NI];
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int idx = min(tid + NT * i, NCH - 1);
-        const int row = idx / CPRK, cc = min(idx - row * CPRK, G::CPR - 1);
-        const int qrow = min(q0 + row, last_row);
-        raw[i] = *reinterpret_cast<const u32x4*>(q_base + static_cast<long>(qrow) * p.q_rs + cc * 8);
-        if (rope) {
-            cs[i] = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
-            sn[i] = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + cc * 4);
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int idx = tid + NT * i;
-        const int row = idx / CPRK, cc = idx - row * CPRK;
-        u32x4 v = raw[i];
-        if (rope) v = rope_chunk<T>(v, cs[i], sn[i], q_scale);
-        else if (q_scale != 1.f) v = scale_chunk<T>(v, q_scale);
-        if (q0 + row > last_row || cc >= G::CPR) v = u32x4{0, 0, 0, 0};
-        if (idx < NCH) *reinterpret_cast<u32x4*>(Qs + row * G::O_STRIDE + cc * 16) = v;
-    }
-    // Split-half pairs (x[p], x[p + D/2]) sit in different 16-byte chunks, so that rotation is a second pass over the
-    // staged rows: one thread takes 4 pairs, i.e. 8 bytes from each half of a row (and the 4 table entries they share),
-    // and writes them back. Same arithmetic and single rounding as the stand-alone pass; rows past the end are zero.
+    QTileLoad<T, D, NT, ROWS> ql;
+    ql.issue(p, q_base, q0, tid, last_row);
+    ql.store(Qs, p, q0, tid, last_row, q_scale);
     if (p.cos_q != nullptr && p.rope_split) {
-        typedef T t4 __attribute__((ext_vector_type(4)));
-        constexpr int UPR = D / 8;             // units of 4 pairs per row
         __syncthreads();
-        for (int u = tid; u < ROWS * UPR; u += NT) {
-            const int row = u / UPR, g = u - row * UPR;
-            const int qrow = min(q0 + row, last_row);
-            const f32x4 c4 = *reinterpret_cast<const f32x4*>(p.cos_q + static_cast<long>(qrow) * (D / 2) + g * 4);
-            const f32x4 s4 = *reinterpret_cast<const f32x4*>(p.sin_q + static_cast<long>(qrow) * (D / 2) + g * 4);
-            t4* const lo_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + g * 8);
-            t4* const hi_p = reinterpret_cast<t4*>(Qs + row * G::O_STRIDE + D + g * 8);
-            t4 lo = *lo_p, hi = *hi_p;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float a = static_cast<float>(lo[e]), b = static_cast<float>(hi[e]);
-                lo[e] = static_cast<T>(rope_re(a, b, c4[e], s4[e]) * q_scale);
-                hi[e] = static_cast<T>(rope_im(a, b, c4[e], s4[e]) * q_scale);
-            }
-            *lo_p = lo;
-            *hi_p = hi;
-        }
+        rope_split_staged<T, D, NT>(Qs, p, q0, tid, last_row, q_scale, 0, ROWS);
     }
 }
 

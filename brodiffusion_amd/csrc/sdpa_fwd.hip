@@ -597,14 +597,19 @@ template <int D> struct DmaGeo {
     static constexpr int VOFF = RING;
     static constexpr int MAXI = (2 * NDMA + 7) / 8;          // most DMA instructions of one wavefront per step
     static constexpr bool SWZ = D == 128;
+    // The Q tile is staged behind the rings, so that the first key tiles can be in flight while it is loaded, rotated and
+    // picked apart; where rings + a whole staged tile exceed the LDS of a compute unit it goes through in two halves
+    // (rows 0..127 for wavefronts 0..3, then rows 128..255 for wavefronts 4..7). The output is staged over the rings,
+    // which are dead by then.
+    static constexpr int QOFF = 2 * RING;
+    static constexpr bool Q_HALVES = QOFF + 256 * G::O_STRIDE > 160 * 1024;
+    static constexpr int Q_BYTES = (Q_HALVES ? 128 : 256) * G::O_STRIDE;
     static constexpr int lds_bytes() {
-        const int kv = 2 * RING;
+        const int kvq = QOFF + Q_BYTES;
         const int o = 256 * G::O_STRIDE;
-        return kv > o ? kv : o;
+        return kvq > o ? kvq : o;
     }
-    // the staged Q tile (finite values) covers the whole K ring before the first key tile arrives, so the pad reads
-    // described above never meet uninitialised LDS
-    static_assert(256 * G::O_STRIDE >= RING, "Q staging must cover the K ring");
+    static_assert(QOFF + Q_BYTES <= 160 * 1024, "rings and Q staging exceed the LDS of a compute unit");
 };
 // (head_dim 40 works the same way but measured no faster than the register-staged kernel: not instantiated)
 template <int D> constexpr bool dma_kernel_available() { return D == 72 || D == 128; }
@@ -712,10 +717,12 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         if (lane == 0) { red[wave] = we.lo_min; red[8 + wave] = we.hi_max; }
     }
     V8 qf[G::KC];
-    stage_q_tile<T, D, kThreads8, BM>(smem, p, q_base, q0, tid);
-    __syncthreads();
-    read_q_frags<T, D>(qf, smem, wave * 32 + lq, lh);
-    __syncthreads();
+    // the Q rows (and their RoPE tables) are requested first; they are rotated and staged further down, behind the issue of
+    // the first key tiles' DMA, so that both latencies run together
+    using QL = QTileLoad<T, D, kThreads8, BM>;
+    static_assert(!DG::Q_HALVES || (QL::NI % 2 == 0 && kThreads8 * (QL::NI / 2) == 128 * QL::CPRK), "half of the load rounds must be half of the rows");
+    QL ql;
+    ql.issue(p, q_base, q0, tid, p.Lq - 1);
     // the first pass through the MFMA stream multiplies a zero P with the last V buffer; the slack behind both rings is zero
     for (int i = tid; i < (DG::TILE + DG::SLACK) / 16; i += kThreads8)
         *reinterpret_cast<u32x4*>(smem + DG::VOFF + (kDmaStages - 1) * DG::TILE + i * 16) = u32x4{0, 0, 0, 0};
@@ -985,6 +992,39 @@ __global__ void __launch_bounds__(kThreads8, 2) sdpa_fwd_pp_dma_kernel(const Sdp
         if (n_tiles > 2) kc.next();
         dma_tiles(false, 0, true, DG::VOFF);
         if (n_tiles > 1) vc.next();
+    }
+    {
+        // the Q tile, rotated on its way into the staging buffer behind the rings; every lane then picks the fragments of
+        // its own row
+        unsigned char* const Qs = smem + DG::QOFF;
+        const bool split_pairs = p.cos_q != nullptr && p.rope_split;
+        if constexpr (!DG::Q_HALVES) {
+            ql.store(Qs, p, q0, tid, p.Lq - 1);
+            if (split_pairs) {
+                __syncthreads();
+                rope_split_staged<T, D, kThreads8>(Qs, p, q0, tid, p.Lq - 1, 1.f, 0, BM);
+            }
+            __syncthreads();
+            read_q_frags<T, D>(qf, Qs, wave * 32 + lq, lh);
+        } else {
+            ql.template store<0, QL::NI / 2>(Qs, p, q0, tid, p.Lq - 1, 1.f, 0);
+            if (split_pairs) {
+                __syncthreads();
+                rope_split_staged<T, D, kThreads8>(Qs, p, q0, tid, p.Lq - 1, 1.f, 0, BM / 2);
+            }
+            __syncthreads();
+            if (grp == 0) read_q_frags<T, D>(qf, Qs, wave * 32 + lq, lh);
+            __syncthreads();
+            ql.template store<QL::NI / 2, QL::NI>(Qs, p, q0, tid, p.Lq - 1, 1.f, BM / 2);
+            if (split_pairs) {
+                __syncthreads();
+                rope_split_staged<T, D, kThreads8>(Qs, p, q0, tid, p.Lq - 1, 1.f, BM / 2, BM / 2);
+            }
+            __syncthreads();
+            if (grp == 1) read_q_frags<T, D>(qf, Qs, (wave - 4) * 32 + lq, lh);
+        }
+    }
+    if (n_tiles > 0) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         for (int t = -1; t < n_tiles; t += 3) {
@@ -1166,7 +1206,7 @@ int launch_d(SdpaDev p, int n_cu, hipStream_t stream) {
     // prefix-KV dial is on as well, or the key sequence is too long for the words to fit: then the 128-row kernel
     const bool xtra = p.key_mask != nullptr || p.bias != nullptr || p.lse != nullptr;
     const long kbits_bytes = p.key_mask ? 8L * ((p.Lk + kBN - 1) / kBN + 2) : 0;
-    const bool xtra_ok = !xtra || (!rope_k && !p.prefix_scaled && kbits_bytes <= 32 * 1024);
+    const bool xtra_ok = !xtra || (!rope_k && !p.prefix_scaled && kbits_bytes <= 24 * 1024);   // (the words share the LDS with rings and Q staging)
     // calls with the prefix-KV dial stay on the 128-row kernel unless the DMA kernel (which has an instance for it) takes them
     const bool dial_ok = !p.prefix_scaled || (dma_kernel_available<D>() && !rope_k && choice != 3);
     const bool pingpong = D <= 128 && xtra_ok && dial_ok && (choice >= 2 || (choice == 0 && tiles256 >= n_cu));
