@@ -39,6 +39,43 @@ __global__ void __launch_bounds__(256) rope_adjacent_kernel(const T* __restrict_
     }
 }
 
+// Adjacent pairs with one table for all heads: a thread rotates the same 16-byte chunk position of 4 heads of a row, so the
+// chunk's table entries are fetched once for the four and 4 data loads are in flight per thread. The heads of a thread
+// are n_hg apart (h = j * n_hg + hg), so that for each j the lanes of a wavefront touch consecutive heads, i.e. one
+// contiguous piece of the row. Same arithmetic per element as the kernel above.
+template <typename T>
+__global__ void __launch_bounds__(256) rope_adjacent_heads_kernel(const T* __restrict__ x, T* __restrict__ out,
+                                                                  const float* __restrict__ cs, const float* __restrict__ sn,
+                                                                  int rows, int H, int d, long x_rs, long o_rs) {
+    typedef T t8 __attribute__((ext_vector_type(8)));
+    constexpr int HB = 4;
+    const int cpd = d / 8, n_hg = H / HB;
+    const long total = static_cast<long>(rows) * n_hg * cpd;
+    for (long idx = blockIdx.x * 256L + threadIdx.x; idx < total; idx += gridDim.x * 256L) {
+        const long t = idx / cpd;
+        const int dcq = static_cast<int>(idx - t * cpd);
+        const long r = t / n_hg;
+        const int hg = static_cast<int>(t - r * n_hg);
+        const f32x4 cv = *reinterpret_cast<const f32x4*>(cs + r * (d / 2) + dcq * 4);
+        const f32x4 sv = *reinterpret_cast<const f32x4*>(sn + r * (d / 2) + dcq * 4);
+        u32x4 raw[HB];
+#pragma unroll
+        for (int j = 0; j < HB; ++j) raw[j] = *reinterpret_cast<const u32x4*>(x + r * x_rs + (j * n_hg + hg) * d + dcq * 8);
+#pragma unroll
+        for (int j = 0; j < HB; ++j) {
+            t8 v = __builtin_bit_cast(t8, raw[j]);
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const float a = static_cast<float>(v[2 * p]);
+                const float b = static_cast<float>(v[2 * p + 1]);
+                v[2 * p] = static_cast<T>(rope_re(a, b, cv[p], sv[p]));
+                v[2 * p + 1] = static_cast<T>(rope_im(a, b, cv[p], sv[p]));
+            }
+            *reinterpret_cast<u32x4*>(out + r * o_rs + (j * n_hg + hg) * d + dcq * 8) = __builtin_bit_cast(u32x4, v);
+        }
+    }
+}
+
 // Split-half pairs (x[p], x[p + d/2]): one thread per pair (d/2 need not be a multiple of 8).
 template <typename T>
 __global__ void __launch_bounds__(256) rope_split_kernel(const T* __restrict__ x, T* __restrict__ out,
@@ -221,6 +258,11 @@ int launch(const mi_rope_args* a, long x_rs, long o_rs, hipStream_t st) {
     } else if (a->split_half) {
         hipLaunchKernelGGL(rope_split_kernel<T>, dim3(blocks), dim3(256), 0, st, x, o, a->cos, a->sin, a->rows,
                            a->num_heads, a->head_dim, x_rs, o_rs, a->per_head);
+    } else if (!a->per_head && a->num_heads % 4 == 0) {
+        long hb = (work / 4 + 255) / 256;
+        if (hb > 256 * 32) hb = 256 * 32;
+        hipLaunchKernelGGL(rope_adjacent_heads_kernel<T>, dim3(hb), dim3(256), 0, st, x, o, a->cos, a->sin, a->rows,
+                           a->num_heads, a->head_dim, x_rs, o_rs);
     } else {
         hipLaunchKernelGGL(rope_adjacent_kernel<T>, dim3(blocks), dim3(256), 0, st, x, o, a->cos, a->sin, a->rows,
                            a->num_heads, a->head_dim, x_rs, o_rs, a->per_head);

@@ -101,3 +101,25 @@ def test_split_half_vector_and_scalar_kernels_agree(oracle, dtype, H, d, L):
     ref = oracle.rope_apply(x, cos, sin, H, d, split_half=True)
     ulp = 2.0 ** -8 if dtype == "bf16" else 2.0 ** -11      # one rounding to the storage dtype
     assert np.max(np.abs(to_np(a) - ref) / np.maximum(np.abs(ref), 1.0)) <= ulp
+
+
+@pytest.mark.parametrize("dtype,H,d,L", [("bf16", 24, 128, 517), ("fp16", 8, 40, 1000), ("bf16", 16, 72, 77), ("bf16", 4, 32, 3), ("fp16", 12, 64, 130)])
+def test_adjacent_pairs_with_head_count_a_multiple_of_four(oracle, dtype, H, d, L):
+    """Head counts that are multiples of 4 take the stand-alone pass in which a thread rotates one chunk position of 4 heads
+    with one fetch of the table entries. Same arithmetic as the general pass: bit-equal to the per-head-table entry point
+    fed the same table once per head (which runs the general pass), on contiguous rows and on column slices of wider
+    buffers; and within the usual bound of the checker."""
+    x = randn(7300 + H + d, (L, H * d), dtype)
+    cos, sin, dcos, dsin = _tables(L, d, 31 + d)
+    dx = to_dev(x, dtype)
+    got = bd.rope_apply(dx, dcos, dsin, d, H)
+    per_head = bd.rope_apply_perhead(dx, dcos.repeat_interleave(H, dim=0).contiguous(), dsin.repeat_interleave(H, dim=0).contiguous(), d, H)
+    assert torch.equal(got, per_head)
+    ref = oracle.rope_apply(x, cos, sin, H, d, round_to_dtype=dtype)
+    assert_close(ref, to_np(got), dtype, f"rope H={H} d={d}")
+    wide_in = torch.zeros((L, 2 * H * d + 8), dtype=dx.dtype, device="cuda")
+    wide_in[:, 8:8 + H * d] = dx
+    wide_out = torch.full((L, 3 * H * d), 7.0, dtype=dx.dtype, device="cuda")
+    bd.rope_apply(wide_in[:, 8:8 + H * d], dcos, dsin, d, H, out=wide_out[:, H * d:2 * H * d])
+    assert torch.equal(wide_out[:, H * d:2 * H * d], got)
+    assert (wide_out[:, :H * d] == 7).all() and (wide_out[:, 2 * H * d:] == 7).all()
