@@ -23,7 +23,7 @@ template <typename T, int D>
 __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
-    __shared__ __attribute__((aligned(16))) unsigned char Ks[G::K_BYTES];
+    __shared__ __attribute__((aligned(16))) unsigned char Ks2[2][G::K_BYTES];   // K tiles of two consecutive heads
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, lq = lane & 31, lh = lane >> 5;
@@ -37,8 +37,7 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
     constexpr float kLog2e = 1.4426950408889634f;
 
     // the zero pad of the head dimension (columns D .. DK-1) is written once; data chunks are rewritten per head
-    for (int i = tid; i < G::K_BYTES / 16; i += kMapThreads) reinterpret_cast<u32x4*>(Ks)[i] = u32x4{0u, 0u, 0u, 0u};
-    __syncthreads();
+    for (int i = tid; i < 2 * G::K_BYTES / 16; i += kMapThreads) reinterpret_cast<u32x4*>(&Ks2[0][0])[i] = u32x4{0u, 0u, 0u, 0u};
 
     f32x16 avg[2];
 #pragma unroll
@@ -60,27 +59,49 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
             pre[kb][e] = v;
         }
 
+    // One head's operands, requested one head ahead so that their latency passes under the previous head's products:
+    // the K tile (64 x d, a few 16-byte chunks per thread, to LDS when their turn comes; rows past the last key repeat
+    // it and are stored as zeros) and this lane's query row as B operands (8 contraction elements at 16 c + 8 lh).
     const T* const qg = static_cast<const T*>(p.q);
     const T* const kg = static_cast<const T*>(p.k);
-    for (int h = 0; h < p.H; ++h) {
-        // K tile of head h: rows past the last key stay zero (their probabilities are discarded below)
-        for (int idx = tid; idx < kBN * G::CPR; idx += kMapThreads) {
+    constexpr int NKC = (kBN * G::CPR + kMapThreads - 1) / kMapThreads;
+    u32x4 kreg[NKC];
+    V8 qn[G::KC];
+    float lse_n = 0.f;
+    auto request = [&](int h) {
+#pragma unroll
+        for (int i = 0; i < NKC; ++i) {
+            const int idx = min(tid + kMapThreads * i, kBN * G::CPR - 1);
             const int row = idx / G::CPR, cc = idx - row * G::CPR;
-            u32x4 v = u32x4{0u, 0u, 0u, 0u};
-            if (j0 + row < p.Lk) v = *reinterpret_cast<const u32x4*>(kg + static_cast<long>(j0 + row) * p.k_rs + h * D + cc * 8);
-            *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = v;
+            kreg[i] = *reinterpret_cast<const u32x4*>(kg + static_cast<long>(min(j0 + row, p.Lk - 1)) * p.k_rs + h * D + cc * 8);
         }
-        // this lane's query row as B operands: 8 contraction elements at 16 c + 8 lh
-        V8 qf[G::KC];
 #pragma unroll
         for (int c = 0; c < G::KC; ++c) {
-            const int col = 16 * c + 8 * lh;
-            u32x4 v = u32x4{0u, 0u, 0u, 0u};
-            if (col < D) v = *reinterpret_cast<const u32x4*>(qg + static_cast<long>(qr) * p.q_rs + h * D + col);
-            qf[c] = __builtin_bit_cast(V8, v);
+            const int col = min(16 * c + 8 * lh, D - 8);
+            const u32x4 v = *reinterpret_cast<const u32x4*>(qg + static_cast<long>(qr) * p.q_rs + h * D + col);
+            qn[c] = __builtin_bit_cast(V8, 16 * c + 8 * lh < D ? v : u32x4{0u, 0u, 0u, 0u});
         }
-        const float lse = p.lse[static_cast<long>(h) * p.Lq + qr];
+        lse_n = p.lse[static_cast<long>(h) * p.Lq + qr];
+    };
+    request(0);
+    __syncthreads();   // the zeroed pads are in place before the first tile's chunks land next to them
+    for (int h = 0; h < p.H; ++h) {
+        unsigned char* const Ks = Ks2[h & 1];
+#pragma unroll
+        for (int i = 0; i < NKC; ++i) {
+            const int idx = tid + kMapThreads * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < kBN * G::CPR)
+                *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = j0 + row < p.Lk ? kreg[i] : u32x4{0u, 0u, 0u, 0u};
+        }
+        V8 qf[G::KC];
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) qf[c] = qn[c];
+        const float lse = lse_n;
+        // one barrier per head: this head's tile is complete, and every wavefront has finished the head before last,
+        // whose buffer the next head's chunks will overwrite
         __syncthreads();
+        if (h + 1 < p.H) request(h + 1);
         f32x16 sacc[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -98,7 +119,6 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
             for (int e = 0; e < 16; ++e) {
                 avg[kb][e] += __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][e], p.scale_log2, pre[kb][e]) - lse);
             }
-        __syncthreads();   // all reads of this head's K tile are done before the next head overwrites it
     }
 
     if (!qvalid) return;
