@@ -8,7 +8,7 @@
 // no atomics, deterministic. Scores are computed transposed (S^T = K Q^T, as in the attention kernels): a lane owns
 // one query row, so lse and the bias row are per-lane scalars, and holds 4 consecutive keys per accumulator group,
 // which leave as 16-byte stores.
-// Per head a work group reads its K tile (64 x d, through LDS) and its Q rows (128 x d, straight into the B operands).
+// Per head a work group reads its K tile (64 x d) and its Q rows (128 x d), both through LDS, one head ahead of the products.
 #include "sdpa_common.h"
 
 namespace mi {
@@ -20,10 +20,11 @@ constexpr int kMapThreads = 256;
 constexpr int kMapRows = 128;
 
 template <typename T, int D>
-__global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
+__global__ void __launch_bounds__(kMapThreads, 2) attn_map_kernel(const MapDev p) {
     using G = HeadGeo<D>;
     using V8 = typename Mma<T>::v8;
     __shared__ __attribute__((aligned(16))) unsigned char Ks2[2][G::K_BYTES];   // K tiles of two consecutive heads
+    __shared__ __attribute__((aligned(16))) unsigned char Qs4[kMapThreads / 64][32 * G::K_STRIDE];   // per wavefront: its 32 query rows
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, lq = lane & 31, lh = lane >> 5;
@@ -61,13 +62,20 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
 
     // One head's operands, requested one head ahead so that their latency passes under the previous head's products:
     // the K tile (64 x d, a few 16-byte chunks per thread, to LDS when their turn comes; rows past the last key repeat
-    // it and are stored as zeros) and this lane's query row as B operands (8 contraction elements at 16 c + 8 lh).
+    // it and are stored as zeros) and the wavefront's 32 query rows, fetched with full-row coalescing (a lane-per-row
+    // fetch of the B operands touches 32 cache lines per instruction and made the address path the busiest unit) and
+    // passed through a slice of LDS that only this wavefront uses, from which every lane picks its row's fragments
+    // (8 contraction elements at 16 c + 8 lh).
     const T* const qg = static_cast<const T*>(p.q);
     const T* const kg = static_cast<const T*>(p.k);
     constexpr int NKC = (kBN * G::CPR + kMapThreads - 1) / kMapThreads;
     u32x4 kreg[NKC];
-    V8 qn[G::KC];
+    constexpr int NQC = (32 * G::CPR + 63) / 64;
+    u32x4 qn[NQC];
     float lse_n = 0.f;
+    unsigned char* const Qs = Qs4[wave];
+    const int wq0 = q0 + wave * 32;
+    for (int i = lane; i < 32 * G::K_STRIDE / 16; i += 64) reinterpret_cast<u32x4*>(Qs)[i] = u32x4{0u, 0u, 0u, 0u};   // (the pad columns stay zero)
     auto request = [&](int h) {
 #pragma unroll
         for (int i = 0; i < NKC; ++i) {
@@ -76,10 +84,10 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
             kreg[i] = *reinterpret_cast<const u32x4*>(kg + static_cast<long>(min(j0 + row, p.Lk - 1)) * p.k_rs + h * D + cc * 8);
         }
 #pragma unroll
-        for (int c = 0; c < G::KC; ++c) {
-            const int col = min(16 * c + 8 * lh, D - 8);
-            const u32x4 v = *reinterpret_cast<const u32x4*>(qg + static_cast<long>(qr) * p.q_rs + h * D + col);
-            qn[c] = __builtin_bit_cast(V8, 16 * c + 8 * lh < D ? v : u32x4{0u, 0u, 0u, 0u});
+        for (int i = 0; i < NQC; ++i) {
+            const int idx = min(lane + 64 * i, 32 * G::CPR - 1);
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            qn[i] = *reinterpret_cast<const u32x4*>(qg + static_cast<long>(min(wq0 + row, p.Lq - 1)) * p.q_rs + h * D + cc * 8);
         }
         lse_n = p.lse[static_cast<long>(h) * p.Lq + qr];
     };
@@ -94,13 +102,19 @@ __global__ void __launch_bounds__(kMapThreads) attn_map_kernel(const MapDev p) {
             if (idx < kBN * G::CPR)
                 *reinterpret_cast<u32x4*>(Ks + row * G::K_STRIDE + cc * 16) = j0 + row < p.Lk ? kreg[i] : u32x4{0u, 0u, 0u, 0u};
         }
-        V8 qf[G::KC];
 #pragma unroll
-        for (int c = 0; c < G::KC; ++c) qf[c] = qn[c];
+        for (int i = 0; i < NQC; ++i) {
+            const int idx = lane + 64 * i;
+            const int row = idx / G::CPR, cc = idx - row * G::CPR;
+            if (idx < 32 * G::CPR) *reinterpret_cast<u32x4*>(Qs + row * G::K_STRIDE + cc * 16) = qn[i];
+        }
         const float lse = lse_n;
         // one barrier per head: this head's tile is complete, and every wavefront has finished the head before last,
         // whose buffer the next head's chunks will overwrite
         __syncthreads();
+        V8 qf[G::KC];
+#pragma unroll
+        for (int c = 0; c < G::KC; ++c) qf[c] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4*>(Qs + lq * G::K_STRIDE + (2 * c + lh) * 16));
         if (h + 1 < p.H) request(h + 1);
         f32x16 sacc[2];
 #pragma unroll
