@@ -13,7 +13,8 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
-@pytest.mark.parametrize("L,H,d,axes", [(577, 24, 128, (16, 56, 56)), (64, 5, 64, (16, 24, 24)), (33, 70, 32, (8, 12, 12)), (1, 1, 128, (16, 56, 56))])
+@pytest.mark.parametrize("L,H,d,axes", [(577, 24, 128, (16, 56, 56)), (64, 5, 64, (16, 24, 24)), (33, 70, 32, (8, 12, 12)), (1, 1, 128, (16, 56, 56)),
+                                      (100, 8, 64, (16, 24, 24)), (50, 12, 32, (8, 12, 12))])   # head counts that are multiples of 4: one thread per 4 heads
 def test_headnorm_rope_matches_checker(oracle, dtype, L, H, d, axes):
     x = randn(9000 + L, (L, H * d), dtype) * 2.5
     x = oracle.round_to(x, dtype)
